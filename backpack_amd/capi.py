@@ -1,0 +1,102 @@
+"""ctypes binding of libbpk_kquant.so (include/bpk_kquant.h).
+
+Device pointers are passed as integers (e.g. torch.Tensor.data_ptr()).  The
+library is loaded from the package directory; it is never built implicitly and
+loading fails loudly when it is missing."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libbpk_kquant.so")
+
+Q4_K = 12
+Q6_K = 14
+
+FAMILY_AUTO, FAMILY_GENERIC, FAMILY_GEMV_ROWS, FAMILY_MFMA_SMALL, FAMILY_MFMA_GEMM = range(5)
+
+
+class BpkError(RuntimeError):
+    def __init__(self, code: int, msg: str):
+        super().__init__(f"bpk error {code}: {msg}")
+        self.code = code
+
+
+class WeightDesc(C.Structure):
+    _fields_ = [("type", C.c_int), ("N", C.c_uint32), ("K", C.c_uint32),
+                ("n_blocks", C.c_uint32), ("row_stride_words", C.c_uint32),
+                ("data", C.c_void_p), ("bytes", C.c_size_t)]
+
+
+_SIGS = {
+    "bpk_version": (C.c_int, []),
+    "bpk_last_error": (C.c_char_p, []),
+    "bpk_last_kernel": (C.c_char_p, []),
+    "bpk_force_kernel": (C.c_int, [C.c_int]),
+    "bpk_set_option": (C.c_int, [C.c_char_p, C.c_int]),
+    "bpk_init": (C.c_int, [C.c_int]),
+    "bpk_shutdown": (C.c_int, []),
+    "bpk_kq_layout": (C.c_int, [C.c_int, C.c_uint32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+    "bpk_kq_pack_host": (C.c_int, [C.c_int, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]),
+    "bpk_weight_create": (C.c_int, [C.c_int, C.c_uint32, C.c_uint32, C.POINTER(C.c_void_p),
+                                    C.POINTER(C.c_uint32), C.POINTER(C.c_void_p)]),
+    "bpk_weight_describe": (C.c_int, [C.c_void_p, C.POINTER(WeightDesc)]),
+    "bpk_weight_destroy": (C.c_int, [C.c_void_p]),
+    "bpk_kq_matmul": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
+                                C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p]),
+    "bpk_kq_matmul_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
+                                     C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p]),
+    "bpk_kq_dequant_rows": (C.c_int, [C.c_int, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_uint32,
+                                      C.c_void_p, C.c_void_p]),
+    "bpk_kq_moe_matmul": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
+                                    C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32,
+                                    C.c_int, C.c_void_p]),
+    "bpk_kq_moe_ffn_scratch_bytes": (C.c_size_t, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32]),
+    "bpk_kq_moe_ffn": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                 C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32,
+                                 C.c_uint32, C.c_uint32, C.c_void_p, C.c_size_t, C.c_void_p]),
+}
+
+_lib = None
+
+
+def exported_names():
+    return sorted(_SIGS)
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is missing: build it with `python -m backpack_amd.build`")
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGS.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise BpkError(rc, lib().bpk_last_error().decode())
+
+
+def layout(type_: int, K: int):
+    nb, rs = C.c_uint32(), C.c_uint32()
+    check(lib().bpk_kq_layout(type_, K, C.byref(nb), C.byref(rs)))
+    return nb.value, rs.value
+
+
+def last_kernel() -> str:
+    return lib().bpk_last_kernel().decode()
+
+
+def force_kernel(family: int) -> None:
+    check(lib().bpk_force_kernel(family))
+
+
+def set_option(name: str, value: int) -> None:
+    check(lib().bpk_set_option(name.encode(), value))

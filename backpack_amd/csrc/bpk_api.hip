@@ -1,0 +1,336 @@
+// bpk_api.hip — the C ABI (include/bpk_kquant.h): argument checking, per-device
+// state, kernel-family choice, launches.  No arithmetic lives here.
+#include "../../include/bpk_kquant.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <vector>
+
+#include "kq_format.h"
+#include "kq_kernels.h"
+
+namespace {
+
+constexpr int kMaxDevices = 16;
+constexpr size_t kPartialFloats = size_t(4) << 20;  // 16 MiB of split-K partial sums
+constexpr uint32_t kCounters = 1u << 16;
+
+thread_local char t_err[512] = "";
+thread_local const char* t_kernel = "";
+thread_local int t_family = 0;
+thread_local int t_splits = 0;
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_err, sizeof t_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what)
+{
+    return fail(BPK_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+struct DeviceState {
+    bool ready = false;
+    kq::SplitScratch split{};
+};
+
+std::mutex g_mu;
+DeviceState g_dev[kMaxDevices];
+
+int ensure_device(int device, DeviceState** out)
+{
+    if (device < 0 || device >= kMaxDevices) return fail(BPK_ERR_DEVICE, "device %d out of range", device);
+    std::lock_guard<std::mutex> lk(g_mu);
+    DeviceState& st = g_dev[device];
+    if (!st.ready) {
+        hipDeviceProp_t prop;
+        hipError_t e = hipGetDeviceProperties(&prop, device);
+        if (e != hipSuccess) return hip_fail(e, "hipGetDeviceProperties");
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+            return fail(BPK_ERR_DEVICE, "device %d is %s; this library is built for gfx950 only", device,
+                        prop.gcnArchName);
+        int cur = -1;
+        (void)hipGetDevice(&cur);
+        if (cur != device) (void)hipSetDevice(device);
+        e = hipMalloc((void**)&st.split.partial, kPartialFloats * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc((void**)&st.split.counters, kCounters * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipMemset(st.split.counters, 0, kCounters * sizeof(uint32_t));
+        if (cur != device && cur >= 0) (void)hipSetDevice(cur);
+        if (e != hipSuccess) return hip_fail(e, "allocating split-K scratch");
+        st.split.capacity_floats = kPartialFloats;
+        st.split.n_counters = kCounters;
+        st.ready = true;
+    }
+    if (out) *out = &st;
+    return BPK_OK;
+}
+
+int current_state(DeviceState** out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    return ensure_device(dev, out);
+}
+
+bool known_type(int type) { return type == BPK_TYPE_Q4_K || type == BPK_TYPE_Q6_K; }
+
+int check_matmul(int type, const void* X, const void* W, const void* Y, uint32_t M, uint32_t N, uint32_t K,
+                 uint32_t n_blocks, uint32_t row_stride_words)
+{
+    if (!known_type(type)) return fail(BPK_ERR_TYPE, "unsupported GGUF type %d (Q4_K=12, Q6_K=14)", type);
+    if (!X || !W || !Y) return fail(BPK_ERR_NULL, "X, W and Y must be non-null");
+    if (K == 0 || K % KQ_QK) return fail(BPK_ERR_SHAPE, "K=%u is not a positive multiple of 256", K);
+    if (N == 0) return fail(BPK_ERR_SHAPE, "N must be positive");
+    if (n_blocks != K / KQ_QK) return fail(BPK_ERR_SHAPE, "n_blocks=%u does not match K/256=%u", n_blocks, K / KQ_QK);
+    const uint64_t row_bytes = (uint64_t)n_blocks * kq::block_bytes(type);
+    if ((uint64_t)row_stride_words * 4u < row_bytes)
+        return fail(BPK_ERR_SHAPE, "row_stride_words=%u is smaller than a row (%llu bytes)", row_stride_words,
+                    (unsigned long long)row_bytes);
+    if ((uint64_t)row_stride_words * 4u > 0xFFFFFFFFull) return fail(BPK_ERR_SHAPE, "row stride too large");
+    if ((uintptr_t)W & 3u) return fail(BPK_ERR_ALIGN, "W must be 4-byte aligned");
+    if ((uintptr_t)X & 3u || (uintptr_t)Y & 3u) return fail(BPK_ERR_ALIGN, "X and Y must be 4-byte aligned");
+    (void)M;
+    return BPK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int bpk_version(void) { return 100; }
+
+const char* bpk_last_error(void) { return t_err; }
+
+const char* bpk_last_kernel(void) { return t_kernel; }
+
+int bpk_force_kernel(int family)
+{
+    if (family < 0 || family > 4) return fail(BPK_ERR_SHAPE, "kernel family %d unknown", family);
+    t_family = family;
+    return BPK_OK;
+}
+
+int bpk_set_option(const char* name, int value)
+{
+    if (!name) return fail(BPK_ERR_NULL, "option name is null");
+    if (!strcmp(name, "gemv_splits")) { t_splits = value; return BPK_OK; }
+    return fail(BPK_ERR_SHAPE, "unknown option '%s'", name);
+}
+
+int bpk_init(int device) { return ensure_device(device, nullptr); }
+
+int bpk_shutdown(void)
+{
+    std::lock_guard<std::mutex> lk(g_mu);
+    int cur = -1;
+    (void)hipGetDevice(&cur);
+    for (int d = 0; d < kMaxDevices; ++d) {
+        DeviceState& st = g_dev[d];
+        if (!st.ready) continue;
+        (void)hipSetDevice(d);
+        (void)hipFree(st.split.partial);
+        (void)hipFree(st.split.counters);
+        st = DeviceState{};
+    }
+    if (cur >= 0) (void)hipSetDevice(cur);
+    return BPK_OK;
+}
+
+int bpk_kq_layout(int type, uint32_t K, uint32_t* n_blocks, uint32_t* row_stride_words)
+{
+    if (!known_type(type)) return fail(BPK_ERR_TYPE, "unsupported GGUF type %d", type);
+    const uint32_t nb = (K + KQ_QK - 1) / KQ_QK;
+    if (n_blocks) *n_blocks = nb;
+    if (row_stride_words) *row_stride_words = (nb * kq::block_bytes(type) + 3u) / 4u;
+    return BPK_OK;
+}
+
+int bpk_kq_pack_host(int type, const void* raw, uint32_t N, uint32_t K, uint32_t* out_words)
+{
+    if (!known_type(type)) return fail(BPK_ERR_TYPE, "unsupported GGUF type %d", type);
+    if (!raw || !out_words) return fail(BPK_ERR_NULL, "raw and out_words must be non-null");
+    uint32_t nb, rs;
+    bpk_kq_layout(type, K, &nb, &rs);
+    const size_t row_bytes = (size_t)nb * kq::block_bytes(type), stride = (size_t)rs * 4u;
+    const uint8_t* src = (const uint8_t*)raw;
+    uint8_t* dst = (uint8_t*)out_words;
+    for (uint32_t n = 0; n < N; ++n) {
+        memcpy(dst + n * stride, src + n * row_bytes, row_bytes);
+        memset(dst + n * stride + row_bytes, 0, stride - row_bytes);
+    }
+    return BPK_OK;
+}
+
+struct bpk_weight {
+    bpk_weight_desc d;
+    int device;
+};
+
+int bpk_weight_create(int type, uint32_t K, uint32_t n_parts, const void* const* parts, const uint32_t* n_rows,
+                      bpk_weight** out)
+{
+    if (!known_type(type)) return fail(BPK_ERR_TYPE, "unsupported GGUF type %d", type);
+    if (!parts || !n_rows || !out) return fail(BPK_ERR_NULL, "parts, n_rows and out must be non-null");
+    if (K == 0 || K % KQ_QK) return fail(BPK_ERR_SHAPE, "K=%u is not a positive multiple of 256", K);
+    uint64_t N = 0;
+    for (uint32_t i = 0; i < n_parts; ++i) {
+        if (!parts[i]) return fail(BPK_ERR_NULL, "parts[%u] is null", i);
+        N += n_rows[i];
+    }
+    if (N == 0 || N > 0xFFFFFFFFull) return fail(BPK_ERR_SHAPE, "total rows %llu out of range", (unsigned long long)N);
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
+    uint32_t nb, rs;
+    bpk_kq_layout(type, K, &nb, &rs);
+    const size_t bytes = (size_t)N * rs * 4u;
+    std::vector<uint32_t> host;
+    try {
+        host.resize((size_t)N * rs);
+    } catch (const std::bad_alloc&) {
+        return fail(BPK_ERR_SHAPE, "host staging of %zu bytes failed", bytes);
+    }
+    size_t row = 0;
+    for (uint32_t i = 0; i < n_parts; ++i) {
+        bpk_kq_pack_host(type, parts[i], n_rows[i], K, host.data() + row * rs);
+        row += n_rows[i];
+    }
+    void* dptr = nullptr;
+    // 16 trailing bytes let 128-bit loads of the last row's tail stay in bounds
+    hipError_t e = hipMalloc(&dptr, bytes + 16);
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc(weights)");
+    e = hipMemcpy(dptr, host.data(), bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemset((uint8_t*)dptr + bytes, 0, 16);
+    if (e != hipSuccess) {
+        (void)hipFree(dptr);
+        return hip_fail(e, "hipMemcpy(weights)");
+    }
+    bpk_weight* w = new (std::nothrow) bpk_weight;
+    if (!w) {
+        (void)hipFree(dptr);
+        return fail(BPK_ERR_SHAPE, "out of host memory");
+    }
+    w->d = bpk_weight_desc{type, (uint32_t)N, K, nb, rs, dptr, bytes};
+    (void)hipGetDevice(&w->device);
+    *out = w;
+    return BPK_OK;
+}
+
+int bpk_weight_describe(const bpk_weight* w, bpk_weight_desc* out)
+{
+    if (!w || !out) return fail(BPK_ERR_NULL, "weight and out must be non-null");
+    *out = w->d;
+    return BPK_OK;
+}
+
+int bpk_weight_destroy(bpk_weight* w)
+{
+    if (!w) return BPK_OK;
+    hipError_t e = hipFree(w->d.data);
+    delete w;
+    return e == hipSuccess ? BPK_OK : hip_fail(e, "hipFree(weights)");
+}
+
+int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, float* Y, uint32_t M, uint32_t N,
+                  uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, uint32_t y_offset, void* stream)
+{
+    if (int rc = check_matmul(type, X, W, Y, M, N, K, n_blocks, row_stride_words)) return rc;
+    if (M == 0) return BPK_OK;
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
+    kq::MatmulArgs a{};
+    a.type = type; a.X = X; a.W = (const uint8_t*)W; a.bias = bias; a.Y = Y;
+    a.M = M; a.N = N; a.K = K; a.n_blocks = n_blocks;
+    a.row_stride_bytes = row_stride_words * 4u;
+    a.y_offset = y_offset;
+    a.ldy = N;
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t e;
+    const bool rows_ok = kq::gemv_rows_supported(a);
+    if (t_family == 2 && !rows_ok) return fail(BPK_ERR_SHAPE, "row-per-lane GEMV cannot serve this call");
+    if (t_family > 2) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
+    if ((t_family == 0 || t_family == 2) && rows_ok) {
+        t_kernel = "gemv_rows";
+        e = kq::launch_gemv_rows(a, st->split, t_splits, s);
+    } else {
+        t_kernel = "generic";
+        e = kq::launch_matmul_generic(a, s);
+    }
+    return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+int bpk_kq_matmul_bf16(int type, const uint16_t* X, const void* W, const float* bias, float* Y, uint32_t M,
+                       uint32_t N, uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, void* stream)
+{
+    if (int rc = check_matmul(type, X, W, Y, M, N, K, n_blocks, row_stride_words)) return rc;
+    (void)bias; (void)stream;
+    return fail(BPK_ERR_SHAPE, "bf16 prefill GEMM is not built yet");
+}
+
+int bpk_kq_dequant_rows(int type, const void* W, uint32_t row_stride_words, const int32_t* rows, uint32_t M,
+                        uint32_t K, float* out, void* stream)
+{
+    if (!known_type(type)) return fail(BPK_ERR_TYPE, "unsupported GGUF type %d", type);
+    if (!W || !out) return fail(BPK_ERR_NULL, "W and out must be non-null");
+    if (K == 0 || K % KQ_QK) return fail(BPK_ERR_SHAPE, "K=%u is not a positive multiple of 256", K);
+    if ((uint64_t)row_stride_words * 4u < (uint64_t)(K / KQ_QK) * kq::block_bytes(type))
+        return fail(BPK_ERR_SHAPE, "row_stride_words=%u is smaller than a row", row_stride_words);
+    if (M == 0) return BPK_OK;
+    if (int rc = current_state(nullptr)) return rc;
+    hipError_t e = kq::launch_dequant_rows(type, (const uint8_t*)W, row_stride_words * 4u, rows, M, K, out,
+                                           (hipStream_t)stream);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, "dequant_rows");
+}
+
+int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* expert_idx, float* Y, uint32_t T,
+                      uint32_t k, uint32_t n_experts, uint32_t N, uint32_t K, uint32_t n_blocks,
+                      uint32_t row_stride_words, int x_per_slot, void* stream)
+{
+    if (int rc = check_matmul(type, X, W, Y, T, N, K, n_blocks, row_stride_words)) return rc;
+    if (!expert_idx) return fail(BPK_ERR_NULL, "expert_idx must be non-null");
+    if (k == 0 || n_experts == 0) return fail(BPK_ERR_SHAPE, "k and n_experts must be positive");
+    if ((uint64_t)T * k > 0xFFFFFFFFull) return fail(BPK_ERR_SHAPE, "T*k overflows");
+    if (T == 0) return BPK_OK;
+    if (int rc = current_state(nullptr)) return rc;
+    kq::MatmulArgs a{};
+    a.type = type; a.X = X; a.W = (const uint8_t*)W; a.bias = nullptr; a.Y = Y;
+    a.M = T * k; a.N = N; a.K = K; a.n_blocks = n_blocks;
+    a.row_stride_bytes = row_stride_words * 4u;
+    a.y_offset = 0;
+    a.ldy = N;
+    a.expert_idx = expert_idx;
+    a.k_slots = k;
+    a.x_per_slot = x_per_slot;
+    t_kernel = "generic_indirect";
+    hipError_t e = kq::launch_matmul_generic(a, (hipStream_t)stream);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+size_t bpk_kq_moe_ffn_scratch_bytes(uint32_t T, uint32_t k, uint32_t hidden, uint32_t inter)
+{
+    // gate, up (act written over gate) and the per-pair down outputs
+    return ((size_t)T * k * inter * 2 + (size_t)T * k * hidden) * sizeof(float);
+}
+
+int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, const void* up, const void* down,
+                   const uint32_t* expert_idx, const float* expert_wt, float* out, uint32_t T, uint32_t k,
+                   uint32_t n_experts, uint32_t hidden, uint32_t inter, void* scratch, size_t scratch_bytes,
+                   void* stream)
+{
+    (void)type_gu; (void)type_dn; (void)X; (void)gate; (void)up; (void)down; (void)expert_idx; (void)expert_wt;
+    (void)out; (void)T; (void)k; (void)n_experts; (void)hidden; (void)inter; (void)scratch; (void)scratch_bytes;
+    (void)stream;
+    return fail(BPK_ERR_SHAPE, "MoE FFN is not built yet");
+}
+
+}  // extern "C"

@@ -1,0 +1,47 @@
+// kq_kernels.h — launch entry points of the HIP kernels (internal to the library).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace kq {
+
+struct MatmulArgs {
+    int type;               // KQ_TYPE_*
+    const void* X;          // f32 [M,K] or bf16 [M,K]
+    const uint8_t* W;       // packed rows
+    const float* bias;      // [N] or nullptr
+    float* Y;               // f32
+    uint32_t M, N, K;
+    uint32_t n_blocks;
+    uint32_t row_stride_bytes;
+    uint32_t y_offset;
+    uint32_t ldy;           // elements between consecutive rows of Y
+    // expert indirection (nullptr for the dense case): pair p uses weight rows
+    // expert_idx[p]*N .. +N-1 and X row p / k_slots (x_per_slot == 0) or p.
+    const uint32_t* expert_idx;
+    uint32_t k_slots;
+    int x_per_slot;
+};
+
+// Per-device scratch for split-K partial sums and arrival counters.
+struct SplitScratch {
+    float* partial;        // capacity_floats floats
+    uint32_t* counters;    // n_counters words, zero between launches
+    size_t capacity_floats;
+    uint32_t n_counters;
+};
+
+hipError_t launch_dequant_rows(int type, const uint8_t* W, uint32_t row_stride_bytes,
+                               const int32_t* rows, uint32_t M, uint32_t K, float* out,
+                               hipStream_t s);
+
+// Any shape with K % 256 == 0, any 4-byte aligned W.  M tiled by 4 inside.
+hipError_t launch_matmul_generic(const MatmulArgs& a, hipStream_t s);
+
+// Row-per-lane decode GEMV (M <= 4): Q4_K and Q6_K with 16-byte aligned rows.
+bool gemv_rows_supported(const MatmulArgs& a);
+size_t gemv_rows_scratch_floats(const MatmulArgs& a, int forced_splits);
+hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, int forced_splits,
+                            hipStream_t s);
+
+}  // namespace kq

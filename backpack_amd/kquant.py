@@ -1,0 +1,138 @@
+"""Host-side op layer over the C ABI, with torch tensors as device memory.
+
+Mirrors the reference's k-quant operator shape: a packed weight descriptor
+(KQuantPacked: data, N, K, rowStrideWords, nBlocks — runtime/gguf_loader.h:108-113)
+and a matmul taking the {X, W, Bias, Y, P} binding set
+(runtime/model_runner.cpp:2404-2413).  torch only owns the buffers and the
+stream; every computation goes through libbpk_kquant.so.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import capi
+from .capi import Q4_K, Q6_K  # noqa: F401
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+@dataclass
+class KQuantPacked:
+    """Packed k-quant matrix resident on the GPU (same fields as the reference's)."""
+    data: torch.Tensor        # uint8, N * row_stride_words * 4 bytes (+16 slack)
+    type: int
+    N: int
+    K: int
+    row_stride_words: int
+    n_blocks: int
+
+    @property
+    def row_stride_bytes(self) -> int:
+        return self.row_stride_words * 4
+
+
+def pack_host(type_: int, raw: np.ndarray, N: int, K: int) -> np.ndarray:
+    """pack_q4k / pack_q6k on the host through the library's packer."""
+    raw = np.ascontiguousarray(raw, dtype=np.uint8)
+    nb, rs = capi.layout(type_, K)
+    assert raw.size == N * nb * (144 if type_ == Q4_K else 210), "raw size does not match N x K"
+    out = np.empty(N * rs, dtype=np.uint32)
+    capi.check(capi.lib().bpk_kq_pack_host(type_, raw.ctypes.data, N, K, out.ctypes.data))
+    return out
+
+
+def upload(type_: int, packed_words: np.ndarray, N: int, K: int, device="cuda") -> KQuantPacked:
+    """Packed host words -> device (the reference's uploadKQWeight)."""
+    nb, rs = capi.layout(type_, K)
+    assert packed_words.size == N * rs
+    host = torch.from_numpy(np.ascontiguousarray(packed_words).view(np.uint8))
+    data = torch.zeros(host.numel() + 16, dtype=torch.uint8, device=device)
+    data[: host.numel()].copy_(host)
+    return KQuantPacked(data, type_, N, K, rs, nb)
+
+
+def from_raw(type_: int, raw: np.ndarray, N: int, K: int, device="cuda") -> KQuantPacked:
+    return upload(type_, pack_host(type_, raw, N, K), N, K, device)
+
+
+def fuse(parts: list[KQuantPacked]) -> KQuantPacked:
+    """Row-wise concatenation of matrices with equal K and type (fuseKQ)."""
+    a = parts[0]
+    assert all(p.K == a.K and p.type == a.type for p in parts)
+    body = [p.data[: p.N * p.row_stride_bytes] for p in parts]
+    data = torch.cat(body + [torch.zeros(16, dtype=torch.uint8, device=a.data.device)])
+    return KQuantPacked(data, a.type, sum(p.N for p in parts), a.K, a.row_stride_words, a.n_blocks)
+
+
+def matmul(x: torch.Tensor, w: KQuantPacked, bias: torch.Tensor | None = None,
+           out: torch.Tensor | None = None, y_offset: int = 0) -> torch.Tensor:
+    """Y[m, y_offset+n] = bias[n] + sum_k X[m,k] * dequant(W)[n,k]; fp32 or bf16 X."""
+    assert x.is_cuda and x.is_contiguous() and x.shape[-1] == w.K
+    M = x.numel() // w.K
+    if out is None:
+        assert y_offset == 0
+        out = torch.empty((M, w.N), dtype=torch.float32, device=x.device)
+    assert out.is_contiguous() and out.dtype == torch.float32
+    L = capi.lib()
+    if x.dtype == torch.float32:
+        rc = L.bpk_kq_matmul(w.type, _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out), M, w.N, w.K,
+                             w.n_blocks, w.row_stride_words, y_offset, _stream())
+    elif x.dtype == torch.bfloat16:
+        assert y_offset == 0
+        rc = L.bpk_kq_matmul_bf16(w.type, _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out), M, w.N, w.K,
+                                  w.n_blocks, w.row_stride_words, _stream())
+    else:
+        raise TypeError(f"X must be float32 or bfloat16, got {x.dtype}")
+    capi.check(rc)
+    return out
+
+
+def dequant_rows(w: KQuantPacked, rows: torch.Tensor | None = None, M: int | None = None) -> torch.Tensor:
+    """fp32 rows of the matrix (the q6k_gather contract); rows: int32 device tensor."""
+    if rows is not None:
+        assert rows.dtype == torch.int32 and rows.is_cuda
+        M = rows.numel()
+    elif M is None:
+        M = w.N
+    out = torch.empty((M, w.K), dtype=torch.float32, device=w.data.device)
+    capi.check(capi.lib().bpk_kq_dequant_rows(w.type, _ptr(w.data), w.row_stride_words, _ptr(rows), M, w.K,
+                                              _ptr(out), _stream()))
+    return out
+
+
+def moe_matmul(x: torch.Tensor, w: KQuantPacked, expert_idx: torch.Tensor, n_experts: int,
+               x_per_slot: bool = False) -> torch.Tensor:
+    """Per (token, slot) matvec against the expert's row slice of a stacked matrix."""
+    assert expert_idx.dtype in (torch.int32, torch.uint32) and expert_idx.is_cuda
+    T, k = expert_idx.shape
+    N = w.N // n_experts
+    assert N * n_experts == w.N
+    out = torch.empty((T, k, N), dtype=torch.float32, device=x.device)
+    capi.check(capi.lib().bpk_kq_moe_matmul(w.type, _ptr(x), _ptr(w.data), _ptr(expert_idx), _ptr(out), T, k,
+                                            n_experts, N, w.K, w.n_blocks, w.row_stride_words,
+                                            int(x_per_slot), _stream()))
+    return out
+
+
+def moe_ffn(x: torch.Tensor, gate: KQuantPacked, up: KQuantPacked, down: KQuantPacked,
+            expert_idx: torch.Tensor, expert_wt: torch.Tensor, n_experts: int) -> torch.Tensor:
+    """Routed-expert FFN: sum_s wt[t,s] * down_e(silu(gate_e x) * up_e x)."""
+    T, k = expert_idx.shape
+    hidden, inter = gate.K, down.K
+    L = capi.lib()
+    nbytes = L.bpk_kq_moe_ffn_scratch_bytes(T, k, hidden, inter)
+    scratch = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    out = torch.empty((T, hidden), dtype=torch.float32, device=x.device)
+    capi.check(L.bpk_kq_moe_ffn(gate.type, down.type, _ptr(x), _ptr(gate.data), _ptr(up.data), _ptr(down.data),
+                                _ptr(expert_idx), _ptr(expert_wt), _ptr(out), T, k, n_experts, hidden, inter,
+                                _ptr(scratch), nbytes, _stream()))
+    return out

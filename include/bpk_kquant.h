@@ -1,0 +1,195 @@
+/*
+ * bpk_kquant.h — C ABI of the MI355X (gfx950) k-quant dequant-matmul library.
+ *
+ * Plain pointers and sizes only.  Device pointers are ordinary HIP device
+ * addresses; a caller that holds a buffer + byte offset view (the reference's
+ * GPUBuffer{handle,size,offset}, runtime/gpu_context.h:47-51) passes
+ * base + offset.  `stream` is a hipStream_t passed as void* (NULL = the null
+ * stream).  Every launch is asynchronous on that stream and in order with the
+ * other work on it; the library never synchronises the device.
+ *
+ * Every function returns BPK_OK (0) or a negative BPK_ERR_* code, and stores a
+ * human-readable message retrievable with bpk_last_error() (thread-local).
+ * The reference's ops return void and print to stderr on failure
+ * (runtime/ops/matmul.cpp:211-212, runtime/model_runner.cpp:154-157); a host
+ * wrapper that wants that behaviour prints bpk_last_error() and returns.
+ *
+ * One host thread per stream, as in the reference (runtime/model_runner.h:27-30).
+ */
+#ifndef BPK_KQUANT_H
+#define BPK_KQUANT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define BPK_API __attribute__((visibility("default")))
+#else
+#define BPK_API
+#endif
+
+/* GGUF tensor type codes (runtime/gguf_loader.h:29-30). */
+#define BPK_TYPE_Q4_K 12
+#define BPK_TYPE_Q6_K 14
+
+enum {
+    BPK_OK = 0,
+    BPK_ERR_TYPE = -1,      /* not Q4_K / Q6_K                               */
+    BPK_ERR_SHAPE = -2,     /* K not a multiple of 256, zero sizes, overflow  */
+    BPK_ERR_NULL = -3,      /* required pointer is NULL                       */
+    BPK_ERR_ALIGN = -4,     /* pointer or stride alignment not met            */
+    BPK_ERR_HIP = -5,       /* a HIP runtime call failed                      */
+    BPK_ERR_DEVICE = -6,    /* the current device is not gfx950               */
+    BPK_ERR_WORKSPACE = -7  /* workspace missing or too small                 */
+};
+
+/* Library version, major*10000 + minor*100 + patch. */
+BPK_API int bpk_version(void);
+
+/* Message of the last failing call on this thread ("" when none). */
+BPK_API const char *bpk_last_error(void);
+
+/* Checks that `device` is a gfx950 part and creates the library's per-device
+ * state (split-K scratch, counters).  Optional: the first launch on a device
+ * does the same.  Replaces GPUContext device bring-up for this path
+ * (runtime/gpu_context.h:86-145). */
+BPK_API int bpk_init(int device);
+
+/* Frees the per-device state of every device.  Outstanding work must have
+ * completed. */
+BPK_API int bpk_shutdown(void);
+
+/* ---- layout: replaces the descriptor half of pack_q4k / pack_q6k ----------
+ * runtime/gguf_loader.cpp:359-379, :403-424; struct KQuantPacked
+ * (runtime/gguf_loader.h:108-113).  n_blocks = ceil(K/256);
+ * row_stride_words = 36*n_blocks (Q4_K) or ceil(210*n_blocks/4) (Q6_K). */
+BPK_API int bpk_kq_layout(int type, uint32_t K, uint32_t *n_blocks,
+                          uint32_t *row_stride_words);
+
+/* Host-side packer: N rows of raw GGUF blocks -> N*row_stride_words words,
+ * pad bytes zero.  Replaces the copy half of pack_q4k / pack_q6k. */
+BPK_API int bpk_kq_pack_host(int type, const void *raw, uint32_t N, uint32_t K,
+                             uint32_t *out_words);
+
+/* ---- weights: replaces uploadKQWeight / fuseKQ ------------------------------
+ * runtime/model_runner.cpp:958-963 (createBuffer + writeBuffer of the packed
+ * words) and :1002-1012 (row-wise concatenation of matrices with equal K).
+ * The handle owns one device allocation that lives until destroy. */
+typedef struct bpk_weight bpk_weight;
+
+typedef struct bpk_weight_desc {
+    int type;                  /* BPK_TYPE_*                     */
+    uint32_t N, K;             /* rows (outputs), columns        */
+    uint32_t n_blocks;         /* superblocks per row            */
+    uint32_t row_stride_words; /* words per packed row           */
+    void *data;                /* device address of row 0        */
+    size_t bytes;              /* size of the device allocation  */
+} bpk_weight_desc;
+
+/* parts[i] points at raw GGUF bytes (host) of an n_rows[i] x K matrix; the
+ * parts are stacked in order (n_parts = 1 for a plain upload).  Synchronous:
+ * the host buffers may be released on return. */
+BPK_API int bpk_weight_create(int type, uint32_t K, uint32_t n_parts,
+                              const void *const *parts, const uint32_t *n_rows,
+                              bpk_weight **out);
+BPK_API int bpk_weight_describe(const bpk_weight *w, bpk_weight_desc *out);
+BPK_API int bpk_weight_destroy(bpk_weight *w);
+
+/* ---- matmul: replaces the q4k_matmul* / q6k_matmul* dispatches -------------
+ * Bindings 0:X 1:W 2:Bias 3:Y 4:P of runtime/kernels/quant_kq/q4k_matmul.wgsl:20-95,
+ * q4k_matmul_128.wgsl:8-17, q4k_matmul_batched4/8.wgsl, q6k_matmul.wgsl:25-114,
+ * q6k_matmul_batched4.wgsl, q6k_matmul_wide.wgsl, with
+ * P = {K, N, nBlocks, rowStrideWords, yOffset} (runtime/model_runner.cpp:2404-2413)
+ * or {K, N, M, nBlocks, rowStrideWords} (:5843-5844).  One entry point serves
+ * every M; the kernel choice the reference makes in kqPipelineFor / mmk
+ * (runtime/model_runner.cpp:2043-2054, :5841-5845) happens inside.
+ *
+ *   Y[m*N + y_offset + n] = bias[n] + sum_k X[m*K + k] * dequant(W)[n, k]
+ *
+ * X: f32 [M,K] (device).  W: packed rows (device, 4-byte aligned; 16-byte
+ * aligned rows take the fast kernels).  bias: f32 [N] or NULL (= zeros).
+ * Y: f32, caller-owned, not cleared.  fp32 accumulation throughout. */
+BPK_API int bpk_kq_matmul(int type, const float *X, const void *W,
+                          const float *bias, float *Y, uint32_t M, uint32_t N,
+                          uint32_t K, uint32_t n_blocks,
+                          uint32_t row_stride_words, uint32_t y_offset,
+                          void *stream);
+
+/* Prefill form: X is bf16 [M,K] (raw 16-bit patterns), Y f32 [M,N].  Weight
+ * tiles are dequantised to bf16 in LDS and contracted on the matrix cores
+ * with fp32 accumulation.  The reference has no such kernel: its k-quant
+ * prefill loops the M=1 path (runtime/model_runner.cpp:6148-6158); the
+ * contract is the same formula as bpk_kq_matmul. */
+BPK_API int bpk_kq_matmul_bf16(int type, const uint16_t *X, const void *W,
+                               const float *bias, float *Y, uint32_t M,
+                               uint32_t N, uint32_t K, uint32_t n_blocks,
+                               uint32_t row_stride_words, void *stream);
+
+/* ---- dequantised rows: replaces q6k_gather / q6k_gather_batched -------------
+ * runtime/kernels/quant_kq/q6k_gather.wgsl:15-44, q6k_gather_batched.wgsl:9-21.
+ * out[m*K + k] = dequant(W)[max(rows[m],0), k], bit-identical to
+ * dequant_kquant (runtime/gguf_loader.cpp:455-573).  rows: i32 [M] (device);
+ * NULL selects rows 0..M-1. */
+BPK_API int bpk_kq_dequant_rows(int type, const void *W,
+                                uint32_t row_stride_words, const int32_t *rows,
+                                uint32_t M, uint32_t K, float *out,
+                                void *stream);
+
+/* ---- MoE expert matmul: replaces the *_matmul_moe indirection ---------------
+ * runtime/kernels/quant_kq/iq4xs_matmul_moe.wgsl:55-66 with offsets from
+ * runtime/kernels/moe/compute_offsets.wgsl:25-36 (decode), and the per-token
+ * form of runtime/ops/moe.cpp:486-592 (expert = expert_indices[tok*k + slot]).
+ * W is the stacked matrix [n_experts*N, K]; expert e owns rows e*N..e*N+N-1.
+ *
+ *   Y[(t*k+s)*N + n] = sum_k X[xrow*K + k] * dequant(W)[idx[t*k+s]*N + n, k]
+ *   xrow = t            when x_per_slot == 0 (gate / up: one X row per token)
+ *        = t*k + s      when x_per_slot != 0 (down: one X row per pair)
+ *
+ * expert_idx: u32 [T*k] (device).  Pairs are grouped by expert on the GPU so
+ * each touched expert's weights are streamed once; no host synchronisation. */
+BPK_API int bpk_kq_moe_matmul(int type, const float *X, const void *W,
+                              const uint32_t *expert_idx, float *Y, uint32_t T,
+                              uint32_t k, uint32_t n_experts, uint32_t N,
+                              uint32_t K, uint32_t n_blocks,
+                              uint32_t row_stride_words, int x_per_slot,
+                              void *stream);
+
+/* Whole routed-expert FFN for T tokens, replacing the per-slot dispatch list of
+ * runtime/model_runner.cpp:3584-3651 (gate, up, silu*mul, down, weighted
+ * accumulate) and the batched form in runtime/ops/moe.cpp:486-592:
+ *   act = silu(gate_e x) * (up_e x);  out[t] = sum_s wt[t,s] * (down_e act)
+ * gate/up: [n_experts*inter, hidden] of type_gu; down: [n_experts*hidden, inter]
+ * of type_dn.  out: f32 [T, hidden], overwritten.  scratch: device memory of
+ * at least bpk_kq_moe_ffn_scratch_bytes(T, k, hidden, inter) bytes. */
+BPK_API size_t bpk_kq_moe_ffn_scratch_bytes(uint32_t T, uint32_t k,
+                                            uint32_t hidden, uint32_t inter);
+BPK_API int bpk_kq_moe_ffn(int type_gu, int type_dn, const float *X,
+                           const void *gate, const void *up, const void *down,
+                           const uint32_t *expert_idx, const float *expert_wt,
+                           float *out, uint32_t T, uint32_t k,
+                           uint32_t n_experts, uint32_t hidden, uint32_t inter,
+                           void *scratch, size_t scratch_bytes, void *stream);
+
+/* ---- introspection for tests and benchmarks --------------------------------
+ * Name of the kernel the last bpk_kq_matmul* call on this thread launched
+ * ("" before the first). */
+BPK_API const char *bpk_last_kernel(void);
+
+/* Force a kernel family for the next calls on this thread (testing only):
+ * 0 = automatic, 1 = generic, 2 = row-per-lane GEMV, 3 = matrix-core small-M,
+ * 4 = matrix-core tiled GEMM.  A forced family that cannot serve the call's
+ * shape fails with BPK_ERR_SHAPE instead of falling back. */
+BPK_API int bpk_force_kernel(int family);
+
+/* Tuning knob for experiments on this thread.  "gemv_splits": number of
+ * K-range splits of the row-per-lane GEMV (0 = automatic). */
+BPK_API int bpk_set_option(const char *name, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BPK_KQUANT_H */
