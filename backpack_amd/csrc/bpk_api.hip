@@ -23,7 +23,7 @@ constexpr uint32_t kCounters = 1u << 16;
 thread_local char t_err[512] = "";
 thread_local const char* t_kernel = "";
 thread_local int t_family = 0;
-thread_local int t_splits = 0;
+thread_local kq::GemvTuning t_gemv;
 
 int fail(int code, const char* fmt, ...)
 {
@@ -124,7 +124,13 @@ int bpk_force_kernel(int family)
 int bpk_set_option(const char* name, int value)
 {
     if (!name) return fail(BPK_ERR_NULL, "option name is null");
-    if (!strcmp(name, "gemv_splits")) { t_splits = value; return BPK_OK; }
+    if (!strcmp(name, "gemv_splits")) { t_gemv.splits = value; return BPK_OK; }
+    if (!strcmp(name, "gemv_waves")) {
+        if (value != 0 && value != 2 && value != 4 && value != 8)
+            return fail(BPK_ERR_SHAPE, "gemv_waves must be 0, 2, 4 or 8");
+        t_gemv.waves = value;
+        return BPK_OK;
+    }
     return fail(BPK_ERR_SHAPE, "unknown option '%s'", name);
 }
 
@@ -261,7 +267,7 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     if (t_family > 2) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
     if ((t_family == 0 || t_family == 2) && rows_ok) {
         t_kernel = "gemv_rows";
-        e = kq::launch_gemv_rows(a, st->split, t_splits, s);
+        e = kq::launch_gemv_rows(a, st->split, t_gemv, s);
     } else {
         t_kernel = "generic";
         e = kq::launch_matmul_generic(a, s);

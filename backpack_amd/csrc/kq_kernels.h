@@ -39,9 +39,13 @@ hipError_t launch_dequant_rows(int type, const uint8_t* W, uint32_t row_stride_b
 hipError_t launch_matmul_generic(const MatmulArgs& a, hipStream_t s);
 
 // Row-per-lane decode GEMV (M <= 4): Q4_K and Q6_K with 16-byte aligned rows.
+struct GemvTuning {
+    int splits = 0;   // workgroups along K, 0 = automatic
+    int waves = 0;    // waves per workgroup (2, 4 or 8), 0 = automatic
+};
 bool gemv_rows_supported(const MatmulArgs& a);
-size_t gemv_rows_scratch_floats(const MatmulArgs& a, int forced_splits);
-hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, int forced_splits,
+size_t gemv_rows_scratch_floats(const MatmulArgs& a, const GemvTuning& t);
+hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const GemvTuning& t,
                             hipStream_t s);
 
 }  // namespace kq

@@ -163,3 +163,31 @@ QWEN3_30B_A3B = {
 def weight_bytes(type_: int, N: int, K: int) -> int:
     """Algorithmic weight bytes (unpadded GGUF size)."""
     return N * n_blocks(K) * BLOCK_BYTES[type_]
+
+
+def make_packed_device(type_: int, N: int, K: int, seed: int = 0, device="cuda"):
+    """Same distributions as make_packed, generated on the GPU with torch's
+    Philox generator (for multi-gigabyte benchmark weight sets).  Returns a
+    uint8 tensor of N*row_stride_words*4 + 16 bytes (16 zero bytes of slack)."""
+    import torch
+    g = torch.Generator(device=device).manual_seed(seed)
+    nb = n_blocks(K)
+    bb = BLOCK_BYTES[type_]
+    rs = row_stride_words(type_, K) * 4
+    rows = torch.zeros((N, rs), dtype=torch.uint8, device=device)
+    blk = torch.randint(0, 256, (N, nb, bb), dtype=torch.uint8, device=device, generator=g)
+
+    def half_scales(cnt):
+        v = (torch.randn((N, nb, cnt), device=device, generator=g) * SIGMA).abs().to(torch.float16)
+        return v.view(torch.uint8).reshape(N, nb, 2 * cnt)
+
+    if type_ == Q4_K:
+        blk[:, :, 0:4] = half_scales(2)          # 12 scale bytes and the quants stay uniform
+    elif type_ == Q6_K:
+        sc = torch.randint(-64, 64, (N, nb, 16), dtype=torch.int8, device=device, generator=g)
+        blk[:, :, 192:208] = sc.view(torch.uint8)
+        blk[:, :, 208:210] = half_scales(1)
+    else:
+        raise ValueError(f"unsupported k-quant type {type_}")
+    rows[:, : nb * bb] = blk.reshape(N, nb * bb)
+    return torch.cat([rows.reshape(-1), torch.zeros(16, dtype=torch.uint8, device=device)])

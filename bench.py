@@ -1,0 +1,281 @@
+#!/usr/bin/env python3
+"""Benchmark of the k-quant decode path on one MI355X.
+
+A step is one pass of the Llama-3-8B-shaped decode layer set at M = 1 in the
+Q4_K_M mix: per layer q|k|v (Q4_K 6144x4096), o (Q4_K 4096x4096), gate|up
+(Q4_K 28672x4096), down (Q6_K 4096x14336), 32 layers with distinct weights,
+plus a Q6_K lm_head 128256x4096 — 129 launches reading 4 841 250 816 weight
+bytes, far beyond the 256 MB last-level cache, all resident in HBM before the
+timed region.  Launches go to one stream in order; by default the step is
+recorded once into a HIP graph and replayed, like the reference's pre-recorded
+per-token command buffer (runtime/model_runner.cpp:5725-5759).
+
+Prints ONE JSON line.  `value` is weight+activation bytes of the step divided by
+wall time.  `roofline` covers the dominant kernel (the Q4_K GEMV on gate|up,
+48 % of the bytes), timed with HIP events on the launch stream over its own
+region of 32 distinct matrices.  `cpu_baseline` times the reference's CPU path
+(dequantise to fp32, sequential fp32 dot) on a bounded sample on the host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+METRIC = "Q4_K M=1 matvec HBM GB/s (% of peak); M=2048 dequant-GEMM TFLOPS (% MFMA)"
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE (profiles/q4k_gemv_gate_up_pmc.txt), scaled by a copy kernel of
+# known size; None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--layers", type=int, default=32, help="layers in the set (32 = the named workload)")
+    ap.add_argument("--prefill", action="store_true", help="also time the M=2048 prefill GEMM on one layer")
+    return ap.parse_args()
+
+
+def build_layer_set(n_layers):
+    import torch
+    from backpack_amd import kquant, synth
+    spec = synth.LLAMA3_8B
+    mats = []   # (name, KQuantPacked, x, y)
+    xs, ys = {}, {}
+    seed = 0
+    for layer in range(n_layers):
+        for name, type_, N, K in spec["layer"]:
+            data = synth.make_packed_device(type_, N, K, seed=seed)
+            seed += 1
+            nb, rs = synth.n_blocks(K), synth.row_stride_words(type_, K)
+            w = kquant.KQuantPacked(data, type_, N, K, rs, nb)
+            if K not in xs:
+                g = torch.Generator(device="cuda").manual_seed(1000 + K)
+                xs[K] = torch.randn(1, K, device="cuda", generator=g)
+            if N not in ys:
+                ys[N] = torch.empty(1, N, device="cuda")
+            mats.append((name, w, xs[K], ys[N]))
+    name, type_, N, K = spec["lm_head"]
+    data = synth.make_packed_device(type_, N, K, seed=seed)
+    w = kquant.KQuantPacked(data, type_, N, K, synth.row_stride_words(type_, K), synth.n_blocks(K))
+    ys[N] = torch.empty(1, N, device="cuda")
+    mats.append((name, w, xs[K], ys[N]))
+    return mats
+
+
+def algorithmic_bytes(mats, M=1):
+    from backpack_amd import synth
+    wb = sum(synth.weight_bytes(w.type, w.N, w.K) for _, w, _, _ in mats)
+    act = sum((w.K + w.N) * 4 * M for _, w, _, _ in mats)
+    return wb, act
+
+
+def run_region(mats, steps, warmup, use_graph):
+    """Times `steps` passes over mats with HIP events on the current stream."""
+    import torch
+    from backpack_amd import kquant
+
+    def one_pass():
+        for _, w, x, y in mats:
+            kquant.matmul(x, w, out=y)
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        one_pass()
+        stream.synchronize()
+        if use_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                one_pass()
+            step = graph.replay
+        else:
+            step = one_pass
+        for _ in range(warmup):
+            step()
+        stream.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for _ in range(steps):
+            step()
+        e1.record(stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    return e0.elapsed_time(e1) * 1e-3, wall
+
+
+def cpu_baseline():
+    """The reference's CPU path on one layer + lm_head of the same workload,
+    single thread, then the same rows split over all host threads."""
+    import concurrent.futures as cf
+
+    import numpy as np
+    from backpack_amd import synth
+    from oracle import kqo
+
+    use_ref = kqo.ref() is not None
+    spec = synth.LLAMA3_8B
+    sample = list(spec["layer"]) + [spec["lm_head"]]
+    rng = np.random.default_rng(0)
+    total_bytes, t_deq, t_dot = 0, 0.0, 0.0
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    t_par = 0.0
+    for i, (name, type_, N, K) in enumerate(sample):
+        # the CPU leg only needs bytes of the right shape: uniform random
+        # blocks with fixed small fp16 super-scales (no NaNs), cheap to make
+        bb = synth.BLOCK_BYTES[type_]
+        nb = synth.n_blocks(K)
+        raw = rng.integers(0, 256, size=(N, nb, bb), dtype=np.uint8)
+        for off in ((0, 2) if type_ == synth.Q4_K else (208,)):
+            raw[:, :, off] = 0x1F
+            raw[:, :, off + 1] = 0x20
+        raw = raw.reshape(N, nb * bb)
+        x = rng.standard_normal((1, K)).astype(np.float32)
+        _, td, tm = kqo.matmul_timed(type_, x, raw, N, K, use_ref=use_ref)
+        t_deq += td
+        t_dot += tm
+        total_bytes += N * nb * bb
+        # all-core leg: contiguous row slabs, one per thread (ctypes drops the GIL)
+        slabs = np.array_split(np.arange(N), cores)
+        t0 = time.perf_counter()
+        with cf.ThreadPoolExecutor(cores) as ex:
+            list(ex.map(lambda s: kqo.matmul_timed(type_, x, raw[s[0]:s[-1] + 1], len(s), K, use_ref=use_ref),
+                        [s for s in slabs if len(s)]))
+        t_par += time.perf_counter() - t0
+        del raw
+    one = total_bytes / (t_deq + t_dot) / 1e9
+    return {
+        "value": round(one, 4), "unit": "GB/s", "cores": 1,
+        "kind": "reference" if use_ref else "port",
+        "sample": "one layer (qkv, o, gate_up, down) + lm_head of the same workload, "
+                  f"{total_bytes} weight bytes; dequant {t_deq:.2f} s + dot {t_dot:.2f} s",
+        "dequant_s": round(t_deq, 3), "dot_s": round(t_dot, 3),
+        "all_cores": {"value": round(total_bytes / t_par / 1e9, 4), "unit": "GB/s", "cores": cores},
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this path has no multi-GPU leg (asked for --gpus {args.gpus}); "
+              "it shards by output rows with no exchange, so N GPUs run N independent copies of this "
+              "benchmark on 1/N of the rows.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from backpack_amd import capi, synth
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    capi.check(capi.lib().bpk_init(0))
+
+    mats = build_layer_set(args.layers)
+    torch.cuda.synchronize()
+    wb, act = algorithmic_bytes(mats)
+    use_graph = not args.no_graph
+
+    sec, wall = run_region(mats, args.steps, args.warmup, use_graph)
+    ms_per_step = sec / args.steps * 1e3
+    gbs = (wb + act) / (sec / args.steps) / 1e9
+
+    # dominant kernel: the Q4_K GEMV on gate|up, every layer's own matrix
+    dom = [m for m in mats if m[0] == "gate_up"]
+    dsec, _ = run_region(dom, max(args.steps, 10), args.warmup, use_graph)
+    launches = len(dom) * max(args.steps, 10)
+    dom_w = dom[0][1]
+    dom_bytes = synth.weight_bytes(dom_w.type, dom_w.N, dom_w.K) + (dom_w.K + dom_w.N) * 4
+    dom_gbs = dom_bytes / (dsec / launches) / 1e9
+    roofline = {
+        "kernel": "kq::q4k_gemv_kernel (gate|up 28672x4096, M=1)",
+        "bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
+        "bytes_per_launch": dom_bytes, "us_per_launch": round(dsec / launches * 1e6, 3),
+        "traffic": MEASURED_TRAFFIC_BYTES,
+    }
+
+    # per-shape breakdown (extra information, same protocol)
+    shapes = {}
+    for name in ("qkv", "o", "down", "lm_head"):
+        sel = [m for m in mats if m[0] == name]
+        reps = max(args.steps, 10) * (8 if name == "lm_head" else 1)
+        s, _ = run_region(sel, reps, 2, use_graph)
+        w = sel[0][1]
+        b = synth.weight_bytes(w.type, w.N, w.K) + (w.K + w.N) * 4
+        shapes[name] = {"us": round(s / (len(sel) * reps) * 1e6, 2),
+                        "GBps": round(b / (s / (len(sel) * reps)) / 1e9, 1)}
+    shapes["gate_up"] = {"us": roofline["us_per_launch"], "GBps": roofline["achieved"]}
+
+    out = {
+        "metric": METRIC, "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8 weights, f32 activations and accumulation", "data": "synthetic",
+        "config": {"workload": "Llama-3-8B-shaped decode layer set, M=1, Q4_K_M mix "
+                               f"({args.layers} layers x [qkv, o, gate_up, down] + lm_head)",
+                   "launches_per_step": len(mats), "weight_bytes": wb, "activation_bytes": act,
+                   "graph_replay": use_graph},
+        "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 2),
+        "tokens_per_s_equiv": round(args.steps / sec, 1),
+        "host_wall_ms_per_step": round(wall / args.steps * 1e3, 4),
+        "roofline": roofline,
+        "per_shape": shapes,
+    }
+    if args.prefill:
+        out["prefill"] = prefill_leg()
+    if not args.no_cpu:
+        del mats, dom
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+def prefill_leg(M=2048):
+    """M=2048 bf16 dequant-GEMM over one layer's four matrices + lm_head."""
+    import torch
+    from backpack_amd import kquant, synth
+    spec = synth.LLAMA3_8B
+    res = {}
+    flops_total, sec_total = 0.0, 0.0
+    for name, type_, N, K in list(spec["layer"]) + [spec["lm_head"]]:
+        data = synth.make_packed_device(type_, N, K, seed=77)
+        w = kquant.KQuantPacked(data, type_, N, K, synth.row_stride_words(type_, K), synth.n_blocks(K))
+        x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+        y = torch.empty(M, N, device="cuda")
+        for _ in range(2):
+            kquant.matmul(x, w, out=y)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 5
+        e0.record()
+        for _ in range(reps):
+            kquant.matmul(x, w, out=y)
+        e1.record()
+        torch.cuda.synchronize()
+        s = e0.elapsed_time(e1) * 1e-3 / reps
+        fl = 2.0 * M * N * K
+        res[name] = {"ms": round(s * 1e3, 3), "TFLOPs": round(fl / s / 1e12, 1)}
+        weight = 32 if name != "lm_head" else 1
+        flops_total += fl * weight
+        sec_total += s * weight
+        del data, w, x, y
+    tf = flops_total / sec_total / 1e12
+    res["layer_set"] = {"TFLOPs": round(tf, 1), "pct_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS * 100, 2),
+                        "M": M, "ms_extrapolated": round(sec_total * 1e3, 2)}
+    return res
+
+
+if __name__ == "__main__":
+    main()

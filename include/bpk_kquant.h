@@ -185,8 +185,9 @@ BPK_API const char *bpk_last_kernel(void);
  * shape fails with BPK_ERR_SHAPE instead of falling back. */
 BPK_API int bpk_force_kernel(int family);
 
-/* Tuning knob for experiments on this thread.  "gemv_splits": number of
- * K-range splits of the row-per-lane GEMV (0 = automatic). */
+/* Tuning knobs for experiments on this thread.  "gemv_splits": number of
+ * K-range splits of the row-per-lane GEMV; "gemv_waves": its waves per
+ * workgroup (2, 4 or 8).  0 = automatic. */
 BPK_API int bpk_set_option(const char *name, int value);
 
 #ifdef __cplusplus

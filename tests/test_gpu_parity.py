@@ -130,21 +130,27 @@ def test_matmul_vs_oracle(gpu, kqo, type_, M, N, K, family):
     _say("   kernel", kern, r)
 
 
-@pytest.mark.parametrize("splits", [1, 2, 3, 4, 16])
-def test_gemv_split_k_and_counter_reset(gpu, kqo, splits):
+@pytest.mark.parametrize("type_", [Q4_K, Q6_K])
+@pytest.mark.parametrize("waves", [2, 4, 8])
+@pytest.mark.parametrize("splits", [1, 2, 3, 16])
+def test_gemv_split_k_and_counter_reset(gpu, kqo, type_, waves, splits):
     from backpack_amd import capi, kquant
-    type_, N, K = Q4_K, 200, 4096
+    N, K, M = 200, 4096, 2
     raw, packed, w = gpu.make_weight(type_, N, K, seed=5)
-    X = np.random.default_rng(splits).standard_normal((1, K)).astype(np.float32)
+    X = np.random.default_rng(splits).standard_normal((M, K)).astype(np.float32)
     capi.set_option("gemv_splits", splits)
+    capi.set_option("gemv_waves", waves)
     try:
+        _say("split", type_, waves, splits)
         xd = gpu.dev(X)
         a = kquant.matmul(xd, w).cpu().numpy()
+        assert capi.last_kernel() == "gemv_rows"
         b = kquant.matmul(xd, w).cpu().numpy()          # counters must have been re-armed
     finally:
         capi.set_option("gemv_splits", 0)
+        capi.set_option("gemv_waves", 0)
     assert np.array_equal(a, b), "split-K result depends on the launch"
-    gpu.check_matmul(kqo, type_, a, X, packed, N, K, label=f"splits={splits}")
+    gpu.check_matmul(kqo, type_, a, X, packed, N, K, label=f"waves={waves} splits={splits}")
 
 
 def test_matmul_y_offset_no_bias(gpu, kqo):
