@@ -24,6 +24,7 @@ thread_local char t_err[512] = "";
 thread_local const char* t_kernel = "";
 thread_local int t_family = 0;
 thread_local kq::GemvTuning t_gemv;
+thread_local int t_gemm_tile = 0;
 
 int fail(int code, const char* fmt, ...)
 {
@@ -129,6 +130,11 @@ int bpk_set_option(const char* name, int value)
         if (value != 0 && value != 2 && value != 4 && value != 8)
             return fail(BPK_ERR_SHAPE, "gemv_waves must be 0, 2, 4 or 8");
         t_gemv.waves = value;
+        return BPK_OK;
+    }
+    if (!strcmp(name, "gemm_tile")) {
+        if (value != 0 && value != 128 && value != 256) return fail(BPK_ERR_SHAPE, "gemm_tile must be 0, 128 or 256");
+        t_gemm_tile = value;
         return BPK_OK;
     }
     return fail(BPK_ERR_SHAPE, "unknown option '%s'", name);
@@ -279,8 +285,19 @@ int bpk_kq_matmul_bf16(int type, const uint16_t* X, const void* W, const float* 
                        uint32_t N, uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, void* stream)
 {
     if (int rc = check_matmul(type, X, W, Y, M, N, K, n_blocks, row_stride_words)) return rc;
-    (void)bias; (void)stream;
-    return fail(BPK_ERR_SHAPE, "bf16 prefill GEMM is not built yet");
+    if (M == 0) return BPK_OK;
+    if (int rc = current_state(nullptr)) return rc;
+    kq::MatmulArgs a{};
+    a.type = type; a.X = X; a.W = (const uint8_t*)W; a.bias = bias; a.Y = Y;
+    a.M = M; a.N = N; a.K = K; a.n_blocks = n_blocks;
+    a.row_stride_bytes = row_stride_words * 4u;
+    a.y_offset = 0;
+    a.ldy = N;
+    if (!kq::gemm_bf16_supported(a))
+        return fail(BPK_ERR_ALIGN, "bf16 GEMM needs 16-byte aligned X and (for Q4_K) 16-byte aligned W rows");
+    t_kernel = "gemm_bf16";
+    hipError_t e = kq::launch_gemm_bf16(a, t_gemm_tile, (hipStream_t)stream);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
 }
 
 int bpk_kq_dequant_rows(int type, const void* W, uint32_t row_stride_words, const int32_t* rows, uint32_t M,

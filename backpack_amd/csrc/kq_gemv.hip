@@ -486,9 +486,11 @@ static hipError_t launch_one(const GemvParams& p, hipStream_t s)
     const size_t shmem = tiles + xs > red ? tiles + xs : red;
     if (shmem > 160u * 1024u) return hipErrorInvalidValue;
     auto kern = TYPE == KQ_TYPE_Q4_K ? q4k_gemv_kernel<MT, NW> : q6k_gemv_kernel<MT, NW>;
-    if (shmem > 64u * 1024u) {
+    static size_t raised = 64u * 1024u;   // per instantiation
+    if (shmem > raised) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return e;
+        raised = shmem;
     }
     hipLaunchKernelGGL(kern, dim3(groups, p.n_splits), dim3(64 * NW), shmem, s, p);
     return hipGetLastError();

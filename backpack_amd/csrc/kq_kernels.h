@@ -48,4 +48,9 @@ size_t gemv_rows_scratch_floats(const MatmulArgs& a, const GemvTuning& t);
 hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const GemvTuning& t,
                             hipStream_t s);
 
+// Prefill GEMM on the matrix cores: X bf16 [M,K], Y f32.  tile = 0 (automatic),
+// 128 or 256 (square workgroup tile).
+bool gemm_bf16_supported(const MatmulArgs& a);
+hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, hipStream_t s);
+
 }  // namespace kq

@@ -210,3 +210,62 @@ def test_moe_matmul_vs_oracle(gpu, kqo, type_, N, K, per_slot):
     want = kqo.moe_matmul(type_, X, packed, eidx, N, K, x_per_slot=per_slot)
     rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
     assert np.all(np.abs(got - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
+
+
+# ---- prefill GEMM on the matrix cores (bf16 X) -------------------------------------------
+GEMM_SHAPES = [
+    # type, M, N, K, tile
+    (Q4_K, 128, 128, 256, 128),
+    (Q4_K, 256, 256, 512, 256),
+    (Q4_K, 200, 300, 1024, 128),     # ragged M and N
+    (Q4_K, 300, 520, 768, 256),
+    (Q4_K, 512, 1024, 4096, 0),
+    (Q4_K, 33, 70, 2048, 0),
+    (Q6_K, 128, 128, 256, 128),
+    (Q6_K, 256, 256, 768, 256),      # odd block count: rows only 8-byte aligned
+    (Q6_K, 190, 260, 1024, 128),
+    (Q6_K, 512, 512, 4096, 0),
+]
+
+
+def _bf16_bits(x32):
+    """Round-to-nearest-even fp32 -> bf16 bit patterns (numpy)."""
+    u = x32.view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+@pytest.mark.parametrize("type_,M,N,K,tile", GEMM_SHAPES)
+def test_gemm_bf16_vs_oracle(gpu, kqo, type_, M, N, K, tile):
+    import torch
+    from backpack_amd import capi, kquant
+    raw, packed, w = gpu.make_weight(type_, N, K, seed=M + N)
+    rng = np.random.default_rng(K + M)
+    X = rng.standard_normal((M, K)).astype(np.float32)
+    bits = _bf16_bits(X)
+    bias = rng.standard_normal(N).astype(np.float32)
+    xd = torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
+    capi.set_option("gemm_tile", tile)
+    try:
+        _say("gemm", type_, M, N, K, tile)
+        got = kquant.matmul(xd, w, bias=gpu.dev(bias)).cpu().numpy()
+        assert capi.last_kernel() == "gemm_bf16"
+    finally:
+        capi.set_option("gemm_tile", 0)
+    Xw = (bits.astype(np.uint32) << 16).view(np.float32)
+    cpu = kqo.matmul(type_, Xw, packed, N, K, bias=bias)        # the reference's fp32 CPU path
+    err = np.abs(got.astype(np.float64) - cpu)
+    peak, rms = float(np.abs(cpu).max()), float(np.sqrt(np.mean(cpu.astype(np.float64) ** 2)))
+    # (1) the stated bar for the bf16 matrix-core path: 1e-2, relative to the
+    #     largest output (bf16 weights carry a unit roundoff of 2^-8, so an
+    #     output near zero can be off by more than 1e-2 of its own size)
+    assert err.max() <= 1e-2 * peak, f"max error {err.max():.3g} vs 1e-2*peak {1e-2 * peak:.3g}"
+    # (2) in aggregate the error is far smaller
+    fro = float(np.sqrt((err ** 2).sum() / (cpu.astype(np.float64) ** 2).sum()))
+    assert fro <= 4e-3, f"Frobenius relative error {fro:.3g}"
+    # (3) and it is *only* that rounding: against the exact contraction of the
+    #     bf16-rounded weights the kernel is accurate to fp32 accumulation
+    deq = kqo.dequant(type_, raw, N, K)
+    wbf = (_bf16_bits(deq).astype(np.uint32) << 16).view(np.float32)
+    exact = Xw.astype(np.float64) @ wbf.astype(np.float64).T + bias.astype(np.float64)
+    assert np.abs(got - exact).max() <= 2e-5 * peak + K * 2.0 ** -24 * rms
+    _say(f"    max err/peak {err.max() / peak:.2e}  max err/rms {err.max() / rms:.2e}  frobenius {fro:.2e}")
