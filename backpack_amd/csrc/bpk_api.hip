@@ -132,6 +132,11 @@ int bpk_set_option(const char* name, int value)
         t_gemv.waves = value;
         return BPK_OK;
     }
+    if (!strcmp(name, "gemv_depth")) {
+        if (value != 0 && value != 1 && value != 2 && value != 4) return fail(BPK_ERR_SHAPE, "gemv_depth must be 0, 1, 2 or 4");
+        t_gemv.depth = value;
+        return BPK_OK;
+    }
     if (!strcmp(name, "gemm_tile")) {
         if (value != 0 && value != 128 && value != 256) return fail(BPK_ERR_SHAPE, "gemm_tile must be 0, 128 or 256");
         t_gemm_tile = value;
@@ -269,9 +274,14 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
     const bool rows_ok = kq::gemv_rows_supported(a);
+    const bool mrow_ok = kq::mrow_supported(a);
     if (t_family == 2 && !rows_ok) return fail(BPK_ERR_SHAPE, "row-per-lane GEMV cannot serve this call");
-    if (t_family > 2) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
-    if ((t_family == 0 || t_family == 2) && rows_ok) {
+    if (t_family == 3 && !mrow_ok) return fail(BPK_ERR_SHAPE, "matrix-core row kernel cannot serve this call");
+    if (t_family > 3) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
+    if ((t_family == 0 || t_family == 3) && mrow_ok) {
+        t_kernel = "mrow";
+        e = kq::launch_mrow(a, st->split, t_gemv, nullptr, nullptr, 1, 0, s);
+    } else if ((t_family == 0 || t_family == 2) && rows_ok) {
         t_kernel = "gemv_rows";
         e = kq::launch_gemv_rows(a, st->split, t_gemv, s);
     } else {

@@ -42,11 +42,18 @@ hipError_t launch_matmul_generic(const MatmulArgs& a, hipStream_t s);
 struct GemvTuning {
     int splits = 0;   // workgroups along K, 0 = automatic
     int waves = 0;    // waves per workgroup (2, 4 or 8), 0 = automatic
+    int depth = 0;    // superblocks a wave keeps in flight (1, 2 or 4), 0 = automatic
 };
 bool gemv_rows_supported(const MatmulArgs& a);
 size_t gemv_rows_scratch_floats(const MatmulArgs& a, const GemvTuning& t);
 hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const GemvTuning& t,
                             hipStream_t s);
+
+// Row-per-lane matvec on the matrix cores, M <= 16 dense or grouped by expert.
+bool mrow_supported(const MatmulArgs& a);
+size_t mrow_scratch_floats(const MatmulArgs& a, const GemvTuning& t);
+hipError_t launch_mrow(const MatmulArgs& a, const SplitScratch& sc, const GemvTuning& t, const uint32_t* tiles,
+                       const uint32_t* n_tiles, uint32_t tiles_bound, int sets, hipStream_t s);
 
 // Prefill GEMM on the matrix cores: X bf16 [M,K], Y f32.  tile = 0 (automatic),
 // 128 or 256 (square workgroup tile).

@@ -187,7 +187,8 @@ BPK_API int bpk_force_kernel(int family);
 
 /* Tuning knobs for experiments on this thread.  "gemv_splits": number of
  * K-range splits of the row-per-lane GEMV; "gemv_waves": its waves per
- * workgroup (2, 4 or 8); "gemm_tile": square workgroup tile of the bf16 GEMM
+ * workgroup (2, 4 or 8); "gemv_depth": superblocks a wave keeps in flight
+ * (1, 2 or 4); "gemm_tile": square workgroup tile of the bf16 GEMM
  * (128 or 256).  0 = automatic. */
 BPK_API int bpk_set_option(const char *name, int value);
 

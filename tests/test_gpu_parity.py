@@ -108,11 +108,15 @@ SHAPES = [
     (Q6_K, 2, 70, 2048),
     (Q6_K, 4, 33, 768),
     (Q6_K, 8, 40, 1024),
+    (Q6_K, 16, 130, 2048),
+    (Q4_K, 7, 300, 4096),
+    (Q4_K, 12, 64, 768),
+    (Q6_K, 3, 2048, 768),       # the MoE down projection: odd block count, 632-byte rows
 ]
 
 
 @pytest.mark.parametrize("type_,M,N,K", SHAPES)
-@pytest.mark.parametrize("family", [0, 1])
+@pytest.mark.parametrize("family", [0, 1, 2, 3])
 def test_matmul_vs_oracle(gpu, kqo, type_, M, N, K, family):
     from backpack_amd import capi, kquant
     raw, packed, w = gpu.make_weight(type_, N, K, seed=N + K)
@@ -122,35 +126,44 @@ def test_matmul_vs_oracle(gpu, kqo, type_, M, N, K, family):
     capi.force_kernel(family)
     try:
         _say("matmul", type_, M, N, K, "family", family)
-        got = kquant.matmul(gpu.dev(X), w, bias=gpu.dev(bias)).cpu().numpy()
+        try:
+            got = kquant.matmul(gpu.dev(X), w, bias=gpu.dev(bias)).cpu().numpy()
+        except capi.BpkError as e:
+            assert family >= 2 and e.code == -2, e     # a forced family may decline a shape
+            pytest.skip(f"family {family} declines this shape")
         kern = capi.last_kernel()
     finally:
         capi.force_kernel(0)
-    r = gpu.check_matmul(kqo, type_, got, X, packed, N, K, bias=bias, label=f"{kern} {type_} {M}x{N}x{K}")
+    r = gpu.check_matmul(kqo, type_, got, X, packed, N, K, bias=bias, label=f"{kern} {type_} {M}x{N}x{K}",
+                         slack=1e-5 if kern == "mrow" else 1e-6)
     _say("   kernel", kern, r)
 
 
 @pytest.mark.parametrize("type_", [Q4_K, Q6_K])
+@pytest.mark.parametrize("family,kernel", [(2, "gemv_rows"), (3, "mrow")])
 @pytest.mark.parametrize("waves", [2, 4, 8])
 @pytest.mark.parametrize("splits", [1, 2, 3, 16])
-def test_gemv_split_k_and_counter_reset(gpu, kqo, type_, waves, splits):
+def test_gemv_split_k_and_counter_reset(gpu, kqo, type_, family, kernel, waves, splits):
     from backpack_amd import capi, kquant
     N, K, M = 200, 4096, 2
     raw, packed, w = gpu.make_weight(type_, N, K, seed=5)
     X = np.random.default_rng(splits).standard_normal((M, K)).astype(np.float32)
     capi.set_option("gemv_splits", splits)
     capi.set_option("gemv_waves", waves)
+    capi.force_kernel(family)
     try:
-        _say("split", type_, waves, splits)
+        _say("split", type_, kernel, waves, splits)
         xd = gpu.dev(X)
         a = kquant.matmul(xd, w).cpu().numpy()
-        assert capi.last_kernel() == "gemv_rows"
+        assert capi.last_kernel() == kernel
         b = kquant.matmul(xd, w).cpu().numpy()          # counters must have been re-armed
     finally:
+        capi.force_kernel(0)
         capi.set_option("gemv_splits", 0)
         capi.set_option("gemv_waves", 0)
     assert np.array_equal(a, b), "split-K result depends on the launch"
-    gpu.check_matmul(kqo, type_, a, X, packed, N, K, label=f"waves={waves} splits={splits}")
+    gpu.check_matmul(kqo, type_, a, X, packed, N, K, label=f"waves={waves} splits={splits}",
+                     slack=1e-5 if kernel == "mrow" else 1e-6)
 
 
 def test_matmul_y_offset_no_bias(gpu, kqo):
