@@ -19,6 +19,7 @@ namespace {
 constexpr int kMaxDevices = 16;
 constexpr size_t kPartialFloats = size_t(4) << 20;  // 16 MiB of split-K partial sums
 constexpr uint32_t kCounters = 1u << 16;
+constexpr size_t kMoeWords = size_t(4) << 20;       // 16 MiB of tile records for bpk_kq_moe_matmul
 
 thread_local char t_err[512] = "";
 thread_local const char* t_kernel = "";
@@ -43,6 +44,7 @@ int hip_fail(hipError_t e, const char* what)
 struct DeviceState {
     bool ready = false;
     kq::SplitScratch split{};
+    uint32_t* moe_tiles = nullptr;   // kMoeWords words
 };
 
 std::mutex g_mu;
@@ -66,6 +68,7 @@ int ensure_device(int device, DeviceState** out)
         e = hipMalloc((void**)&st.split.partial, kPartialFloats * sizeof(float));
         if (e == hipSuccess) e = hipMalloc((void**)&st.split.counters, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMemset(st.split.counters, 0, kCounters * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipMalloc((void**)&st.moe_tiles, kMoeWords * sizeof(uint32_t));
         if (cur != device && cur >= 0) (void)hipSetDevice(cur);
         if (e != hipSuccess) return hip_fail(e, "allocating split-K scratch");
         st.split.capacity_floats = kPartialFloats;
@@ -158,6 +161,7 @@ int bpk_shutdown(void)
         (void)hipSetDevice(d);
         (void)hipFree(st.split.partial);
         (void)hipFree(st.split.counters);
+        (void)hipFree(st.moe_tiles);
         st = DeviceState{};
     }
     if (cur >= 0) (void)hipSetDevice(cur);
@@ -334,7 +338,8 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
     if (k == 0 || n_experts == 0) return fail(BPK_ERR_SHAPE, "k and n_experts must be positive");
     if ((uint64_t)T * k > 0xFFFFFFFFull) return fail(BPK_ERR_SHAPE, "T*k overflows");
     if (T == 0) return BPK_OK;
-    if (int rc = current_state(nullptr)) return rc;
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
     kq::MatmulArgs a{};
     a.type = type; a.X = X; a.W = (const uint8_t*)W; a.bias = nullptr; a.Y = Y;
     a.M = T * k; a.N = N; a.K = K; a.n_blocks = n_blocks;
@@ -344,15 +349,30 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
     a.expert_idx = expert_idx;
     a.k_slots = k;
     a.x_per_slot = x_per_slot;
-    t_kernel = "generic_indirect";
-    hipError_t e = kq::launch_matmul_generic(a, (hipStream_t)stream);
+    hipStream_t s = (hipStream_t)stream;
+    const int sets = kq::moe_sets_for(T * k, n_experts);
+    hipError_t e;
+    if (t_family != 1 && kq::mrow_supported(a) && n_experts <= 8192u &&
+        kq::moe_tiles_bound(T * k, n_experts, sets) <= 65535u &&
+        kq::moe_tiles_words(T * k, n_experts, sets) <= kMoeWords) {
+        t_kernel = "mrow_grouped";
+        uint32_t* n_tiles = st->moe_tiles;
+        uint32_t* tiles = st->moe_tiles + 1;
+        e = kq::launch_moe_group(expert_idx, T * k, n_experts, sets, tiles, n_tiles, s);
+        if (e == hipSuccess)
+            e = kq::launch_mrow(a, st->split, t_gemv, tiles, n_tiles, kq::moe_tiles_bound(T * k, n_experts, sets), sets, s);
+    } else {
+        t_kernel = "generic_indirect";
+        e = kq::launch_matmul_generic(a, s);
+    }
     return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
 }
 
 size_t bpk_kq_moe_ffn_scratch_bytes(uint32_t T, uint32_t k, uint32_t hidden, uint32_t inter)
 {
-    // gate, up (act written over gate) and the per-pair down outputs
-    return ((size_t)T * k * inter * 2 + (size_t)T * k * hidden) * sizeof(float);
+    // gate, up (the activation overwrites gate), per-pair down outputs, tile records
+    const size_t P = (size_t)T * k;
+    return (P * inter * 2 + P * hidden) * sizeof(float) + (P * 10 + 4) * sizeof(uint32_t);
 }
 
 int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, const void* up, const void* down,
@@ -360,10 +380,61 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
                    uint32_t n_experts, uint32_t hidden, uint32_t inter, void* scratch, size_t scratch_bytes,
                    void* stream)
 {
-    (void)type_gu; (void)type_dn; (void)X; (void)gate; (void)up; (void)down; (void)expert_idx; (void)expert_wt;
-    (void)out; (void)T; (void)k; (void)n_experts; (void)hidden; (void)inter; (void)scratch; (void)scratch_bytes;
-    (void)stream;
-    return fail(BPK_ERR_SHAPE, "MoE FFN is not built yet");
+    if (!known_type(type_gu) || !known_type(type_dn)) return fail(BPK_ERR_TYPE, "unsupported GGUF type");
+    if (!X || !gate || !up || !down || !expert_idx || !expert_wt || !out)
+        return fail(BPK_ERR_NULL, "X, gate, up, down, expert_idx, expert_wt and out must be non-null");
+    if (k == 0 || n_experts == 0) return fail(BPK_ERR_SHAPE, "k and n_experts must be positive");
+    if (hidden == 0 || hidden % KQ_QK || inter == 0 || inter % KQ_QK)
+        return fail(BPK_ERR_SHAPE, "hidden=%u and inter=%u must be positive multiples of 256", hidden, inter);
+    if ((uint64_t)T * k > 0x0FFFFFFFull) return fail(BPK_ERR_SHAPE, "T*k too large");
+    if (T == 0) return BPK_OK;
+    if (!scratch || scratch_bytes < bpk_kq_moe_ffn_scratch_bytes(T, k, hidden, inter))
+        return fail(BPK_ERR_WORKSPACE, "scratch must hold %zu bytes", bpk_kq_moe_ffn_scratch_bytes(T, k, hidden, inter));
+    if ((uintptr_t)scratch & 15u) return fail(BPK_ERR_ALIGN, "scratch must be 16-byte aligned");
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    const uint32_t P = T * k;
+    float* G = (float*)scratch;
+    float* U = G + (size_t)P * inter;
+    float* D = U + (size_t)P * inter;
+    uint32_t* n_tiles = (uint32_t*)(D + (size_t)P * hidden);
+    uint32_t* tiles = n_tiles + 4;
+    const int sets = kq::moe_sets_for(P, n_experts);
+    const uint32_t bound = kq::moe_tiles_bound(P, n_experts, sets);
+
+    uint32_t nb_gu, rs_gu, nb_dn, rs_dn;
+    bpk_kq_layout(type_gu, hidden, &nb_gu, &rs_gu);
+    bpk_kq_layout(type_dn, inter, &nb_dn, &rs_dn);
+    kq::MatmulArgs a{};
+    a.type = type_gu; a.X = X; a.W = (const uint8_t*)gate; a.Y = G;
+    a.M = P; a.N = inter; a.K = hidden; a.n_blocks = nb_gu; a.row_stride_bytes = rs_gu * 4u; a.ldy = inter;
+    a.expert_idx = expert_idx; a.k_slots = k; a.x_per_slot = 0;
+    kq::MatmulArgs d{};
+    d.type = type_dn; d.X = G; d.W = (const uint8_t*)down; d.Y = D;
+    d.M = P; d.N = hidden; d.K = inter; d.n_blocks = nb_dn; d.row_stride_bytes = rs_dn * 4u; d.ldy = hidden;
+    d.expert_idx = expert_idx; d.k_slots = k; d.x_per_slot = 1;
+    const bool fast = t_family != 1 && n_experts <= 8192u && bound <= 65535u && kq::mrow_supported(a) &&
+                      kq::mrow_supported(d);
+    hipError_t e = hipSuccess;
+    if (fast) {
+        t_kernel = "moe_ffn_mrow";
+        e = kq::launch_moe_group(expert_idx, P, n_experts, sets, tiles, n_tiles, s);
+        if (e == hipSuccess) e = kq::launch_mrow(a, st->split, t_gemv, tiles, n_tiles, bound, sets, s);
+        a.W = (const uint8_t*)up; a.Y = U;
+        if (e == hipSuccess) e = kq::launch_mrow(a, st->split, t_gemv, tiles, n_tiles, bound, sets, s);
+        if (e == hipSuccess) e = kq::launch_moe_silu_mul(G, U, G, (size_t)P * inter, s);
+        if (e == hipSuccess) e = kq::launch_mrow(d, st->split, t_gemv, tiles, n_tiles, bound, sets, s);
+    } else {
+        t_kernel = "moe_ffn_generic";
+        e = kq::launch_matmul_generic(a, s);
+        a.W = (const uint8_t*)up; a.Y = U;
+        if (e == hipSuccess) e = kq::launch_matmul_generic(a, s);
+        if (e == hipSuccess) e = kq::launch_moe_silu_mul(G, U, G, (size_t)P * inter, s);
+        if (e == hipSuccess) e = kq::launch_matmul_generic(d, s);
+    }
+    if (e == hipSuccess) e = kq::launch_moe_combine(D, expert_wt, out, T, k, hidden, s);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
 }
 
 }  // extern "C"

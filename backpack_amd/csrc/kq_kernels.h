@@ -55,6 +55,17 @@ size_t mrow_scratch_floats(const MatmulArgs& a, const GemvTuning& t);
 hipError_t launch_mrow(const MatmulArgs& a, const SplitScratch& sc, const GemvTuning& t, const uint32_t* tiles,
                        const uint32_t* n_tiles, uint32_t tiles_bound, int sets, hipStream_t s);
 
+// MoE: bucket (token, slot) pairs by expert into tiles of 2*sets pairs, the
+// activation between gate/up and down, and the weighted combine.
+int moe_sets_for(uint32_t n_pairs, uint32_t n_experts);
+uint32_t moe_tiles_bound(uint32_t n_pairs, uint32_t n_experts, int sets);
+size_t moe_tiles_words(uint32_t n_pairs, uint32_t n_experts, int sets);
+hipError_t launch_moe_group(const uint32_t* expert_idx, uint32_t n_pairs, uint32_t n_experts, int sets, uint32_t* tiles,
+                            uint32_t* n_tiles, hipStream_t s);
+hipError_t launch_moe_silu_mul(const float* gate, const float* up, float* act, size_t n, hipStream_t s);
+hipError_t launch_moe_combine(const float* down, const float* wt, float* out, uint32_t T, uint32_t k, uint32_t hidden,
+                              hipStream_t s);
+
 // Prefill GEMM on the matrix cores: X bf16 [M,K], Y f32.  tile = 0 (automatic),
 // 128 or 256 (square workgroup tile).
 bool gemm_bf16_supported(const MatmulArgs& a);

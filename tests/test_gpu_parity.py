@@ -282,3 +282,90 @@ def test_gemm_bf16_vs_oracle(gpu, kqo, type_, M, N, K, tile):
     exact = Xw.astype(np.float64) @ wbf.astype(np.float64).T + bias.astype(np.float64)
     assert np.abs(got - exact).max() <= 2e-5 * peak + K * 2.0 ** -24 * rms
     _say(f"    max err/peak {err.max() / peak:.2e}  max err/rms {err.max() / rms:.2e}  frobenius {fro:.2e}")
+
+
+# ---- MoE expert FFN ---------------------------------------------------------------------
+def _routing(rng, T, E, k):
+    eidx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.uint32)
+    logits = rng.standard_normal((T, k)).astype(np.float32)
+    ew = np.exp(logits - logits.max(axis=1, keepdims=True))
+    ew = (ew / ew.sum(axis=1, keepdims=True)).astype(np.float32)
+    return eidx, ew
+
+
+@pytest.mark.parametrize("family", [0, 1])
+@pytest.mark.parametrize("T,E,k,H,I", [(1, 8, 2, 512, 512), (5, 6, 3, 512, 768), (40, 16, 4, 512, 512),
+                                       (3, 4, 2, 512, 256)])
+def test_moe_ffn_vs_oracle(gpu, kqo, family, T, E, k, H, I):
+    from backpack_amd import capi, kquant
+    _say("moe_ffn", T, E, k, H, I, "family", family)
+    _, gp, gw = gpu.make_weight(Q4_K, E * I, H, seed=41)
+    _, up, uw = gpu.make_weight(Q4_K, E * I, H, seed=42)
+    _, dp, dw = gpu.make_weight(Q6_K, E * H, I, seed=43)
+    rng = np.random.default_rng(T + E)
+    eidx, ew = _routing(rng, T, E, k)
+    X = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
+    capi.force_kernel(family)
+    try:
+        got = kquant.moe_ffn(gpu.dev(X), gw, uw, dw, gpu.dev(eidx.view(np.int32)), gpu.dev(ew), E).cpu().numpy()
+        kern = capi.last_kernel()
+    finally:
+        capi.force_kernel(0)
+    # a single-block Q6_K down projection (inter = 256) is outside the row kernel's reach
+    assert kern == ("moe_ffn_generic" if family == 1 or I == 256 else "moe_ffn_mrow")
+    want = kqo.moe_ffn(Q4_K, Q6_K, X, gp, up, dp, eidx, ew, H, I)
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    err = np.abs(got - want)
+    # three chained fp32 matvecs and an exp(): 1e-3 relative, floor 1e-3 of the output rms
+    assert np.all(err <= 1e-3 * rms + 1e-3 * np.abs(want)), f"max err {err.max():.3g} rms {rms:.3g}"
+
+
+def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
+    """Qwen3-30B-A3B-shaped experts (128 x [768x2048 Q4_K gate/up, 2048x768 Q6_K down]),
+    top-8 routing: T=1 against the oracle, T=256 grouped path against the ungrouped
+    one on the GPU plus an oracle spot check of four tokens."""
+    import torch
+    from backpack_amd import capi, kquant, synth
+    E, k, H, I = 128, 8, 2048, 768
+    mk = lambda t, N, K, seed: kquant.KQuantPacked(synth.make_packed_device(t, N, K, seed=seed), t, N, K,
+                                                   synth.row_stride_words(t, K), synth.n_blocks(K))
+    gw, uw, dw = mk(Q4_K, E * I, H, 51), mk(Q4_K, E * I, H, 52), mk(Q6_K, E * H, I, 53)
+    host = lambda w: w.data[: w.N * w.row_stride_bytes].cpu().numpy().view(np.uint32)
+    gp, up, dp = host(gw), host(uw), host(dw)
+    rng = np.random.default_rng(5)
+    for T in (1, 256):
+        _say("moe qwen3 T", T)
+        eidx, ew = _routing(rng, T, E, k)
+        X = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
+        xd, ed, wd = gpu.dev(X), gpu.dev(eidx.view(np.int32)), gpu.dev(ew)
+        got = kquant.moe_ffn(xd, gw, uw, dw, ed, wd, E).cpu().numpy()
+        assert capi.last_kernel() == "moe_ffn_mrow"
+        sel = np.arange(T) if T == 1 else np.array([0, 100, 101, 255])
+        want = kqo.moe_ffn(Q4_K, Q6_K, X[sel], gp, up, dp, eidx[sel], ew[sel], H, I)
+        rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+        assert np.all(np.abs(got[sel] - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
+        if T > 1:
+            capi.force_kernel(1)
+            try:
+                ref = kquant.moe_ffn(xd, gw, uw, dw, ed, wd, E).cpu().numpy()
+            finally:
+                capi.force_kernel(0)
+            assert np.all(np.abs(got - ref) <= 1e-3 * rms + 1e-3 * np.abs(ref))
+            again = kquant.moe_ffn(xd, gw, uw, dw, ed, wd, E).cpu().numpy()
+            assert np.array_equal(got, again), "grouped path must not depend on bucket fill order"
+
+
+@pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True)])
+def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot):
+    """Ragged lists: some experts get many pairs, some none; repeated experts inside a token."""
+    from backpack_amd import capi, kquant
+    E, T, k = 12, 37, 4
+    raw, packed, w = gpu.make_weight(type_, E * N, K, seed=61)
+    rng = np.random.default_rng(62)
+    eidx = rng.choice([0, 1, 1, 1, 5, 5, 7, 11], size=(T, k)).astype(np.uint32)   # experts 2,3,4,6,8,9,10 idle
+    X = rng.standard_normal((T * k if per_slot else T, K)).astype(np.float32)
+    got = kquant.moe_matmul(gpu.dev(X), w, gpu.dev(eidx.view(np.int32)), E, x_per_slot=per_slot).cpu().numpy()
+    assert capi.last_kernel() == "mrow_grouped"
+    want = kqo.moe_matmul(type_, X, packed, eidx, N, K, x_per_slot=per_slot)
+    rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    assert np.all(np.abs(got - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
