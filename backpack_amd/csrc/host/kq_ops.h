@@ -1,0 +1,74 @@
+// kq_ops.h — C++ host layer over the C ABI, shaped like the reference's k-quant
+// operator interface so that a ModelRunner-style caller can switch to it:
+//
+//   KQuantPacked, pack_q4k, pack_q6k     runtime/gguf_loader.h:108-124
+//   GPUBuffer {handle, size, offset}     runtime/gpu_context.h:47-51 (non-owning view)
+//   uploadKQWeight, fuseKQ               runtime/model_runner.cpp:958-963, :1002-1012
+//   makeKQParams  P = {K,N,nBlocks,rowStrideWords,yOffset}   runtime/model_runner.cpp:2404-2413
+//   Dispatch {pipeline, bindGroup, gx,gy,gz, name}           runtime/gpu_context.h:36-44
+//
+// A KQDispatch is the counterpart of one recorded dispatch: the binding set
+// {0:X 1:W 2:Bias 3:Y 4:P} plus M, replayed with run(stream).  Kernel choice
+// (the reference's kqPipelineFor / mmk) happens inside the library.  Errors
+// follow the reference's convention: a message on stderr and an early return;
+// run() additionally returns the library's status code.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "../../../include/bpk_kquant.h"
+
+namespace bp {
+
+enum GGUFType : uint32_t { GGUF_TYPE_Q4_K = BPK_TYPE_Q4_K, GGUF_TYPE_Q6_K = BPK_TYPE_Q6_K };
+
+struct KQuantPacked {
+    std::vector<uint32_t> data;   // raw block data as u32 words, rows padded to 4 bytes
+    uint32_t N = 0, K = 0;        // output rows, input columns
+    uint32_t rowStrideWords = 0;
+    uint32_t nBlocks = 0;
+    GGUFType type = GGUF_TYPE_Q4_K;
+};
+
+KQuantPacked pack_q4k(const void* raw_data, uint32_t N, uint32_t K);
+KQuantPacked pack_q6k(const void* raw_data, uint32_t N, uint32_t K);
+
+// Row-wise concatenation of packed matrices with equal K and type (q|k|v, gate|up).
+KQuantPacked fuseKQ(const std::vector<const KQuantPacked*>& parts);
+
+struct GPUBuffer {
+    void* handle = nullptr;   // device allocation
+    size_t size = 0;
+    size_t offset = 0;        // bind offset in bytes
+    void* ptr() const { return handle ? (char*)handle + offset : nullptr; }
+};
+
+GPUBuffer createBuffer(const std::string& name, size_t bytes);
+void writeBuffer(const GPUBuffer& b, const void* src, size_t bytes);
+void readBuffer(const GPUBuffer& b, void* dst, size_t bytes);   // synchronises the device
+void releaseBuffer(GPUBuffer& b);
+
+GPUBuffer uploadKQWeight(const std::string& name, const KQuantPacked& w);
+
+struct KQParams { uint32_t v[5]; };
+inline KQParams makeKQParams(uint32_t K, uint32_t N, uint32_t nBlocks, uint32_t rowStride, uint32_t yOffset = 0)
+{
+    return KQParams{{K, N, nBlocks, rowStride, yOffset}};
+}
+
+struct KQDispatch {
+    GGUFType type;
+    GPUBuffer X, W, Bias, Y;   // Bias.handle == nullptr binds zeros
+    KQParams P;
+    uint32_t M = 1;
+    std::string name;
+    int run(void* stream = nullptr) const;
+};
+
+// Dequantised rows (the q6k_gather / q6k_gather_batched dispatch).
+int gatherKQ(GGUFType type, const GPUBuffer& W, uint32_t rowStrideWords, const GPUBuffer& tokens, uint32_t M,
+             uint32_t K, const GPUBuffer& out, void* stream = nullptr);
+
+}  // namespace bp

@@ -1,0 +1,187 @@
+// The reference's nine Q4_K / Q6_K kernel tests (runtime/tests/kernel_test.cpp:1678-1748)
+// re-stated against the C++ host layer: same names, same closed-form inputs, same
+// tolerances.  Expected values come from the CPU oracle (test infrastructure),
+// which plays the part of dequant_kquant + the sequential fp32 dot.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "../../backpack_amd/csrc/host/kq_ops.h"
+#include "../../oracle/kq_oracle.h"
+
+using namespace bp;
+
+struct CheckResult { bool ok; std::string msg; };
+struct TestEntry { const char* name; std::function<CheckResult()> fn; };
+static std::vector<TestEntry>& registry() { static std::vector<TestEntry> r; return r; }
+#define TEST(name) \
+    static CheckResult test_##name(); \
+    static struct Reg_##name { Reg_##name() { registry().push_back({#name, test_##name}); } } reg_##name; \
+    static CheckResult test_##name()
+
+static std::vector<float> randnVec(uint32_t seed, int n)
+{
+    kqo_rng r; kqo_rng_seed(&r, seed);
+    std::vector<float> v(n); kqo_rng_randn_vec(&r, v.data(), n); return v;
+}
+static uint16_t f32ToF16(float f) { return kqo_f32_to_f16_trunc(f); }
+
+static CheckResult assertClose(const float* a, const float* e, int n, float atol, float rtol)
+{
+    float worst = 0;
+    int bad = kqo_assert_close(a, e, n, atol, rtol, &worst);
+    if (!bad) return {true, ""};
+    char buf[128]; snprintf(buf, sizeof buf, "%d elements outside tolerance, worst excess %g", bad, worst);
+    return {false, buf};
+}
+
+// raw blocks -> pack -> upload -> dispatch -> readback, expected = oracle
+static CheckResult runMatmul(GGUFType type, const std::vector<uint8_t>& raw, int M, int N, int K,
+                             const std::vector<float>& x, const std::vector<float>& bias, bool biasFirst)
+{
+    KQuantPacked pk = type == GGUF_TYPE_Q4_K ? pack_q4k(raw.data(), N, K) : pack_q6k(raw.data(), N, K);
+    std::vector<float> expected(M * N);
+    kqo_matmul((int)type, x.data(), pk.data.data(), biasFirst ? bias.data() : nullptr, expected.data(), M, N, K,
+               pk.rowStrideWords, 0, 0);
+    GPUBuffer bx = createBuffer("X", x.size() * 4), bw = uploadKQWeight("W", pk), bb = createBuffer("B", N * 4),
+              by = createBuffer("Y", (size_t)M * N * 4);
+    writeBuffer(bx, x.data(), x.size() * 4);
+    writeBuffer(bb, bias.data(), N * 4);
+    KQDispatch d{type, bx, bw, bb, by, makeKQParams(K, N, pk.nBlocks, pk.rowStrideWords, 0), (uint32_t)M, "kq"};
+    if (d.run() != BPK_OK) return {false, bpk_last_error()};
+    std::vector<float> got(M * N);
+    readBuffer(by, got.data(), got.size() * 4);
+    releaseBuffer(bx); releaseBuffer(bw); releaseBuffer(bb); releaseBuffer(by);
+    return assertClose(got.data(), expected.data(), M * N, 2e-4f, 2e-4f);
+}
+
+static std::vector<uint8_t> q4kRaw(int N, int NB, std::function<float(int, int)> d, std::function<float(int, int)> dm,
+                                   std::function<int(int, int, int)> byte)
+{
+    std::vector<uint8_t> raw((size_t)N * NB * 144);
+    for (int n = 0; n < N; n++) for (int b = 0; b < NB; b++) {
+        uint8_t* p = raw.data() + ((size_t)n * NB + b) * 144;
+        uint16_t hd = f32ToF16(d(n, b)), hm = f32ToF16(dm(n, b));
+        memcpy(p, &hd, 2); memcpy(p + 2, &hm, 2);
+        for (int i = 4; i < 144; i++) p[i] = (uint8_t)byte(n, b, i);
+    }
+    return raw;
+}
+static std::vector<uint8_t> q6kRaw(int N, int NB, std::function<float(int, int)> d, std::function<int(int, int, int)> byte)
+{
+    std::vector<uint8_t> raw((size_t)N * NB * 210);
+    for (int n = 0; n < N; n++) for (int b = 0; b < NB; b++) {
+        uint8_t* p = raw.data() + ((size_t)n * NB + b) * 210;
+        for (int i = 0; i < 208; i++) p[i] = (uint8_t)byte(n, b, i);
+        uint16_t hd = f32ToF16(d(n, b)); memcpy(p + 208, &hd, 2);
+    }
+    return raw;
+}
+static std::vector<float> biasVec(int N, bool on) { std::vector<float> b(N, 0.f); if (on) for (int n = 0; n < N; n++) b[n] = .01f * n; return b; }
+
+TEST(q4k_matmul_reference) {
+    const int N = 8, K = 256;
+    auto raw = q4kRaw(N, 1, [](int n, int) { return .02f + .001f * n; }, [](int n, int) { return .01f + .0005f * n; },
+                      [](int n, int, int i) { return (n * 31 + i * 17 + 3) & 255; });
+    return runMatmul(GGUF_TYPE_Q4_K, raw, 1, N, K, randnVec(4343, K), biasVec(N, false), false);
+}
+TEST(q4k_matmul_128_reference) {
+    const int N = 7, K = 512;
+    auto raw = q4kRaw(N, 2, [](int n, int) { return .02f + .001f * n; }, [](int, int b) { return .01f + .0002f * b; },
+                      [](int n, int b, int j) { return n * 31 + b * 13 + j * 17; });
+    return runMatmul(GGUF_TYPE_Q4_K, raw, 1, N, K, randnVec(5555, K), biasVec(N, true), true);
+}
+TEST(q6k_matmul_reference) {
+    const int N = 8, K = 768;
+    auto raw = q6kRaw(N, 3, [](int n, int q) { return .02f + .001f * n + .0003f * q; },
+                      [](int n, int q, int i) { return (n * 29 + q * 23 + i * 19 + 5) & 255; });
+    return runMatmul(GGUF_TYPE_Q6_K, raw, 1, N, K, randnVec(4646, K), biasVec(N, false), false);
+}
+TEST(q6k_matmul_wide_reference) {
+    const int N = 19, K = 768;
+    auto raw = q6kRaw(N, 3, [](int n, int b) { return .018f + .0007f * n + .0002f * b; },
+                      [](int n, int b, int i) { return (n * 37 + b * 17 + i * 13 + 11) & 255; });
+    return runMatmul(GGUF_TYPE_Q6_K, raw, 1, N, K, randnVec(4747, K), biasVec(N, true), true);
+}
+TEST(q4k_matmul_batched4_reference) {
+    const int M = 5, N = 9, K = 512;
+    auto raw = q4kRaw(N, 2, [](int n, int) { return .02f + .001f * n; }, [](int, int b) { return .01f + .0002f * b; },
+                      [](int n, int b, int i) { return n * 31 + b * 13 + i * 17; });
+    return runMatmul(GGUF_TYPE_Q4_K, raw, M, N, K, randnVec(4848, M * K), biasVec(N, true), true);
+}
+TEST(q6k_matmul_batched4_reference) {
+    const int M = 5, N = 9, K = 768;
+    auto raw = q6kRaw(N, 3, [](int n, int b) { return .018f + .0007f * n + .0002f * b; },
+                      [](int n, int b, int i) { return n * 23 + b * 17 + i * 13; });
+    return runMatmul(GGUF_TYPE_Q6_K, raw, M, N, K, randnVec(5050, M * K), biasVec(N, true), true);
+}
+TEST(q4k_matmul_batched8_reference) {
+    const int M = 9, N = 9, K = 512;
+    auto raw = q4kRaw(N, 2, [](int n, int) { return .02f + .001f * n; }, [](int, int b) { return .01f + .0002f * b; },
+                      [](int n, int b, int i) { return n * 31 + b * 13 + i * 17; });
+    return runMatmul(GGUF_TYPE_Q4_K, raw, M, N, K, randnVec(5151, M * K), biasVec(N, true), true);
+}
+
+static CheckResult runGather(const std::vector<uint8_t>& raw, int N, int K, const std::vector<int32_t>& toks)
+{
+    KQuantPacked pk = pack_q6k(raw.data(), N, K);
+    const int M = (int)toks.size();
+    std::vector<float> expected((size_t)M * K), got((size_t)M * K);
+    kqo_dequant_rows(KQO_TYPE_Q6_K, pk.data.data(), pk.rowStrideWords, toks.data(), M, K, expected.data());
+    GPUBuffer bw = uploadKQWeight("W", pk), bt = createBuffer("T", M * 4), bx = createBuffer("X", got.size() * 4);
+    writeBuffer(bt, toks.data(), M * 4);
+    if (gatherKQ(GGUF_TYPE_Q6_K, bw, pk.rowStrideWords, bt, M, K, bx) != BPK_OK) return {false, bpk_last_error()};
+    readBuffer(bx, got.data(), got.size() * 4);
+    releaseBuffer(bw); releaseBuffer(bt); releaseBuffer(bx);
+    return assertClose(got.data(), expected.data(), M * K, 1e-6f, 1e-6f);
+}
+TEST(q6k_gather_reference) {
+    auto raw = q6kRaw(3, 3, [](int n, int b) { return .015f + .001f * n + .0002f * b; },
+                      [](int n, int b, int i) { return (n * 41 + b * 23 + i * 11 + 9) & 255; });
+    return runGather(raw, 3, 768, {2});
+}
+TEST(q6k_gather_batched_reference) {
+    auto raw = q6kRaw(4, 3, [](int n, int) { return .014f + .001f * n; }, [](int n, int b, int i) { return n * 43 + b * 19 + i * 7 + 3; });
+    return runGather(raw, 4, 768, {3, 0, 2});
+}
+TEST(fuse_qkv_rows) {
+    // q|k|v fused upload: the fused matvec equals the three separate ones
+    const int K = 512, Nq = 9, Nk = 3;
+    auto mk = [&](int N, int salt) {
+        return q4kRaw(N, 2, [](int n, int) { return .02f + .001f * n; }, [](int, int b) { return .01f + .0002f * b; },
+                      [salt](int n, int b, int i) { return n * 31 + b * 13 + i * 17 + salt; });
+    };
+    auto rq = mk(Nq, 1), rk = mk(Nk, 2), rv = mk(Nk, 3);
+    KQuantPacked q = pack_q4k(rq.data(), Nq, K), k = pack_q4k(rk.data(), Nk, K), v = pack_q4k(rv.data(), Nk, K);
+    KQuantPacked f = fuseKQ({&q, &k, &v});
+    if (f.N != (uint32_t)(Nq + 2 * Nk)) return {false, "fused row count"};
+    auto x = randnVec(77, K);
+    std::vector<float> expected(f.N), got(f.N), zero(f.N, 0.f);
+    kqo_matmul(KQO_TYPE_Q4_K, x.data(), q.data.data(), nullptr, expected.data(), 1, Nq, K, q.rowStrideWords, 0, 0);
+    kqo_matmul(KQO_TYPE_Q4_K, x.data(), k.data.data(), nullptr, expected.data() + Nq, 1, Nk, K, k.rowStrideWords, 0, 0);
+    kqo_matmul(KQO_TYPE_Q4_K, x.data(), v.data.data(), nullptr, expected.data() + Nq + Nk, 1, Nk, K, v.rowStrideWords, 0, 0);
+    GPUBuffer bx = createBuffer("X", K * 4), bw = uploadKQWeight("qkv", f), by = createBuffer("Y", f.N * 4);
+    writeBuffer(bx, x.data(), K * 4);
+    KQDispatch d{GGUF_TYPE_Q4_K, bx, bw, GPUBuffer{}, by, makeKQParams(K, f.N, f.nBlocks, f.rowStrideWords), 1, "qkv"};
+    if (d.run() != BPK_OK) return {false, bpk_last_error()};
+    readBuffer(by, got.data(), f.N * 4);
+    releaseBuffer(bx); releaseBuffer(bw); releaseBuffer(by);
+    return assertClose(got.data(), expected.data(), f.N, 2e-4f, 2e-4f);
+}
+
+int main()
+{
+    if (bpk_init(0) != BPK_OK) { fprintf(stderr, "bpk_init: %s\n", bpk_last_error()); return 2; }
+    int failed = 0;
+    for (auto& t : registry()) {
+        CheckResult r = t.fn();
+        printf("%-36s %s %s\n", t.name, r.ok ? "PASS" : "FAIL", r.msg.c_str());
+        fflush(stdout);
+        failed += !r.ok;
+    }
+    printf("%zu tests, %d failed\n", registry().size(), failed);
+    return failed ? 1 : 0;
+}
