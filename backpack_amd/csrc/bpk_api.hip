@@ -282,12 +282,16 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     if (t_family == 2 && !rows_ok) return fail(BPK_ERR_SHAPE, "row-per-lane GEMV cannot serve this call");
     if (t_family == 3 && !mrow_ok) return fail(BPK_ERR_SHAPE, "matrix-core row kernel cannot serve this call");
     if (t_family > 3) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
-    if ((t_family == 0 || t_family == 3) && mrow_ok) {
-        t_kernel = "mrow";
-        e = kq::launch_mrow(a, st->split, t_gemv, nullptr, nullptr, 1, 0, s);
-    } else if ((t_family == 0 || t_family == 2) && rows_ok) {
+    // automatic choice: M <= 2 on the VALU row kernel (the 4x4x4 MFMA does not
+    // overlap with VALU work on this part), M = 3..16 on the matrix-core row kernel
+    const bool use_rows = rows_ok && (t_family == 2 || (t_family == 0 && (M <= 2 || !mrow_ok)));
+    const bool use_mrow = mrow_ok && !use_rows && (t_family == 0 || t_family == 3);
+    if (use_rows) {
         t_kernel = "gemv_rows";
         e = kq::launch_gemv_rows(a, st->split, t_gemv, s);
+    } else if (use_mrow) {
+        t_kernel = "mrow";
+        e = kq::launch_mrow(a, st->split, t_gemv, nullptr, nullptr, 1, 0, s);
     } else {
         t_kernel = "generic";
         e = kq::launch_matmul_generic(a, s);
