@@ -25,7 +25,8 @@ FLAGS = [
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
+    extra = os.environ.get("BPK_EXTRA_FLAGS", "").split()   # experiments only, e.g. -DKQ_PLAIN_LOADS
+    cmd = [HIPCC, *FLAGS, *extra, "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode:

@@ -44,6 +44,12 @@ __device__ __forceinline__ void wave_lds_fence()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+#ifdef KQ_NT_LOADS
+#define KQ_WLOAD(ptr) __builtin_nontemporal_load(ptr)
+#else
+#define KQ_WLOAD(ptr) (*(ptr))
+#endif
+
 constexpr float TWO24 = 16777216.0f;
 constexpr float TWO20 = 1048576.0f;
 
@@ -205,38 +211,103 @@ __device__ __forceinline__ void q4k_block_dot(const u32x4& hdr, const u32x4 (&q)
     }
 }
 
-// Q6_K block: 53 words, delivered through `word(j)`.
-template <int MT, typename WordFn>
-__device__ __forceinline__ void q6k_block_dot(WordFn word, const float* __restrict__ X, uint32_t K, uint32_t M,
-                                              uint32_t k0, const float* xsum, uint32_t xsum_stride, float (&acc)[MT])
+template <int MT, int NW>
+__global__ __launch_bounds__(64 * NW) void q4k_gemv_kernel(GemvParams p)
 {
-    const float d = half_bits_to_float(word(52) & 0xFFFFu);
-    uint32_t scw[4];
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int TILE = 64 * KQ_Q4K_BYTES;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t row0 = blockIdx.x * 64u;
+    const uint32_t b_begin = blockIdx.y * p.blocks_per_split;
+    const uint32_t b_end = min(p.n_blocks, b_begin + p.blocks_per_split);
+    const uint32_t nblk = b_end - b_begin;
+
+    u32x4* tile = (u32x4*)(smem + wave * TILE);   // 576 pieces of 16 B
+    float* xs = (float*)(smem + NW * TILE);         // [MT][nblk][8]
+    float* red = (float*)smem;                      // reused at the end
+
+    stage_x_sums<MT, 32, 64 * NW>(p.X, p.K, p.M, b_begin, nblk, xs);
+
+    // piece i*64+lane of the wave's 64x144-byte tile: row r, 16-byte segment s
+    uint32_t goff[9];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) scw[i] = word(48 + i);
-    float tot[MT];
+    for (int i = 0; i < 9; ++i) {
+        const uint32_t pc = i * 64u + lane;
+        const uint32_t r = pc / 9u, s = pc - r * 9u;
+        const uint32_t row = min(row0 + r, p.N - 1u);
+        goff[i] = (row - row0) * p.row_stride_bytes + s * 16u;
+    }
+    const uint8_t* wbase = p.W + (size_t)row0 * p.row_stride_bytes;
+
+    float acc[MT];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) tot[m] = 0.0f;
+    for (int m = 0; m < MT; ++m) acc[m] = 0.0f;
+
+    u32x4 v[9];
+    uint32_t b = b_begin + wave;
+    if (b < b_end) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        uint32_t ql[16], qh[8];
+        for (int i = 0; i < 9; ++i)
+            v[i] = KQ_WLOAD((const u32x4*)(wbase + goff[i] + (size_t)b * KQ_Q4K_BYTES));
+    }
+    __syncthreads();  // xs ready
+
+    for (; b < b_end; b += NW) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) ql[i] = word(16 * h + i);
+        for (int i = 0; i < 9; ++i) tile[i * 64 + lane] = v[i];
+        const uint32_t bn = b + NW;
+        if (bn < b_end) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) qh[i] = word(32 + 8 * h + i);
+            for (int i = 0; i < 9; ++i)
+                v[i] = KQ_WLOAD((const u32x4*)(wbase + goff[i] + (size_t)bn * KQ_Q4K_BYTES));
+        }
+        wave_lds_fence();
+        const u32x4 hdr = tile[lane * 9];
+        u32x4 q[8];
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const float* __restrict__ x = X + (size_t)(m < (int)M ? m : 0) * K + k0 + 128 * h;
+        for (int s = 0; s < 8; ++s) q[s] = tile[lane * 9 + 1 + s];
+        wave_lds_fence();
+        q4k_block_dot<MT>(hdr, q, p.X, p.K, p.M, b * KQ_QK, xs + (size_t)(b - b_begin) * 8, nblk * 8, acc);
+    }
+    finish_rows<MT, NW>(p, acc, red, row0, lane, wave);
+}
+
+// ---------------------------------------------------------------------------
+// Q6_K: 210-byte blocks.  The wave copies a 224-byte window per row (14 pieces)
+// that starts at the block for even b and 14 bytes before it for odd b, so the
+// window always begins 4-byte aligned and never leaves the row; in LDS rows
+// are 240 bytes apart (odd multiple of 16: conflict-free 128-bit reads).
+// Odd blocks sit 2 bytes off a word boundary and are realigned with one
+// v_alignbit per word.
+// ---------------------------------------------------------------------------
+constexpr int Q6_WIN_PIECES = 14;
+constexpr int Q6_LDS_ROW = 240;
+
+// 32 x 16 elements of one (half, 16-lane quarter) chunk: words A (ql[l]),
+// B (ql[l+32]), H (qh[l]) for l = 16*uq .. 16*uq+15, four words each.
+template <int MT>
+__device__ __forceinline__ void q6k_block_dot(const uint32_t (&w)[53], const float* __restrict__ X, uint32_t K,
+                                              uint32_t M, uint32_t k0, const float* xsum, uint32_t xsum_stride,
+                                              float (&acc)[MT])
+{
+    const float d = half_bits_to_float(w[52] & 0xFFFFu);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const float* __restrict__ x = X + (size_t)(m < (int)M ? m : 0) * K + k0;
+        float tot = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
 #pragma unroll
             for (int uq = 0; uq < 2; ++uq) {
                 float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int uu = 0; uu < 4; ++uu) {
                     const int u = uq * 4 + uu;
-                    const uint32_t A = ql[u], B = ql[8 + u], H = qh[u];
+                    const uint32_t A = w[16 * h + u], B = w[16 * h + 8 + u], H = w[32 + 8 * h + u];
                     const uint32_t A8 = A >> 8, B8 = B >> 8;
                     const uint32_t Hl4 = H << 4, Hl2 = H << 2, Hr4 = H >> 4, Hr6 = H >> 6;
-                    // [t][pair]: pair a holds l, l+2; pair b holds l+1, l+3
+                    // [t][pair]: pair 0 holds l, l+2; pair 1 holds l+1, l+3
                     const half2_t q0a = as_half2((A & 0x000F000Fu) | (Hl4 & 0x00300030u));
                     const half2_t q2a = as_half2((A & 0x00F000F0u) | (Hl4 & 0x03000300u));
                     const half2_t q1a = as_half2((B & 0x000F000Fu) | (Hl2 & 0x00300030u));
@@ -245,7 +316,7 @@ __device__ __forceinline__ void q6k_block_dot(WordFn word, const float* __restri
                     const half2_t q2b = as_half2((A8 & 0x00F000F0u) | (Hr4 & 0x03000300u));
                     const half2_t q1b = as_half2((B8 & 0x000F000Fu) | (Hr6 & 0x00300030u));
                     const half2_t q3b = as_half2((B8 & 0x00F000F0u) | (Hr6 & 0x03000300u));
-                    const float* xl = x + 4 * u;
+                    const float* xl = x + 128 * h + 4 * u;
                     a[0] = fma_h(q0a.x, xl[0], a[0]);
                     a[0] = fma_h(q0b.x, xl[1], a[0]);
                     a[0] = fma_h(q0a.y, xl[2], a[0]);
@@ -266,47 +337,21 @@ __device__ __forceinline__ void q6k_block_dot(WordFn word, const float* __restri
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const int j = 8 * h + 2 * t + uq;   // scale / 16-element group index
-                    const float sc = (float)(int)(int8_t)((scw[j >> 2] >> (8 * (j & 3))) & 255u);
+                    const float sc = (float)(int)(int8_t)((w[48 + (j >> 2)] >> (8 * (j & 3))) & 255u);
                     const float s = fmaf(a[t], t < 2 ? TWO24 : TWO20, -32.0f * xsum[m * xsum_stride + j]);
-                    tot[m] = fmaf(sc, s, tot[m]);
+                    tot = fmaf(sc, s, tot);
                 }
             }
         }
+        acc[m] = fmaf(d, tot, acc[m]);
     }
-#pragma unroll
-    for (int m = 0; m < MT; ++m) acc[m] = fmaf(d, tot[m], acc[m]);
 }
 
-// ---------------------------------------------------------------------------
-// The kernel.  Q4_K: 144-byte blocks = 9 pieces of 16 bytes, the LDS tile is a
-// byte copy of 64 blocks.  Q6_K: 210-byte blocks; the wave copies a 224-byte
-// window per row (14 pieces) that starts at the block (even b), 14 bytes before
-// it (odd b) or 12 bytes before it (an even block that closes a row of an odd
-// number of blocks), so the window is always 4-byte aligned and never leaves the
-// row; LDS rows are 240 bytes apart (an odd number of 16-byte slots).  A block
-// then starts `base` words into its LDS row, `sh` bits into that word, and
-// every word is recovered with one v_alignbit (sh = 0 returns the word as is).
-//
-// Each wave keeps the pieces of up to DEPTH of its superblocks in registers and
-// issues those loads before anything else, so that for the usual case (a wave
-// owns <= DEPTH blocks) every HBM request of the launch is in flight within the
-// first microsecond; the ring is refilled as blocks are consumed.
-// ---------------------------------------------------------------------------
-constexpr int Q6_WIN_PIECES = 14;
-constexpr int Q6_LDS_ROW = 240;
-
-template <int TYPE, int MT, int NW, int DEPTH>
-__global__ __launch_bounds__(64 * NW) void gemv_rows_kernel(GemvParams p)
+template <int MT, int NW>
+__global__ __launch_bounds__(64 * NW) void q6k_gemv_kernel(GemvParams p)
 {
     extern __shared__ __align__(16) uint8_t smem[];
-    constexpr bool Q4 = TYPE == KQ_TYPE_Q4_K;
-    constexpr int BB = Q4 ? KQ_Q4K_BYTES : KQ_Q6K_BYTES;
-    constexpr int NPIECE = Q4 ? 9 : Q6_WIN_PIECES;
-    constexpr int LROW = Q4 ? KQ_Q4K_BYTES : Q6_LDS_ROW;
-    constexpr int SEG = Q4 ? 32 : 16;
-    constexpr int NSEG = 256 / SEG;
-    constexpr int TILE = 64 * LROW;
-
+    constexpr int TILE = 64 * Q6_LDS_ROW;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t row0 = blockIdx.x * 64u;
@@ -315,84 +360,70 @@ __global__ __launch_bounds__(64 * NW) void gemv_rows_kernel(GemvParams p)
     const uint32_t nblk = b_end - b_begin;
 
     uint8_t* tile = smem + wave * TILE;
-    float* xs = (float*)(smem + NW * TILE);   // [MT][nblk][NSEG]
-    float* red = (float*)smem;                // reused at the end
+    float* xs = (float*)(smem + NW * TILE);   // [MT][nblk][16]
+    float* red = (float*)smem;
 
-    // ---- piece i*64+lane of the tile: row r, 16-byte segment s (64 = 7*9+1 = 4*14+8)
-    uint32_t goff[NPIECE], loff[NPIECE];
-    {
-        uint32_t r = lane / NPIECE, sg = lane - r * NPIECE;
+    stage_x_sums<MT, 16, 64 * NW>(p.X, p.K, p.M, b_begin, nblk, xs);
+
+    // piece i*64+lane of the 64x224-byte window: row r, segment s
+    uint32_t goff[Q6_WIN_PIECES], loff[Q6_WIN_PIECES];
 #pragma unroll
-        for (int i = 0; i < NPIECE; ++i) {
-            const uint32_t row = min(row0 + r, p.N - 1u);
-            goff[i] = (row - row0) * p.row_stride_bytes + sg * 16u;
-            loff[i] = r * LROW + sg * 16u;
-            r += 64 / NPIECE;
-            sg += 64 % NPIECE;
-            if (sg >= (uint32_t)NPIECE) { sg -= NPIECE; r += 1; }
-        }
+    for (int i = 0; i < Q6_WIN_PIECES; ++i) {
+        const uint32_t pc = i * 64u + lane;
+        const uint32_t r = pc / Q6_WIN_PIECES, s = pc - r * Q6_WIN_PIECES;
+        const uint32_t row = min(row0 + r, p.N - 1u);
+        goff[i] = (row - row0) * p.row_stride_bytes + s * 16u;
+        loff[i] = r * Q6_LDS_ROW + s * 16u;
     }
     const uint8_t* wbase = p.W + (size_t)row0 * p.row_stride_bytes;
-    const uint32_t last_even = (p.n_blocks & 1u) ? p.n_blocks - 1u : 0xFFFFFFFFu;
-    auto back = [&](uint32_t b) -> uint32_t {   // bytes the Q6_K window starts before the block
-        return Q4 ? 0u : (b & 1u) ? 14u : (b == last_even ? 12u : 0u);
-    };
-
-    // ---- all of this wave's first DEPTH blocks go in flight now
-    u32x4 v[DEPTH][NPIECE];
-#pragma unroll
-    for (int dpt = 0; dpt < DEPTH; ++dpt) {
-        const uint32_t b = b_begin + wave + dpt * NW;
-        if (b < b_end) {
-            const size_t o = (size_t)b * BB - back(b);
-#pragma unroll
-            for (int i = 0; i < NPIECE; ++i)
-                v[dpt][i] = __builtin_nontemporal_load((const u32x4*)(wbase + goff[i] + o));
-        }
-    }
-
-    stage_x_sums<MT, SEG, 64 * NW>(p.X, p.K, p.M, b_begin, nblk, xs);
 
     float acc[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[m] = 0.0f;
+
+    // window start of block b relative to the row: 210*b for even b, 210*b - 14 for odd b
+    auto win = [](uint32_t b) { return (size_t)b * KQ_Q6K_BYTES - ((b & 1u) ? 14u : 0u); };
+
+    u32x4 v[Q6_WIN_PIECES];
+    uint32_t b = b_begin + wave;
+    if (b < b_end) {
+#pragma unroll
+        for (int i = 0; i < Q6_WIN_PIECES; ++i)
+            v[i] = KQ_WLOAD((const u32x4*)(wbase + goff[i] + win(b)));
+    }
     __syncthreads();  // xs ready
 
-    uint32_t it = 0;
-    for (uint32_t b = b_begin + wave; b < b_end; b += NW, ++it) {
-        // ---- ring slot it % DEPTH -> LDS, then refill it with block b + DEPTH*NW
-        const uint32_t slot = it % DEPTH;
-        const uint32_t bn = b + DEPTH * NW;
+    for (; b < b_end; b += NW) {
 #pragma unroll
-        for (int dpt = 0; dpt < DEPTH; ++dpt) {
-            if (slot == (uint32_t)dpt) {
+        for (int i = 0; i < Q6_WIN_PIECES; ++i) *(u32x4*)(tile + loff[i]) = v[i];
+        const uint32_t bn = b + NW;
+        if (bn < b_end) {
 #pragma unroll
-                for (int i = 0; i < NPIECE; ++i) *(u32x4*)(tile + loff[i]) = v[dpt][i];
-                if (bn < b_end) {
-                    const size_t o = (size_t)bn * BB - back(bn);
-#pragma unroll
-                    for (int i = 0; i < NPIECE; ++i)
-                        v[dpt][i] = __builtin_nontemporal_load((const u32x4*)(wbase + goff[i] + o));
-                }
-            }
+            for (int i = 0; i < Q6_WIN_PIECES; ++i)
+                v[i] = KQ_WLOAD((const u32x4*)(wbase + goff[i] + win(bn)));
         }
         wave_lds_fence();
-        const uint8_t* mine = tile + lane * LROW;
-        if (Q4) {
-            const u32x4 hdr = *(const u32x4*)mine;
-            u32x4 q[8];
+        u32x4 raw[Q6_WIN_PIECES];
 #pragma unroll
-            for (int sgm = 0; sgm < 8; ++sgm) q[sgm] = *(const u32x4*)(mine + 16 + sgm * 16);
-            wave_lds_fence();
-            q4k_block_dot<MT>(hdr, q, p.X, p.K, p.M, b * KQ_QK, xs + (size_t)(b - b_begin) * NSEG, nblk * NSEG, acc);
+        for (int s = 0; s < Q6_WIN_PIECES; ++s) raw[s] = *(const u32x4*)(tile + lane * Q6_LDS_ROW + s * 16);
+        wave_lds_fence();
+
+        // 53 block words: bytes 0..211 of the block (the last half-word unused)
+        uint32_t w[53];
+        if (b & 1u) {
+            // the block starts at byte 14 of the window: word j = bytes 14+4j .. 17+4j
+#pragma unroll
+            for (int j = 0; j < 53; ++j) {
+                const int lo = 3 + j, hi = 4 + j;
+                const uint32_t wl = raw[lo >> 2][lo & 3];
+                const uint32_t wh = hi < 56 ? raw[hi >> 2][hi & 3] : 0u;
+                w[j] = __builtin_amdgcn_alignbit(wh, wl, 16);
+            }
         } else {
-            const uint32_t bk = back(b);
-            const uint32_t* rw = (const uint32_t*)(mine + (bk & ~3u));   // 0 or 12 bytes in
-            const uint32_t sh = (bk & 2u) * 8u;                            // 0 or 16 bits
-            auto word = [&](int j) -> uint32_t { return __builtin_amdgcn_alignbit(rw[j + 1], rw[j], sh); };
-            q6k_block_dot<MT>(word, p.X, p.K, p.M, b * KQ_QK, xs + (size_t)(b - b_begin) * NSEG, nblk * NSEG, acc);
-            wave_lds_fence();
+#pragma unroll
+            for (int j = 0; j < 53; ++j) w[j] = raw[j >> 2][j & 3];
         }
+        q6k_block_dot<MT>(w, p.X, p.K, p.M, b * KQ_QK, xs + (size_t)(b - b_begin) * 16, nblk * 16, acc);
     }
     finish_rows<MT, NW>(p, acc, red, row0, lane, wave);
 }
@@ -402,7 +433,6 @@ __global__ __launch_bounds__(64 * NW) void gemv_rows_kernel(GemvParams p)
 // ---------------------------------------------------------------------------
 struct GemvPlan {
     int nw;             // waves per workgroup
-    int depth;          // superblocks a wave keeps in flight
     uint32_t bps;       // superblock columns per workgroup
     uint32_t splits;    // workgroups along K
 };
@@ -413,10 +443,9 @@ static GemvPlan plan_gemv(const MatmulArgs& a, const GemvTuning& t)
 {
     GemvPlan pl;
     const uint32_t groups = (a.N + 63u) / 64u;
-    pl.nw = t.waves > 0 ? t.waves : 4;
-    // measured on MI355X: about 450 workgroups of 4 waves is the sweet spot for
-    // every Llama-3-8B shape (more splits pay the cross-workgroup fold, fewer
-    // leave CUs idle)
+    // measured on MI355X: long Q4_K grids like 8 waves sharing a row group,
+    // everything else 4; about 450 workgroups keep 256 CUs fed
+    pl.nw = t.waves > 0 ? t.waves : (a.type == KQ_TYPE_Q4_K && groups >= 256u) ? 8 : 4;
     uint32_t want = t.splits > 0 ? (uint32_t)t.splits : (448u + groups - 1u) / groups;
     const uint32_t max_splits = (a.n_blocks + pl.nw - 1u) / pl.nw;
     if (want > max_splits) want = max_splits;
@@ -425,12 +454,6 @@ static GemvPlan plan_gemv(const MatmulArgs& a, const GemvTuning& t)
     bps = (bps + pl.nw - 1u) / pl.nw * pl.nw;
     pl.bps = bps;
     pl.splits = (a.n_blocks + bps - 1u) / bps;
-    const uint32_t per_wave = bps / pl.nw;
-    const int max_depth = a.type == KQ_TYPE_Q4_K ? 4 : 2;
-    // deeper rings cost registers (occupancy) and measured slower: default 1
-    pl.depth = t.depth > 0 ? t.depth : 1;
-    if (pl.depth > max_depth) pl.depth = max_depth;
-    (void)per_wave;
     return pl;
 }
 
@@ -441,8 +464,9 @@ bool gemv_rows_supported(const MatmulArgs& a)
     if (a.type != KQ_TYPE_Q4_K && a.type != KQ_TYPE_Q6_K) return false;
     if (((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u)) return false;
     if (((uintptr_t)a.X & 15u) || (a.K & 3u)) return false;
-    // Q6_K windows borrow up to 14 bytes from a neighbouring block of the same row
-    if (a.type == KQ_TYPE_Q6_K && a.n_blocks < 2) return false;
+    // Q6_K windows reach 14 bytes into the neighbouring block of the same row:
+    // rows must hold an even number of blocks so that odd blocks end the row
+    if (a.type == KQ_TYPE_Q6_K && (a.n_blocks & 1u)) return false;
     if ((size_t)64 * a.row_stride_bytes > 0x7FFFFFFFull) return false;
     return true;
 }
@@ -456,7 +480,7 @@ size_t gemv_rows_scratch_floats(const MatmulArgs& a, const GemvTuning& t)
     return (size_t)pl.splits * mt_of(a.M) * ((a.N + 63u) / 64u) * 64u;
 }
 
-template <int TYPE, int MT, int NW, int DEPTH>
+template <int TYPE, int MT, int NW>
 static hipError_t launch_one(const GemvParams& p, hipStream_t s)
 {
     const uint32_t groups = (p.N + 63u) / 64u;
@@ -467,7 +491,7 @@ static hipError_t launch_one(const GemvParams& p, hipStream_t s)
     const size_t red = (size_t)NW * MT * 64 * sizeof(float);
     const size_t shmem = tiles + xs > red ? tiles + xs : red;
     if (shmem > 160u * 1024u) return hipErrorInvalidValue;
-    auto kern = gemv_rows_kernel<TYPE, MT, NW, DEPTH>;
+    auto kern = TYPE == KQ_TYPE_Q4_K ? q4k_gemv_kernel<MT, NW> : q6k_gemv_kernel<MT, NW>;
     static size_t raised = 64u * 1024u;   // per instantiation
     if (shmem > raised) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -478,23 +502,13 @@ static hipError_t launch_one(const GemvParams& p, hipStream_t s)
     return hipGetLastError();
 }
 
-template <int TYPE, int MT, int NW>
-static hipError_t launch_depth(const GemvParams& p, int depth, hipStream_t s)
-{
-    if constexpr (TYPE == KQ_TYPE_Q4_K) {
-        if (depth >= 4) return launch_one<TYPE, MT, NW, 4>(p, s);
-    }
-    if (depth >= 2) return launch_one<TYPE, MT, NW, 2>(p, s);
-    return launch_one<TYPE, MT, NW, 1>(p, s);
-}
-
 template <int TYPE, int NW>
-static hipError_t launch_mt(const GemvParams& p, int depth, hipStream_t s)
+static hipError_t launch_mt(const GemvParams& p, hipStream_t s)
 {
     switch (mt_of(p.M)) {
-    case 1: return launch_depth<TYPE, 1, NW>(p, depth, s);
-    case 2: return launch_depth<TYPE, 2, NW>(p, depth, s);
-    default: return launch_depth<TYPE, 4, NW>(p, depth, s);
+    case 1: return launch_one<TYPE, 1, NW>(p, s);
+    case 2: return launch_one<TYPE, 2, NW>(p, s);
+    default: return launch_one<TYPE, 4, NW>(p, s);
     }
 }
 
@@ -522,9 +536,9 @@ hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const G
     }
     const bool q4 = a.type == KQ_TYPE_Q4_K;
     switch (pl.nw) {
-    case 2: return q4 ? launch_mt<KQ_TYPE_Q4_K, 2>(p, pl.depth, s) : launch_mt<KQ_TYPE_Q6_K, 2>(p, pl.depth, s);
-    case 4: return q4 ? launch_mt<KQ_TYPE_Q4_K, 4>(p, pl.depth, s) : launch_mt<KQ_TYPE_Q6_K, 4>(p, pl.depth, s);
-    case 8: return q4 ? launch_mt<KQ_TYPE_Q4_K, 8>(p, pl.depth, s) : launch_mt<KQ_TYPE_Q6_K, 8>(p, pl.depth, s);
+    case 2: return q4 ? launch_mt<KQ_TYPE_Q4_K, 2>(p, s) : launch_mt<KQ_TYPE_Q6_K, 2>(p, s);
+    case 4: return q4 ? launch_mt<KQ_TYPE_Q4_K, 4>(p, s) : launch_mt<KQ_TYPE_Q6_K, 4>(p, s);
+    case 8: return q4 ? launch_mt<KQ_TYPE_Q4_K, 8>(p, s) : launch_mt<KQ_TYPE_Q6_K, 8>(p, s);
     default: return hipErrorInvalidValue;
     }
 }
