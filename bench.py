@@ -32,9 +32,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 METRIC = "Q4_K M=1 matvec HBM GB/s (% of peak); M=2048 dequant-GEMM TFLOPS (% MFMA)"
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE (profiles/q4k_gemv_gate_up_pmc.txt), scaled by a copy kernel of
-# known size; None until measured.
-MEASURED_TRAFFIC_BYTES = None
+# WRITE_SIZE (profiles/q4k_gemv_gate_up_hbm_traffic_pmc.txt): FETCH_SIZE 32601.0
+# x 2.000 KiB + WRITE_SIZE 112.0 x 1.000 KiB, the factors being what the same
+# counters read for a 256 MiB copy kernel.
+MEASURED_TRAFFIC_BYTES = 66881536
 
 
 def parse():
@@ -46,6 +47,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--layers", type=int, default=32, help="layers in the set (32 = the named workload)")
     ap.add_argument("--prefill", action="store_true", help="also time the M=2048 prefill GEMM on one layer")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run one 256 MiB device-to-device copy kernel: under rocprofv3 --pmc its "
+                         "FETCH_SIZE / WRITE_SIZE readings give the counters' scale")
     return ap.parse_args()
 
 
@@ -182,6 +186,14 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     capi.check(capi.lib().bpk_init(0))
 
+    if args.calibrate_copy:
+        src = torch.zeros(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
+
     mats = build_layer_set(args.layers)
     torch.cuda.synchronize()
     wb, act = algorithmic_bytes(mats)
@@ -199,7 +211,7 @@ def main():
     dom_bytes = synth.weight_bytes(dom_w.type, dom_w.N, dom_w.K) + (dom_w.K + dom_w.N) * 4
     dom_gbs = dom_bytes / (dsec / launches) / 1e9
     roofline = {
-        "kernel": "kq::q4k_gemv_kernel (gate|up 28672x4096, M=1)",
+        "kernel": "kq::q4k_gemv_kernel<1, 8> (gate|up 28672x4096 Q4_K, M=1)",
         "bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
         "bytes_per_launch": dom_bytes, "us_per_launch": round(dsec / launches * 1e6, 3),
