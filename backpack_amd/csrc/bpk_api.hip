@@ -120,7 +120,7 @@ const char* bpk_last_kernel(void) { return t_kernel; }
 
 int bpk_force_kernel(int family)
 {
-    if (family < 0 || family > 4) return fail(BPK_ERR_SHAPE, "kernel family %d unknown", family);
+    if (family < 0 || family > 5) return fail(BPK_ERR_SHAPE, "kernel family %d unknown", family);
     t_family = family;
     return BPK_OK;
 }
@@ -136,7 +136,7 @@ int bpk_set_option(const char* name, int value)
         return BPK_OK;
     }
     if (!strcmp(name, "gemv_depth")) {
-        if (value != 0 && value != 1 && value != 2 && value != 4) return fail(BPK_ERR_SHAPE, "gemv_depth must be 0, 1, 2 or 4");
+        if (value < 0 || value > 8) return fail(BPK_ERR_SHAPE, "gemv_depth must be 0..8");
         t_gemv.depth = value;
         return BPK_OK;
     }
@@ -281,7 +281,16 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     const bool mrow_ok = kq::mrow_supported(a);
     if (t_family == 2 && !rows_ok) return fail(BPK_ERR_SHAPE, "row-per-lane GEMV cannot serve this call");
     if (t_family == 3 && !mrow_ok) return fail(BPK_ERR_SHAPE, "matrix-core row kernel cannot serve this call");
-    if (t_family > 3) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
+    const bool stream_ok = kq::gemv_stream_supported(a);
+    if (t_family == 5 && !stream_ok) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");
+    if (t_family == 4) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
+    // short Q4_K matrices at M = 1 are latency-bound: the lanes-along-K kernel has
+    // no LDS staging, no workgroup barrier and no K split to fold
+    if (t_family == 5 || (t_family == 0 && stream_ok && N <= 12288u)) {
+        t_kernel = "gemv_stream";
+        e = kq::launch_gemv_stream(a, t_gemv, s);
+        return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+    }
     // automatic choice: M <= 2 on the VALU row kernel (the 4x4x4 MFMA does not
     // overlap with VALU work on this part), M = 3..16 on the matrix-core row kernel
     const bool use_rows = rows_ok && (t_family == 2 || (t_family == 0 && (M <= 2 || !mrow_ok)));

@@ -49,6 +49,11 @@ size_t gemv_rows_scratch_floats(const MatmulArgs& a, const GemvTuning& t);
 hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const GemvTuning& t,
                             hipStream_t s);
 
+// Lanes-along-K decode GEMV (M = 1): a wave owns whole rows, activations stay
+// in registers.  t.splits, when set, overrides the rows per wave.
+bool gemv_stream_supported(const MatmulArgs& a);
+hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStream_t s);
+
 // Row-per-lane matvec on the matrix cores, M <= 16 dense or grouped by expert.
 bool mrow_supported(const MatmulArgs& a);
 size_t mrow_scratch_floats(const MatmulArgs& a, const GemvTuning& t);

@@ -96,6 +96,8 @@ SHAPES = [
     (Q4_K, 1, 4096, 4096),      # one decode projection (config 0)
     (Q4_K, 1, 1024, 4096),      # k / v projection
     (Q4_K, 1, 100, 256),        # ragged N, single block
+    (Q4_K, 1, 333, 3072),       # 12 blocks: the second pass of the lanes-along-K kernel is partial
+    (Q4_K, 1, 6144, 4096),      # fused q|k|v
     (Q4_K, 1, 64, 14336),       # long rows
     (Q4_K, 2, 200, 1024),
     (Q4_K, 3, 130, 2048),
@@ -116,7 +118,7 @@ SHAPES = [
 
 
 @pytest.mark.parametrize("type_,M,N,K", SHAPES)
-@pytest.mark.parametrize("family", [0, 1, 2, 3])
+@pytest.mark.parametrize("family", [0, 1, 2, 3, 5])
 def test_matmul_vs_oracle(gpu, kqo, type_, M, N, K, family):
     from backpack_amd import capi, kquant
     raw, packed, w = gpu.make_weight(type_, N, K, seed=N + K)
@@ -164,6 +166,38 @@ def test_gemv_split_k_and_counter_reset(gpu, kqo, type_, family, kernel, waves, 
     assert np.array_equal(a, b), "split-K result depends on the launch"
     gpu.check_matmul(kqo, type_, a, X, packed, N, K, label=f"waves={waves} splits={splits}",
                      slack=1e-5 if kernel == "mrow" else 1e-6)
+
+
+@pytest.mark.parametrize("N,K", [(9, 256), (70, 1280), (257, 2048), (1000, 4096)])
+@pytest.mark.parametrize("depth", [1, 2, 4])
+@pytest.mark.parametrize("rows_per_wave", [1, 3, 64])
+def test_gemv_stream_shapes(gpu, kqo, N, K, depth, rows_per_wave):
+    """The lanes-along-K kernel over its tuning space: rows in flight per wave,
+    rows per wave (1 = every wave a single row, 64 = fewer waves than one
+    workgroup holds), one and two passes per row, with a y offset and bias."""
+    import torch
+    from backpack_amd import capi, kquant
+    raw, packed, w = gpu.make_weight(Q4_K, N, K, seed=N)
+    rng = np.random.default_rng(depth * 100 + rows_per_wave)
+    X = rng.standard_normal((1, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    out = torch.full((1, N + 7), 123.0, device="cuda")
+    capi.set_option("gemv_depth", depth)
+    capi.set_option("gemv_splits", rows_per_wave)
+    capi.force_kernel(5)
+    try:
+        _say("stream", N, K, depth, rows_per_wave)
+        xd, bd = gpu.dev(X), gpu.dev(bias)      # named: the buffers must outlive the call
+        capi.check(capi.lib().bpk_kq_matmul(Q4_K, xd.data_ptr(), w.data.data_ptr(), bd.data_ptr(),
+                                            out.data_ptr(), 1, N, K, w.n_blocks, w.row_stride_words, 7, None))
+        assert capi.last_kernel() == "gemv_stream"
+    finally:
+        capi.force_kernel(0)
+        capi.set_option("gemv_depth", 0)
+        capi.set_option("gemv_splits", 0)
+    got = out.cpu().numpy()
+    assert np.all(got[:, :7] == 123.0), "wrote before y_offset"
+    gpu.check_matmul(kqo, Q4_K, got[:, 7:], X, packed, N, K, bias=bias, label=f"stream {N}x{K} d{depth} r{rows_per_wave}")
 
 
 def test_matmul_y_offset_no_bias(gpu, kqo):
