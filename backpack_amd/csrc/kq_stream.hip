@@ -176,15 +176,224 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
     }
 }
 
+// ---------------------------------------------------------------------------
+// Q6_K.  Lane (b, t) = (lane / 8, lane % 8) of a pass takes, in superblock b of
+// the pass's eight, half n = t / 4 and the eight positions l = 8*(t%4) .. +7:
+// 8 bytes of ql[64n + l], 8 of ql[64n + 32 + l], 8 of qh[32n + l] — the 32
+// elements 128n + 32k + l, k = 0..3 — plus the half's 8 scale bytes and d.
+// Blocks are 210 bytes, so these loads are only 2-byte aligned; the hardware
+// takes them as they are.  A row longer than 8*P blocks is cut into KW slices,
+// one wave each; the slices' sums meet in LDS once per 64 rows.
+// ---------------------------------------------------------------------------
+typedef uint32_t s_u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ s_u32x2 load8_a2(const uint8_t* p)
+{
+    s_u32x2 v;
+    __builtin_memcpy(&v, p, 8);
+    return v;
+}
+
+__device__ __forceinline__ uint32_t load2_a2(const uint8_t* p)
+{
+    uint16_t v;
+    __builtin_memcpy(&v, p, 2);
+    return v;
+}
+
+struct Q6Piece {
+    s_u32x2 a, b, h, sc;
+    uint32_t d;
+};
+
+__device__ __forceinline__ Q6Piece q6k_piece_load(const uint8_t* row, uint32_t boff, uint32_t n, uint32_t lg)
+{
+    Q6Piece v;
+    const uint8_t* blk = row + boff;
+    v.a = load8_a2(blk + 64u * n + 8u * lg);
+    v.b = load8_a2(blk + 64u * n + 32u + 8u * lg);
+    v.h = load8_a2(blk + 128u + 32u * n + 8u * lg);
+    v.sc = load8_a2(blk + 192u + 8u * n);
+    v.d = load2_a2(blk + 208u);
+    return v;
+}
+
+// x[k][i]: activation of element 128n + 32k + 8lg + i;  m32xs[k] = -32 * sum_i x[k][i]
+__device__ __forceinline__ float q6k_piece_dot(const Q6Piece& v, const float (&x)[4][8], const float (&m32xs)[4],
+                                               uint32_t sc_shift)
+{
+    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const uint32_t A = v.a[u], B = v.b[u], H = v.h[u];
+        const uint32_t A8 = A >> 8, B8 = B >> 8;
+        const uint32_t Hl4 = H << 4, Hl2 = H << 2, Hr4 = H >> 4, Hr6 = H >> 6;
+        // [k][pair]: pair a holds positions l, l+2; pair b holds l+1, l+3
+        const s_half2 q0a = __builtin_bit_cast(s_half2, (A & 0x000F000Fu) | (Hl4 & 0x00300030u));
+        const s_half2 q2a = __builtin_bit_cast(s_half2, (A & 0x00F000F0u) | (Hl4 & 0x03000300u));
+        const s_half2 q1a = __builtin_bit_cast(s_half2, (B & 0x000F000Fu) | (Hl2 & 0x00300030u));
+        const s_half2 q3a = __builtin_bit_cast(s_half2, (B & 0x00F000F0u) | (Hl2 & 0x03000300u));
+        const s_half2 q0b = __builtin_bit_cast(s_half2, (A8 & 0x000F000Fu) | (Hr4 & 0x00300030u));
+        const s_half2 q2b = __builtin_bit_cast(s_half2, (A8 & 0x00F000F0u) | (Hr4 & 0x03000300u));
+        const s_half2 q1b = __builtin_bit_cast(s_half2, (B8 & 0x000F000Fu) | (Hr6 & 0x00300030u));
+        const s_half2 q3b = __builtin_bit_cast(s_half2, (B8 & 0x00F000F0u) | (Hr6 & 0x03000300u));
+        const int i = 4 * u;
+        a[0] = s_fma_h(q0a.x, x[0][i + 0], a[0]);
+        a[1] = s_fma_h(q1a.x, x[1][i + 0], a[1]);
+        a[2] = s_fma_h(q2a.x, x[2][i + 0], a[2]);
+        a[3] = s_fma_h(q3a.x, x[3][i + 0], a[3]);
+        a[0] = s_fma_h(q0b.x, x[0][i + 1], a[0]);
+        a[1] = s_fma_h(q1b.x, x[1][i + 1], a[1]);
+        a[2] = s_fma_h(q2b.x, x[2][i + 1], a[2]);
+        a[3] = s_fma_h(q3b.x, x[3][i + 1], a[3]);
+        a[0] = s_fma_h(q0a.y, x[0][i + 2], a[0]);
+        a[1] = s_fma_h(q1a.y, x[1][i + 2], a[1]);
+        a[2] = s_fma_h(q2a.y, x[2][i + 2], a[2]);
+        a[3] = s_fma_h(q3a.y, x[3][i + 2], a[3]);
+        a[0] = s_fma_h(q0b.y, x[0][i + 3], a[0]);
+        a[1] = s_fma_h(q1b.y, x[1][i + 3], a[1]);
+        a[2] = s_fma_h(q2b.y, x[2][i + 3], a[2]);
+        a[3] = s_fma_h(q3b.y, x[3][i + 3], a[3]);
+    }
+    // scale of (half n, k, l/16) is byte 2k + l/16 of the half's eight: sc_shift = 8 * (l/16)
+    const uint32_t s01 = v.sc.x >> sc_shift, s23 = v.sc.y >> sc_shift;
+    const float sc0 = (float)(int)(int8_t)(s01 & 255u), sc1 = (float)(int)(int8_t)((s01 >> 16) & 255u);
+    const float sc2 = (float)(int)(int8_t)(s23 & 255u), sc3 = (float)(int)(int8_t)((s23 >> 16) & 255u);
+    float tot = sc0 * __builtin_fmaf(a[0], 16777216.0f, m32xs[0]);
+    tot = __builtin_fmaf(sc1, __builtin_fmaf(a[1], 16777216.0f, m32xs[1]), tot);
+    tot = __builtin_fmaf(sc2, __builtin_fmaf(a[2], 1048576.0f, m32xs[2]), tot);
+    tot = __builtin_fmaf(sc3, __builtin_fmaf(a[3], 1048576.0f, m32xs[3]), tot);
+    return half_bits_to_float(v.d) * tot;
+}
+
+// Workgroup = KW waves, one K slice of 8*P superblocks each; the workgroup walks
+// rows blockIdx.x, + gridDim.x, ...; D rows in flight per wave.
+template <int P, int KW, int D>
+__global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
+{
+    __shared__ float part[KW > 1 ? KW : 1][64];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t g = blockIdx.x, stride = gridDim.x;
+    const uint32_t n_rows = g < p.N ? (p.N - g + stride - 1u) / stride : 0u;
+    const uint32_t bl = lane >> 3, t = lane & 7u, n = t >> 2, lg = t & 3u;
+    const uint32_t sc_shift = 8u * (lg >> 1);
+
+    float x[P][4][8], m32xs[P][4];
+    uint32_t boff[P];
+#pragma unroll
+    for (int pass = 0; pass < P; ++pass) {
+        uint32_t b = (wave * P + pass) * 8u + bl;
+        const bool valid = b < p.n_blocks;
+        b = valid ? b : p.n_blocks - 1u;
+        boff[pass] = b * KQ_Q6K_BYTES;
+        const float4* xp = (const float4*)(p.X + (size_t)b * KQ_QK + 128u * n + 8u * lg);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float4 lo = xp[8 * k], hi = xp[8 * k + 1];
+            if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
+            x[pass][k][0] = lo.x; x[pass][k][1] = lo.y; x[pass][k][2] = lo.z; x[pass][k][3] = lo.w;
+            x[pass][k][4] = hi.x; x[pass][k][5] = hi.y; x[pass][k][6] = hi.z; x[pass][k][7] = hi.w;
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sum += x[pass][k][i];
+            m32xs[pass][k] = -32.0f * sum;
+        }
+    }
+
+    Q6Piece ring[D][P];
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        const uint32_t r = g + min((uint32_t)d, n_rows ? n_rows - 1u : 0u) * stride;
+        const uint8_t* rp = p.W + (size_t)min(r, p.N - 1u) * p.row_stride_bytes;
+#pragma unroll
+        for (int pass = 0; pass < P; ++pass) ring[d][pass] = q6k_piece_load(rp, boff[pass], n, lg);
+    }
+    float res = 0.0f;   // lane i keeps the sum of the workgroup's row i0 + i
+    for (uint32_t i0 = 0; i0 < n_rows; i0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const uint32_t i = i0 + d;
+            if (i < n_rows) {
+                float acc = 0.0f;
+#pragma unroll
+                for (int pass = 0; pass < P; ++pass) acc += q6k_piece_dot(ring[d][pass], x[pass], m32xs[pass], sc_shift);
+                if (i + D < n_rows) {
+                    const uint8_t* rp = p.W + (size_t)(g + (i + D) * stride) * p.row_stride_bytes;
+#pragma unroll
+                    for (int pass = 0; pass < P; ++pass) ring[d][pass] = q6k_piece_load(rp, boff[pass], n, lg);
+                }
+                const float tot = wave_sum(acc);
+                res = lane == (i & 63u) ? tot : res;
+                if ((i & 63u) == 63u || i + 1u == n_rows) {
+                    // rows i - (i & 63) .. i are complete in this wave: fold the K slices and store
+                    if (KW > 1) {
+                        part[wave][lane] = res;
+                        __syncthreads();
+                    }
+                    if (wave == 0 && lane <= (i & 63u)) {
+                        float y = res;
+                        if (KW > 1) {
+                            y = part[0][lane];
+#pragma unroll
+                            for (int w = 1; w < KW; ++w) y += part[w][lane];
+                        }
+                        const uint32_t r = g + (i - (i & 63u) + lane) * stride;
+                        p.Y[p.y_offset + r] = y + (p.bias ? p.bias[r] : 0.0f);
+                    }
+                    if (KW > 1) __syncthreads();
+                }
+            }
+        }
+    }
+}
+
+// Compute units of the current device (cached per device id).
+static uint32_t cu_count()
+{
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256u;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return (uint32_t)cached[dev];
+}
+
+// Workgroups for a kernel whose workgroups hold waves_per_wg waves and walk rows
+// g, g + wgs, ...: a whole multiple of the CU count, so that every CU gets the
+// same number of workgroups, about eight waves per CU (measured on MI355X: more
+// waves, or deeper per-wave prefetch, are slower), at least two rows each so
+// that the activations are not loaded for a single row.
+static uint32_t stream_workgroups(uint32_t N, uint32_t waves_per_wg, int rows_override)
+{
+    if (rows_override > 0) return (N + (uint32_t)rows_override - 1u) / (uint32_t)rows_override;
+    const uint32_t cus = cu_count();
+    const uint32_t per_cu = waves_per_wg >= 8u ? 1u : 8u / waves_per_wg;
+    const uint32_t want = cus * per_cu;
+    const uint32_t most = (N + 1u) / 2u;
+    return most < want ? (most ? most : 1u) : want;
+}
+
 bool gemv_stream_supported(const MatmulArgs& a)
 {
     if (a.expert_idx) return false;
     if (a.M != 1) return false;
-    if (a.type != KQ_TYPE_Q4_K) return false;
-    if (a.n_blocks < 1 || a.n_blocks > 16) return false;
-    if (((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u)) return false;
     if (((uintptr_t)a.X & 15u)) return false;
-    return true;
+    if (a.n_blocks < 1) return false;
+    if (a.type == KQ_TYPE_Q4_K) {
+        if (a.n_blocks > 16) return false;
+        if (((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u)) return false;
+        return true;
+    }
+    if (a.type == KQ_TYPE_Q6_K) {
+        if (a.n_blocks > 112) return false;
+        if (((uintptr_t)a.W & 1u) || (a.row_stride_bytes & 1u)) return false;
+        return true;
+    }
+    return false;
 }
 
 hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStream_t s)
@@ -198,14 +407,31 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     p.n_blocks = a.n_blocks;
     p.row_stride_bytes = a.row_stride_bytes;
     p.y_offset = a.y_offset;
-    // about 4096 waves (16 per CU), at least two rows each so that the
-    // activations are not loaded for a single row
-    uint32_t rpw = t.splits > 0 ? (uint32_t)t.splits : (a.N + 4095u) / 4096u;
-    if (t.splits <= 0 && rpw < 2u) rpw = 2u;
+    const int depth = t.depth > 0 ? t.depth : 1;
+    if (a.type == KQ_TYPE_Q6_K) {
+        // K slices of 8 or 16 superblocks, one wave each
+        const uint32_t nb = a.n_blocks;
+        const int kw = nb <= 16u ? 1 : nb <= 32u ? 4 : 7;
+        const int pp = nb <= 8u ? 1 : nb <= 16u ? 2 : nb <= 56u ? 1 : 2;
+        const uint32_t wgs = stream_workgroups(a.N, (uint32_t)kw, t.splits);
+#define KQ_STREAM6(P, KW) \
+    do { \
+        if (depth <= 1) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 1>), dim3(wgs), dim3(64 * KW), 0, s, p); \
+        else if (depth <= 2) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 2>), dim3(wgs), dim3(64 * KW), 0, s, p); \
+        else hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 4>), dim3(wgs), dim3(64 * KW), 0, s, p); \
+    } while (0)
+        if (kw == 1 && pp == 1) KQ_STREAM6(1, 1);
+        else if (kw == 1) KQ_STREAM6(2, 1);
+        else if (kw == 4) KQ_STREAM6(1, 4);
+        else if (pp == 1) KQ_STREAM6(1, 7);
+        else KQ_STREAM6(2, 7);
+#undef KQ_STREAM6
+        return hipGetLastError();
+    }
     constexpr int NW = 4;
-    const uint32_t waves = (a.N + rpw - 1u) / rpw;
-    const uint32_t wgs = (waves + NW - 1u) / NW;
-    const int depth = t.depth > 0 ? t.depth : 2;
+    // a Q4_K workgroup is NW independent waves, each with its own rows
+    const uint32_t wgs = t.splits > 0 ? ((a.N + (uint32_t)t.splits - 1u) / (uint32_t)t.splits + NW - 1u) / NW
+                                      : stream_workgroups((a.N + NW - 1u) / NW, NW, 0);
 #define KQ_STREAM_LAUNCH(P, D) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D>), dim3(wgs), dim3(64 * NW), 0, s, p)
     if (a.n_blocks <= 8u) {
         if (depth <= 1) KQ_STREAM_LAUNCH(1, 1);

@@ -168,16 +168,24 @@ def test_gemv_split_k_and_counter_reset(gpu, kqo, type_, family, kernel, waves, 
                      slack=1e-5 if kernel == "mrow" else 1e-6)
 
 
-@pytest.mark.parametrize("N,K", [(9, 256), (70, 1280), (257, 2048), (1000, 4096)])
+STREAM_SHAPES = [
+    (Q4_K, 9, 256), (Q4_K, 70, 1280), (Q4_K, 257, 2048), (Q4_K, 1000, 4096),
+    # Q6_K: one pass, two passes, 4 K-slices (one partial), 7 slices, 7 slices x 2 passes
+    (Q6_K, 9, 256), (Q6_K, 70, 768), (Q6_K, 300, 4096), (Q6_K, 130, 6400), (Q6_K, 200, 14336), (Q6_K, 40, 28672),
+]
+
+
+@pytest.mark.parametrize("type_,N,K", STREAM_SHAPES)
 @pytest.mark.parametrize("depth", [1, 2, 4])
-@pytest.mark.parametrize("rows_per_wave", [1, 3, 64])
-def test_gemv_stream_shapes(gpu, kqo, N, K, depth, rows_per_wave):
+@pytest.mark.parametrize("rows_per_wave", [1, 3, 100])
+def test_gemv_stream_shapes(gpu, kqo, type_, N, K, depth, rows_per_wave):
     """The lanes-along-K kernel over its tuning space: rows in flight per wave,
-    rows per wave (1 = every wave a single row, 64 = fewer waves than one
-    workgroup holds), one and two passes per row, with a y offset and bias."""
+    rows per wave (1 = every wave a single row, 100 = more than the 64 rows a
+    wave folds at a time), every pass / K-slice configuration, ragged last
+    pass, with a y offset and bias."""
     import torch
     from backpack_amd import capi, kquant
-    raw, packed, w = gpu.make_weight(Q4_K, N, K, seed=N)
+    raw, packed, w = gpu.make_weight(type_, N, K, seed=N)
     rng = np.random.default_rng(depth * 100 + rows_per_wave)
     X = rng.standard_normal((1, K)).astype(np.float32)
     bias = rng.standard_normal(N).astype(np.float32)
@@ -186,9 +194,9 @@ def test_gemv_stream_shapes(gpu, kqo, N, K, depth, rows_per_wave):
     capi.set_option("gemv_splits", rows_per_wave)
     capi.force_kernel(5)
     try:
-        _say("stream", N, K, depth, rows_per_wave)
+        _say("stream", type_, N, K, depth, rows_per_wave)
         xd, bd = gpu.dev(X), gpu.dev(bias)      # named: the buffers must outlive the call
-        capi.check(capi.lib().bpk_kq_matmul(Q4_K, xd.data_ptr(), w.data.data_ptr(), bd.data_ptr(),
+        capi.check(capi.lib().bpk_kq_matmul(type_, xd.data_ptr(), w.data.data_ptr(), bd.data_ptr(),
                                             out.data_ptr(), 1, N, K, w.n_blocks, w.row_stride_words, 7, None))
         assert capi.last_kernel() == "gemv_stream"
     finally:
@@ -197,7 +205,8 @@ def test_gemv_stream_shapes(gpu, kqo, N, K, depth, rows_per_wave):
         capi.set_option("gemv_splits", 0)
     got = out.cpu().numpy()
     assert np.all(got[:, :7] == 123.0), "wrote before y_offset"
-    gpu.check_matmul(kqo, Q4_K, got[:, 7:], X, packed, N, K, bias=bias, label=f"stream {N}x{K} d{depth} r{rows_per_wave}")
+    gpu.check_matmul(kqo, type_, got[:, 7:], X, packed, N, K, bias=bias,
+                     label=f"stream {type_} {N}x{K} d{depth} r{rows_per_wave}")
 
 
 def test_matmul_y_offset_no_bias(gpu, kqo):
