@@ -284,9 +284,10 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     const bool stream_ok = kq::gemv_stream_supported(a);
     if (t_family == 5 && !stream_ok) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");
     if (t_family == 4) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
-    // matrices of up to a few thousand rows at M = 1 are latency-bound: the
-    // lanes-along-K kernel has no LDS staging and no K split to fold
-    if (t_family == 5 || (t_family == 0 && stream_ok && N <= 12288u)) {
+    // up to a few tens of thousands of rows the lanes-along-K kernel wins at M = 1
+    // (no LDS staging, no K split to fold); longer matrices reach a steady state
+    // in which the row-per-lane kernel streams faster
+    if (t_family == 5 || (t_family == 0 && stream_ok && N <= 32768u)) {
         t_kernel = "gemv_stream";
         e = kq::launch_gemv_stream(a, t_gemv, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);

@@ -56,6 +56,38 @@ __device__ __forceinline__ float wave_sum(float v)
     return (a + b) + (c + d);
 }
 
+// Weight loads whose completion is waited for by hand.  The compiler's own
+// s_waitcnt placement drains the whole queue at the loop head when a register
+// ring is refilled inside a loop, which serialises fetch and arithmetic; these
+// loads are invisible to it.  Rules that keep this sound: (1) a register
+// filled by one of these loads is not read until it has passed through
+// ring_wait<N>() below (the "+v" operands make every later use depend on the
+// wait); (2) vector memory operations complete in issue order, so after
+// s_waitcnt vmcnt(N) every load but the N youngest has landed; (3) loads the
+// compiler does track only ever wait for more than they need.
+typedef uint32_t s_u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ s_u32x4 ring_load16(const uint8_t* ptr)
+{
+    s_u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(ptr));
+    return v;
+}
+
+__device__ __forceinline__ s_u32x2 ring_load8(const uint8_t* ptr)
+{
+    s_u32x2 v;
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(ptr));
+    return v;
+}
+
+__device__ __forceinline__ uint32_t ring_load2(const uint8_t* ptr)
+{
+    uint32_t v;
+    asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(ptr));
+    return v;
+}
+
 // One lane's share of one pass of a Q4_K row.
 //   hdr: the block's first 16 bytes; q: 16 quant bytes (piece j of the block)
 //   xlo/xhi: activations of the piece's 16 elements in the even / odd sub-block
@@ -100,6 +132,29 @@ __device__ __forceinline__ float q4k_piece_dot(const s_u32x4 hdr, const s_u32x4 
     return __builtin_fmaf(d * 16777216.0f, t, -(dmin * u));
 }
 
+// One row in flight for the Q4_K kernel: P headers and P quant pieces per lane.
+template <int P>
+struct Q4Slot {
+    s_u32x4 hdr[P], q[P];
+    __device__ __forceinline__ void fill(const uint8_t* row, const uint32_t (&hoff)[P], uint32_t j)
+    {
+#pragma unroll
+        for (int pass = 0; pass < P; ++pass) {
+            hdr[pass] = ring_load16(row + hoff[pass]);
+            q[pass] = ring_load16(row + hoff[pass] + 16u + 16u * j);
+        }
+    }
+    // Every register of the slot passes through the wait.
+    template <int N>
+    __device__ __forceinline__ void wait()
+    {
+        if constexpr (P == 1)
+            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(hdr[0]), "+v"(q[0]) : "n"(N));
+        else
+            asm volatile("s_waitcnt vmcnt(%4)" : "+v"(hdr[0]), "+v"(q[0]), "+v"(hdr[1]), "+v"(q[1]) : "n"(N));
+    }
+};
+
 // P passes of 8 superblocks cover a row (n_blocks <= 8 * P); D rows in flight.
 template <int P, int NW, int D>
 __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
@@ -139,41 +194,42 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
         xs_hi[pass] = sh_;
     }
 
-    s_u32x4 hdr[D][P], q[D][P];
+    // Ring of D rows in flight.  Slot d is refilled as soon as its row has been
+    // consumed; the wait before a slot's arithmetic leaves the (D-1) younger
+    // slots' loads outstanding.  Past the end of the wave's rows the last row is
+    // fetched and summed again (cache hits, result dropped), so the row loop has
+    // no branch and the number of loads in flight is the same at every wait.
+    constexpr int SLOT_LOADS = 2 * P;
+    Q4Slot<P> ring[D];
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-        const uint32_t r = gw + min((uint32_t)d, n_rows - 1u) * stride;
-        const uint8_t* rp = p.W + (size_t)r * p.row_stride_bytes;
+    for (int d = 0; d < D; ++d)
+        ring[d].fill(p.W + (size_t)(gw + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, hoff, j);
+    // Rows are taken 64 at a time: lane i keeps the sum of the chunk's row i, and the
+    // chunk is stored (bias added) after its last row.
+    for (uint32_t c0 = 0; c0 < n_rows; c0 += 64u) {
+        const uint32_t cnt = min(64u, n_rows - c0);
+        float res = 0.0f;
+        for (uint32_t i0 = 0; i0 < cnt; i0 += D) {
 #pragma unroll
-        for (int pass = 0; pass < P; ++pass) {
-            hdr[d][pass] = *(const s_u32x4*)(rp + hoff[pass]);
-            q[d][pass] = *(const s_u32x4*)(rp + hoff[pass] + 16u + 16u * j);
-        }
-    }
-    for (uint32_t i0 = 0; i0 < n_rows; i0 += D) {
-#pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const uint32_t i = i0 + d;
-            if (i < n_rows) {
-                const uint32_t r = gw + i * stride;
+            for (int d = 0; d < D; ++d) {
+                const uint32_t i = i0 + d;
+                ring[d].template wait<(D - 1) * SLOT_LOADS>();
                 float acc = 0.0f;
 #pragma unroll
                 for (int pass = 0; pass < P; ++pass)
-                    acc += q4k_piece_dot(hdr[d][pass], q[d][pass], xlo[pass], xhi[pass], xs_lo[pass], xs_hi[pass],
-                                         sel_hi, sh);
-                if (i + D < n_rows) {
-                    const uint8_t* rp = p.W + (size_t)(r + D * stride) * p.row_stride_bytes;
-#pragma unroll
-                    for (int pass = 0; pass < P; ++pass) {
-                        hdr[d][pass] = *(const s_u32x4*)(rp + hoff[pass]);
-                        q[d][pass] = *(const s_u32x4*)(rp + hoff[pass] + 16u + 16u * j);
-                    }
-                }
+                    acc += q4k_piece_dot(ring[d].hdr[pass], ring[d].q[pass], xlo[pass], xhi[pass], xs_lo[pass],
+                                         xs_hi[pass], sel_hi, sh);
+                ring[d].fill(p.W + (size_t)(gw + min(c0 + i + D, n_rows - 1u) * stride) * p.row_stride_bytes, hoff, j);
                 const float tot = wave_sum(acc);
-                if (lane == 0) p.Y[p.y_offset + r] = tot + (p.bias ? p.bias[r] : 0.0f);
+                res = (lane == i && i < cnt) ? tot : res;
             }
         }
+        if (lane < cnt) {
+            const uint32_t r = gw + (c0 + lane) * stride;
+            p.Y[p.y_offset + r] = res + (p.bias ? p.bias[r] : 0.0f);
+        }
     }
+    asm volatile("s_waitcnt vmcnt(0)");   // the ring's last refills land before the wave ends
 }
 
 // ---------------------------------------------------------------------------
@@ -185,38 +241,42 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
 // takes them as they are.  A row longer than 8*P blocks is cut into KW slices,
 // one wave each; the slices' sums meet in LDS once per 64 rows.
 // ---------------------------------------------------------------------------
-typedef uint32_t s_u32x2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ s_u32x2 load8_a2(const uint8_t* p)
-{
-    s_u32x2 v;
-    __builtin_memcpy(&v, p, 8);
-    return v;
-}
-
-__device__ __forceinline__ uint32_t load2_a2(const uint8_t* p)
-{
-    uint16_t v;
-    __builtin_memcpy(&v, p, 2);
-    return v;
-}
 
 struct Q6Piece {
     s_u32x2 a, b, h, sc;
     uint32_t d;
 };
 
-__device__ __forceinline__ Q6Piece q6k_piece_load(const uint8_t* row, uint32_t boff, uint32_t n, uint32_t lg)
-{
-    Q6Piece v;
-    const uint8_t* blk = row + boff;
-    v.a = load8_a2(blk + 64u * n + 8u * lg);
-    v.b = load8_a2(blk + 64u * n + 32u + 8u * lg);
-    v.h = load8_a2(blk + 128u + 32u * n + 8u * lg);
-    v.sc = load8_a2(blk + 192u + 8u * n);
-    v.d = load2_a2(blk + 208u);
-    return v;
-}
+// One row in flight for the Q6_K kernel: P pieces per lane, 5 loads each.
+template <int P>
+struct Q6Slot {
+    Q6Piece v[P];
+    __device__ __forceinline__ void fill(const uint8_t* row, const uint32_t (&boff)[P], uint32_t n, uint32_t lg)
+    {
+#pragma unroll
+        for (int pass = 0; pass < P; ++pass) {
+            const uint8_t* blk = row + boff[pass];
+            v[pass].a = ring_load8(blk + 64u * n + 8u * lg);
+            v[pass].b = ring_load8(blk + 64u * n + 32u + 8u * lg);
+            v[pass].h = ring_load8(blk + 128u + 32u * n + 8u * lg);
+            v[pass].sc = ring_load8(blk + 192u + 8u * n);
+            v[pass].d = ring_load2(blk + 208u);
+        }
+    }
+    template <int N>
+    __device__ __forceinline__ void wait()
+    {
+        if constexpr (P == 1)
+            asm volatile("s_waitcnt vmcnt(%5)"
+                         : "+v"(v[0].a), "+v"(v[0].b), "+v"(v[0].h), "+v"(v[0].sc), "+v"(v[0].d)
+                         : "n"(N));
+        else
+            asm volatile("s_waitcnt vmcnt(%10)"
+                         : "+v"(v[0].a), "+v"(v[0].b), "+v"(v[0].h), "+v"(v[0].sc), "+v"(v[0].d), "+v"(v[1].a),
+                           "+v"(v[1].b), "+v"(v[1].h), "+v"(v[1].sc), "+v"(v[1].d)
+                         : "n"(N));
+    }
+};
 
 // x[k][i]: activation of element 128n + 32k + 8lg + i;  m32xs[k] = -32 * sum_i x[k][i]
 __device__ __forceinline__ float q6k_piece_dot(const Q6Piece& v, const float (&x)[4][8], const float (&m32xs)[4],
@@ -301,51 +361,49 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
         }
     }
 
-    Q6Piece ring[D][P];
+    if (n_rows == 0) return;   // whole workgroup
+    constexpr int SLOT_LOADS = 5 * P;
+    Q6Slot<P> ring[D];
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-        const uint32_t r = g + min((uint32_t)d, n_rows ? n_rows - 1u : 0u) * stride;
-        const uint8_t* rp = p.W + (size_t)min(r, p.N - 1u) * p.row_stride_bytes;
+    for (int d = 0; d < D; ++d)
+        ring[d].fill(p.W + (size_t)(g + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, boff, n, lg);
+    // Rows are taken 64 at a time: lane i keeps the sum of the chunk's row i; the K
+    // slices are folded and the chunk stored after its last row.  The row loop is
+    // the one of the Q4_K kernel.
+    for (uint32_t c0 = 0; c0 < n_rows; c0 += 64u) {
+        const uint32_t cnt = min(64u, n_rows - c0);
+        float res = 0.0f;
+        for (uint32_t i0 = 0; i0 < cnt; i0 += D) {
 #pragma unroll
-        for (int pass = 0; pass < P; ++pass) ring[d][pass] = q6k_piece_load(rp, boff[pass], n, lg);
-    }
-    float res = 0.0f;   // lane i keeps the sum of the workgroup's row i0 + i
-    for (uint32_t i0 = 0; i0 < n_rows; i0 += D) {
-#pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const uint32_t i = i0 + d;
-            if (i < n_rows) {
+            for (int d = 0; d < D; ++d) {
+                const uint32_t i = i0 + d;
+                ring[d].template wait<(D - 1) * SLOT_LOADS>();
                 float acc = 0.0f;
 #pragma unroll
-                for (int pass = 0; pass < P; ++pass) acc += q6k_piece_dot(ring[d][pass], x[pass], m32xs[pass], sc_shift);
-                if (i + D < n_rows) {
-                    const uint8_t* rp = p.W + (size_t)(g + (i + D) * stride) * p.row_stride_bytes;
-#pragma unroll
-                    for (int pass = 0; pass < P; ++pass) ring[d][pass] = q6k_piece_load(rp, boff[pass], n, lg);
-                }
+                for (int pass = 0; pass < P; ++pass)
+                    acc += q6k_piece_dot(ring[d].v[pass], x[pass], m32xs[pass], sc_shift);
+                ring[d].fill(p.W + (size_t)(g + min(c0 + i + D, n_rows - 1u) * stride) * p.row_stride_bytes, boff, n, lg);
                 const float tot = wave_sum(acc);
-                res = lane == (i & 63u) ? tot : res;
-                if ((i & 63u) == 63u || i + 1u == n_rows) {
-                    // rows i - (i & 63) .. i are complete in this wave: fold the K slices and store
-                    if (KW > 1) {
-                        part[wave][lane] = res;
-                        __syncthreads();
-                    }
-                    if (wave == 0 && lane <= (i & 63u)) {
-                        float y = res;
-                        if (KW > 1) {
-                            y = part[0][lane];
-#pragma unroll
-                            for (int w = 1; w < KW; ++w) y += part[w][lane];
-                        }
-                        const uint32_t r = g + (i - (i & 63u) + lane) * stride;
-                        p.Y[p.y_offset + r] = y + (p.bias ? p.bias[r] : 0.0f);
-                    }
-                    if (KW > 1) __syncthreads();
-                }
+                res = (lane == i && i < cnt) ? tot : res;
             }
         }
+        if (KW > 1) {
+            part[wave][lane] = res;
+            __syncthreads();
+        }
+        if (wave == 0 && lane < cnt) {
+            float y = res;
+            if (KW > 1) {
+                y = part[0][lane];
+#pragma unroll
+                for (int w = 1; w < KW; ++w) y += part[w][lane];
+            }
+            const uint32_t r = g + (c0 + lane) * stride;
+            p.Y[p.y_offset + r] = y + (p.bias ? p.bias[r] : 0.0f);
+        }
+        if (KW > 1) __syncthreads();
     }
+    asm volatile("s_waitcnt vmcnt(0)");   // the ring's last refills land before the wave ends
 }
 
 // Compute units of the current device (cached per device id).
@@ -362,17 +420,13 @@ static uint32_t cu_count()
     return (uint32_t)cached[dev];
 }
 
-// Workgroups for a kernel whose workgroups hold waves_per_wg waves and walk rows
-// g, g + wgs, ...: a whole multiple of the CU count, so that every CU gets the
-// same number of workgroups, about eight waves per CU (measured on MI355X: more
-// waves, or deeper per-wave prefetch, are slower), at least two rows each so
-// that the activations are not loaded for a single row.
-static uint32_t stream_workgroups(uint32_t N, uint32_t waves_per_wg, int rows_override)
+// Workgroups for a kernel whose workgroups walk rows g, g + wgs, ...: a whole
+// multiple of the CU count, so that every CU gets the same number of workgroups,
+// at least two rows each so that the activations are not loaded for a single row.
+static uint32_t stream_workgroups(uint32_t N, uint32_t per_cu, int rows_override)
 {
     if (rows_override > 0) return (N + (uint32_t)rows_override - 1u) / (uint32_t)rows_override;
-    const uint32_t cus = cu_count();
-    const uint32_t per_cu = waves_per_wg >= 8u ? 1u : 8u / waves_per_wg;
-    const uint32_t want = cus * per_cu;
+    const uint32_t want = cu_count() * per_cu;
     const uint32_t most = (N + 1u) / 2u;
     return most < want ? (most ? most : 1u) : want;
 }
@@ -407,13 +461,16 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     p.n_blocks = a.n_blocks;
     p.row_stride_bytes = a.row_stride_bytes;
     p.y_offset = a.y_offset;
-    const int depth = t.depth > 0 ? t.depth : 1;
+    // Measured on MI355X: these kernels run best with about 40 KB of weight loads
+    // in flight per CU: 4 to 8 waves, two to four rows in flight each.  More waves
+    // or deeper rings are slower.
     if (a.type == KQ_TYPE_Q6_K) {
         // K slices of 8 or 16 superblocks, one wave each
         const uint32_t nb = a.n_blocks;
         const int kw = nb <= 16u ? 1 : nb <= 32u ? 4 : 7;
         const int pp = nb <= 8u ? 1 : nb <= 16u ? 2 : nb <= 56u ? 1 : 2;
-        const uint32_t wgs = stream_workgroups(a.N, (uint32_t)kw, t.splits);
+        const uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 8u / (uint32_t)kw, t.splits);
+        const int depth = t.depth > 0 ? t.depth : 2;
 #define KQ_STREAM6(P, KW) \
     do { \
         if (depth <= 1) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 1>), dim3(wgs), dim3(64 * KW), 0, s, p); \
@@ -431,7 +488,8 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     constexpr int NW = 4;
     // a Q4_K workgroup is NW independent waves, each with its own rows
     const uint32_t wgs = t.splits > 0 ? ((a.N + (uint32_t)t.splits - 1u) / (uint32_t)t.splits + NW - 1u) / NW
-                                      : stream_workgroups((a.N + NW - 1u) / NW, NW, 0);
+                                      : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
+    const int depth = t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
 #define KQ_STREAM_LAUNCH(P, D) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D>), dim3(wgs), dim3(64 * NW), 0, s, p)
     if (a.n_blocks <= 8u) {
         if (depth <= 1) KQ_STREAM_LAUNCH(1, 1);
