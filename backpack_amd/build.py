@@ -6,6 +6,7 @@ from __future__ import annotations
 import concurrent.futures as cf
 import glob
 import os
+import re
 import subprocess
 import sys
 
@@ -23,12 +24,28 @@ FLAGS = [
 ]
 
 
+# A source that carries this marker issues global loads from inline asm and waits
+# for them by hand; that is only sound while the loaded registers stay where they
+# are, so such a file must compile without any register spill or scratch use.
+NO_SPILL_MARKER = "KQ_REQUIRES_NO_SPILL"
+
+
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", ".o"))
-    extra = os.environ.get("BPK_EXTRA_FLAGS", "").split()   # experiments only, e.g. -DKQ_PLAIN_LOADS
+    extra = os.environ.get("BPK_EXTRA_FLAGS", "").split()   # experiments only
+    with open(src) as f:
+        guarded = NO_SPILL_MARKER in f.read()
+    if guarded:
+        extra.append("-Rpass-analysis=kernel-resource-usage")
     cmd = [HIPCC, *FLAGS, *extra, "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
-    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+    lines = r.stderr.splitlines()
+    if guarded:
+        bad = [l for l in lines if re.search(r"(Spill|ScratchSize[^:]*):\s*[1-9]", l)]
+        if bad and r.returncode == 0:
+            raise RuntimeError(f"{src} must not spill registers (hand-waited loads):\n" + "\n".join(bad[:8]))
+        lines = [l for l in lines if "kernel-resource-usage" not in l and not re.match(r"^\s*\d*\s*\|", l)]
+    err = "\n".join(l for l in lines if "packed-fp32-ops" not in l)
     if r.returncode:
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
     if err.strip():

@@ -1,14 +1,21 @@
 // kq_gemm.hip — prefill dequant-GEMM: Y[M,N] = X[M,K] (bf16) * dequant(W)[N,K]^T.
 //
-// A workgroup of 4 waves owns a BM x BN tile of Y and walks K in steps of 64.
-// Per step the X tile is copied to LDS as is, and the W tile is dequantised
-// from its Q4_K / Q6_K bytes to bf16 (fp32 arithmetic, one RNE rounding)
-// straight into LDS, so weights cross HBM as 4.5 / 6.56 bits per element and
-// are expanded once per BM tokens.  The four waves (2 x 2) contract their
-// quarter of the tile with v_mfma_f32_32x32x16_bf16, fp32 accumulation in
-// registers.  LDS is double-buffered with one barrier per step; the global
-// loads of step t+1 are issued before the MFMAs of step t, the dequantisation
-// of step t+1 runs after them.
+// A workgroup owns a BM x BN tile of Y and walks K in steps of 64.  Per step the
+// X tile is copied to LDS as is, and the W tile is dequantised from its Q4_K /
+// Q6_K bytes to bf16 (fp32 arithmetic, one RNE rounding) straight into LDS, so
+// weights cross HBM as 4.5 / 6.56 bits per element and are expanded once per
+// BM tokens.  The waves contract their part of the tile with
+// v_mfma_f32_32x32x16_bf16, fp32 accumulation in registers.  LDS is
+// double-buffered with one barrier per step.
+//
+// The 256 x 256 tile runs 8 waves (2 x 4, 128 x 64 each), two per SIMD, in two
+// phases: waves 0..3 issue the global loads of step t+1, run the MFMAs of step
+// t and then dequantise step t+1; waves 4..7 first dequantise step t+1 from
+// registers loaded a step earlier, issue the loads of step t+2, then run the
+// MFMAs of step t.  On every SIMD one wave's conversion arithmetic therefore
+// overlaps the other wave's matrix work.  The 128 x 128 tile runs 4 waves
+// (2 x 2) and fits twice on a CU, which gives the same overlap between
+// workgroups.
 //
 // LDS rows are 64 bf16 + 16 bytes of padding (144 B = an odd number of 16-byte
 // slots), which makes the 128-bit fragment reads of 32 consecutive rows
@@ -97,15 +104,22 @@ __device__ __forceinline__ void q6k_load(const uint8_t* row, uint32_t kc, uint32
 {
     const uint32_t c = kc & 3u, h = c >> 1, t = (c & 1u) * 2u + hf;
     const uint8_t* blk = row + (size_t)(kc >> 2) * KQ_Q6K_BYTES;
-    const uint16_t* ql = (const uint16_t*)(blk + 64u * h + 32u * (t & 1u));
-    const uint16_t* qh = (const uint16_t*)(blk + 128u + 32u * h);
+    // 2-byte aligned 128-bit loads: the hardware takes them as they are
+    u32x4 a0, a1, b0, b1;
+    __builtin_memcpy(&a0, blk + 64u * h + 32u * (t & 1u), 16);
+    __builtin_memcpy(&a1, blk + 64u * h + 32u * (t & 1u) + 16u, 16);
+    __builtin_memcpy(&b0, blk + 128u + 32u * h, 16);
+    __builtin_memcpy(&b1, blk + 128u + 32u * h + 16u, 16);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        r.ql[i] = (uint32_t)ql[2 * i] | ((uint32_t)ql[2 * i + 1] << 16);
-        r.qh[i] = (uint32_t)qh[2 * i] | ((uint32_t)qh[2 * i + 1] << 16);
+    for (int i = 0; i < 4; ++i) {
+        r.ql[i] = a0[i]; r.ql[4 + i] = a1[i];
+        r.qh[i] = b0[i]; r.qh[4 + i] = b1[i];
     }
-    r.sc2 = *(const uint16_t*)(blk + 192u + 8u * h + 2u * t);
-    r.d16 = *(const uint16_t*)(blk + 208u);
+    uint16_t s2, d2;
+    __builtin_memcpy(&s2, blk + 192u + 8u * h + 2u * t, 2);
+    __builtin_memcpy(&d2, blk + 208u, 2);
+    r.sc2 = s2;
+    r.d16 = d2;
 }
 
 __device__ __forceinline__ void q6k_expand(const Q6Raw& r, uint32_t kc, uint32_t hf, uint8_t* dst)
@@ -135,35 +149,41 @@ __device__ __forceinline__ void q6k_expand(const Q6Raw& r, uint32_t kc, uint32_t
     }
 }
 
-template <int TYPE, int BM, int BN>
-__global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmParams p)
+template <int TYPE, int BM, int BN, int NWAVES>
+__global__ __launch_bounds__(64 * NWAVES) void gemm_bf16_kernel(GemmParams p)
 {
     extern __shared__ __align__(16) uint8_t smem[];
-    constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    constexpr int NT = 64 * NWAVES;
+    constexpr int WAVES_N = NWAVES / 2;                       // waves are laid out 2 (M) x NWAVES/2 (N)
+    constexpr int WM = BM / 2, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int A_BYTES = BM * GEMM_LD, B_BYTES = BN * GEMM_LD;
-    constexpr int XP = BM / 32;          // X passes: 32 rows x 128 bytes per pass
-    constexpr int WI = BN * 2 / 256;     // W items (row, 32-element run) per thread
+    constexpr int XROWS = NT / 8;         // X rows per pass: 8 threads x 16 bytes per row
+    constexpr int XP = BM / XROWS;        // X passes
+    constexpr int WI = BN * 2 / NT;       // W items (row, 32-element run) per thread
+    constexpr bool PHASED = NWAVES == 8;  // second half of the waves converts before it multiplies
     uint8_t* As = smem;
     uint8_t* Bs = smem + 2 * A_BYTES;
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t wm = wave >> 1, wn = wave & 1u;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave / WAVES_N, wn = wave % WAVES_N;
     const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const uint32_t nk = p.K / GEMM_BK;
+    const bool convert_first = PHASED && wave >= NWAVES / 2;   // wave-uniform
 
     // X: thread -> (row tid/8 of each pass, 16-byte column tid%8)
     const uint8_t* xsrc[XP];
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
-        const uint32_t m = min(m0 + i * 32u + (tid >> 3), p.M - 1u);
+        const uint32_t m = min(m0 + i * XROWS + (tid >> 3), p.M - 1u);
         xsrc[i] = (const uint8_t*)p.X + (size_t)m * p.K * 2u + (tid & 7u) * 16u;
     }
-    // W: item it -> row (tid + 256*it)/2, run (tid + 256*it)%2
+    // W: item it -> row (tid + NT*it)/2, run (tid + NT*it)%2
     const uint8_t* wsrc[WI];
     uint32_t wrow[WI], whf[WI];
 #pragma unroll
     for (int i = 0; i < WI; ++i) {
-        const uint32_t item = tid + 256u * i;
+        const uint32_t item = tid + NT * i;
         wrow[i] = item >> 1;
         whf[i] = item & 1u;
         wsrc[i] = p.W + (size_t)min(n0 + wrow[i], p.N - 1u) * p.row_stride_bytes;
@@ -195,7 +215,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmParams p)
         uint8_t* b = Bs + buf * B_BYTES;
 #pragma unroll
         for (int i = 0; i < XP; ++i)
-            *(u32x4*)(a + (i * 32u + (tid >> 3)) * GEMM_LD + (tid & 7u) * 16u) = xr[i];
+            *(u32x4*)(a + (i * XROWS + (tid >> 3)) * GEMM_LD + (tid & 7u) * 16u) = xr[i];
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
             uint8_t* dst = b + wrow[i] * GEMM_LD + whf[i] * 64u;
@@ -203,14 +223,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmParams p)
             else q6k_expand(w6[i], kt, whf[i], dst);
         }
     };
-
-    load_tile(0);
-    store_tile(0, 0);
-    __syncthreads();
-
-    for (uint32_t kt = 0; kt < nk; ++kt) {
-        const uint32_t buf = kt & 1u;
-        if (kt + 1 < nk) load_tile(kt + 1);
+    auto multiply = [&](uint32_t buf) {
         const uint8_t* a = As + buf * A_BYTES + (wm * WM + (lane & 31u)) * GEMM_LD + (lane >> 5) * 16u;
         const uint8_t* b = Bs + buf * B_BYTES + (wn * WN + (lane & 31u)) * GEMM_LD + (lane >> 5) * 16u;
 #pragma unroll
@@ -226,7 +239,23 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmParams p)
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < nk) store_tile(kt + 1, buf ^ 1u);
+    };
+
+    load_tile(0);
+    store_tile(0, 0);
+    if (convert_first && nk > 1) load_tile(1);
+    __syncthreads();
+
+    for (uint32_t kt = 0; kt < nk; ++kt) {
+        const uint32_t buf = kt & 1u;
+        if (convert_first) {
+            if (kt + 1 < nk) store_tile(kt + 1, buf ^ 1u);
+            if (kt + 2 < nk) load_tile(kt + 2);
+        } else {
+            if (kt + 1 < nk) load_tile(kt + 1);
+        }
+        multiply(buf);
+        if (!convert_first && kt + 1 < nk) store_tile(kt + 1, buf ^ 1u);
         __syncthreads();
     }
 
@@ -257,11 +286,11 @@ bool gemm_bf16_supported(const MatmulArgs& a)
     return true;
 }
 
-template <int TYPE, int BM, int BN>
+template <int TYPE, int BM, int BN, int NWAVES>
 static hipError_t launch_gemm(const GemmParams& p, hipStream_t s)
 {
     constexpr size_t shmem = 2 * (size_t)(BM + BN) * GEMM_LD;
-    auto kern = gemm_bf16_kernel<TYPE, BM, BN>;
+    auto kern = gemm_bf16_kernel<TYPE, BM, BN, NWAVES>;
     if (shmem > 64u * 1024u) {
         static bool raised = false;   // per instantiation
         if (!raised) {
@@ -271,7 +300,7 @@ static hipError_t launch_gemm(const GemmParams& p, hipStream_t s)
         }
     }
     dim3 grid((p.N + BN - 1) / BN, (p.M + BM - 1) / BM);
-    hipLaunchKernelGGL(kern, grid, dim3(256), shmem, s, p);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NWAVES), shmem, s, p);
     return hipGetLastError();
 }
 
@@ -290,8 +319,8 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, hipStream_t s)
     const uint64_t big = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 255u) / 256u);
     const bool use_big = tile == 256 || (tile == 0 && big >= 256u);
     const bool q4 = a.type == KQ_TYPE_Q4_K;
-    if (use_big) return q4 ? launch_gemm<KQ_TYPE_Q4_K, 256, 256>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 256, 256>(p, s);
-    return q4 ? launch_gemm<KQ_TYPE_Q4_K, 128, 128>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 128, 128>(p, s);
+    if (use_big) return q4 ? launch_gemm<KQ_TYPE_Q4_K, 256, 256, 8>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 256, 256, 8>(p, s);
+    return q4 ? launch_gemm<KQ_TYPE_Q4_K, 128, 128, 4>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 128, 128, 4>(p, s);
 }
 
 }  // namespace kq

@@ -56,6 +56,7 @@ __device__ __forceinline__ float wave_sum(float v)
     return (a + b) + (c + d);
 }
 
+// KQ_REQUIRES_NO_SPILL (the build refuses this file if any kernel in it spills).
 // Weight loads whose completion is waited for by hand.  The compiler's own
 // s_waitcnt placement drains the whole queue at the loop head when a register
 // ring is refilled inside a loop, which serialises fetch and arithmetic; these
@@ -64,28 +65,26 @@ __device__ __forceinline__ float wave_sum(float v)
 // ring_wait<N>() below (the "+v" operands make every later use depend on the
 // wait); (2) vector memory operations complete in issue order, so after
 // s_waitcnt vmcnt(N) every load but the N youngest has landed; (3) loads the
-// compiler does track only ever wait for more than they need.
+// compiler does track only ever wait for more than they need; (4) the
+// destination is an in/out operand, so a ring variable keeps its register from
+// one refill to the next, and the file is built with a check that nothing
+// spills: a register that was saved and reused before its load landed would
+// be overwritten by the late data.
 typedef uint32_t s_u32x2 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ s_u32x4 ring_load16(const uint8_t* ptr)
+__device__ __forceinline__ void ring_load16(s_u32x4& v, const uint8_t* ptr)
 {
-    s_u32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(ptr));
-    return v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(v) : "v"(ptr));
 }
 
-__device__ __forceinline__ s_u32x2 ring_load8(const uint8_t* ptr)
+__device__ __forceinline__ void ring_load8(s_u32x2& v, const uint8_t* ptr)
 {
-    s_u32x2 v;
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(ptr));
-    return v;
+    asm volatile("global_load_dwordx2 %0, %1, off" : "+v"(v) : "v"(ptr));
 }
 
-__device__ __forceinline__ uint32_t ring_load2(const uint8_t* ptr)
+__device__ __forceinline__ void ring_load2(uint32_t& v, const uint8_t* ptr)
 {
-    uint32_t v;
-    asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(ptr));
-    return v;
+    asm volatile("global_load_ushort %0, %1, off" : "+v"(v) : "v"(ptr));
 }
 
 // One lane's share of one pass of a Q4_K row.
@@ -140,8 +139,8 @@ struct Q4Slot {
     {
 #pragma unroll
         for (int pass = 0; pass < P; ++pass) {
-            hdr[pass] = ring_load16(row + hoff[pass]);
-            q[pass] = ring_load16(row + hoff[pass] + 16u + 16u * j);
+            ring_load16(hdr[pass], row + hoff[pass]);
+            ring_load16(q[pass], row + hoff[pass] + 16u + 16u * j);
         }
     }
     // Every register of the slot passes through the wait.
@@ -200,7 +199,7 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
     // fetched and summed again (cache hits, result dropped), so the row loop has
     // no branch and the number of loads in flight is the same at every wait.
     constexpr int SLOT_LOADS = 2 * P;
-    Q4Slot<P> ring[D];
+    Q4Slot<P> ring[D] = {};
 #pragma unroll
     for (int d = 0; d < D; ++d)
         ring[d].fill(p.W + (size_t)(gw + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, hoff, j);
@@ -256,11 +255,11 @@ struct Q6Slot {
 #pragma unroll
         for (int pass = 0; pass < P; ++pass) {
             const uint8_t* blk = row + boff[pass];
-            v[pass].a = ring_load8(blk + 64u * n + 8u * lg);
-            v[pass].b = ring_load8(blk + 64u * n + 32u + 8u * lg);
-            v[pass].h = ring_load8(blk + 128u + 32u * n + 8u * lg);
-            v[pass].sc = ring_load8(blk + 192u + 8u * n);
-            v[pass].d = ring_load2(blk + 208u);
+            ring_load8(v[pass].a, blk + 64u * n + 8u * lg);
+            ring_load8(v[pass].b, blk + 64u * n + 32u + 8u * lg);
+            ring_load8(v[pass].h, blk + 128u + 32u * n + 8u * lg);
+            ring_load8(v[pass].sc, blk + 192u + 8u * n);
+            ring_load2(v[pass].d, blk + 208u);
         }
     }
     template <int N>
@@ -363,7 +362,7 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
 
     if (n_rows == 0) return;   // whole workgroup
     constexpr int SLOT_LOADS = 5 * P;
-    Q6Slot<P> ring[D];
+    Q6Slot<P> ring[D] = {};
 #pragma unroll
     for (int d = 0; d < D; ++d)
         ring[d].fill(p.W + (size_t)(g + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, boff, n, lg);

@@ -47,6 +47,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--layers", type=int, default=32, help="layers in the set (32 = the named workload)")
     ap.add_argument("--prefill", action="store_true", help="also time the M=2048 prefill GEMM on one layer")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the M=2048 prefill GEMM leg and print its figures (for profiling)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run one 256 MiB device-to-device copy kernel: under rocprofv3 --pmc its "
                          "FETCH_SIZE / WRITE_SIZE readings give the counters' scale")
@@ -193,6 +195,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill_leg()}))
+        return
 
     mats = build_layer_set(args.layers)
     torch.cuda.synchronize()
