@@ -47,6 +47,11 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--layers", type=int, default=32, help="layers in the set (32 = the named workload)")
     ap.add_argument("--prefill", action="store_true", help="also time the M=2048 prefill GEMM on one layer")
+    ap.add_argument("--verify", action="store_true",
+                    help="also time the layer set at M = 2, 4, 8, 16 (speculative-decode verify batches)")
+    ap.add_argument("--moe", action="store_true",
+                    help="also time the Qwen3-30B-A3B-shaped routed-expert FFN at T = 1 and T = 256")
+    ap.add_argument("--all", action="store_true", help="--prefill --verify --moe")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the M=2048 prefill GEMM leg and print its figures (for profiling)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -251,13 +256,82 @@ def main():
         "roofline": roofline,
         "per_shape": shapes,
     }
-    if args.prefill:
+    if args.verify or args.all:
+        out["verify"] = verify_leg(mats, wb, use_graph)
+    if args.moe or args.all:
+        out["moe"] = moe_leg()
+    if args.prefill or args.all:
         out["prefill"] = prefill_leg()
+        out["prefill_m512"] = prefill_leg(512)
     if not args.no_cpu:
         del mats, dom
         torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
+
+
+def verify_leg(mats, wb, use_graph):
+    """The decode layer set at M = 2..16 tokens: the same weight bytes per step;
+    the aim is a step time that stays near the M = 1 time."""
+    import torch
+    from backpack_amd import capi
+    res = {}
+    for M in (2, 4, 8, 16):
+        xs, ys, ms = {}, {}, []
+        for name, w, x, y in mats:
+            if w.K not in xs:
+                xs[w.K] = torch.randn(M, w.K, device="cuda")
+            if w.N not in ys:
+                ys[w.N] = torch.empty(M, w.N, device="cuda")
+            ms.append((name, w, xs[w.K], ys[w.N]))
+        sec, _ = run_region(ms, 10, 2, use_graph)
+        act = sum((w.K + w.N) * 4 * M for _, w, _, _ in ms)
+        res[f"M{M}"] = {"ms_per_step": round(sec / 10 * 1e3, 4), "GBps": round((wb + act) / (sec / 10) / 1e9, 1),
+                        "kernel": capi.last_kernel()}
+    return res
+
+
+def moe_leg():
+    """Routed-expert FFN, Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048,
+    expert FFN 768, Q4_K gate/up and Q6_K down; one layer, T = 1 and T = 256.
+    Bytes = each touched expert's three matrices once."""
+    import torch
+    from backpack_amd import capi, kquant, synth
+    c = synth.QWEN3_30B_A3B
+    E, k, H, I = c["n_experts"], c["top_k"], c["hidden"], c["inter"]
+
+    def stacked(type_, N, K, seed):
+        data = synth.make_packed_device(type_, E * N, K, seed=seed)
+        return kquant.KQuantPacked(data, type_, E * N, K, synth.row_stride_words(type_, K), synth.n_blocks(K))
+    # several layers' worth of distinct expert stacks so that replays do not run from cache
+    layers = [(stacked(c["gate_up_type"], I, H, 10 + 3 * l), stacked(c["gate_up_type"], I, H, 11 + 3 * l),
+               stacked(c["down_type"], H, I, 12 + 3 * l)) for l in range(4)]
+    per_expert = 2 * synth.weight_bytes(c["gate_up_type"], I, H) + synth.weight_bytes(c["down_type"], H, I)
+    res = {}
+    g = torch.Generator(device="cpu").manual_seed(7)
+    for T in (1, 256):
+        idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).cuda()
+        wt = torch.softmax(torch.randn(T, k, generator=g), dim=-1).cuda()
+        x = torch.randn(T, H, device="cuda")
+        touched = int(torch.unique(idx).numel())
+        for gu, up, dn in layers:
+            kquant.moe_ffn(x, gu, up, dn, idx, wt, E)
+        torch.cuda.synchronize()
+        reps = 20
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for gu, up, dn in layers:
+                kquant.moe_ffn(x, gu, up, dn, idx, wt, E)
+        e1.record()
+        torch.cuda.synchronize()
+        sec = e0.elapsed_time(e1) * 1e-3 / (reps * len(layers))
+        nbytes = touched * per_expert
+        flops = 2.0 * T * k * 3 * H * I
+        res[f"T{T}"] = {"us_per_layer": round(sec * 1e6, 2), "experts_touched": touched, "weight_bytes": nbytes,
+                        "GBps": round(nbytes / sec / 1e9, 1), "TFLOPs": round(flops / sec / 1e12, 2),
+                        "kernel": capi.last_kernel()}
+    return res
 
 
 def prefill_leg(M=2048):
@@ -276,7 +350,7 @@ def prefill_leg(M=2048):
             kquant.matmul(x, w, out=y)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        reps = 5
+        reps = 20
         e0.record()
         for _ in range(reps):
             kquant.matmul(x, w, out=y)
