@@ -120,7 +120,7 @@ const char* bpk_last_kernel(void) { return t_kernel; }
 
 int bpk_force_kernel(int family)
 {
-    if (family < 0 || family > 5) return fail(BPK_ERR_SHAPE, "kernel family %d unknown", family);
+    if (family < 0 || family > 6) return fail(BPK_ERR_SHAPE, "kernel family %d unknown", family);
     t_family = family;
     return BPK_OK;
 }
@@ -282,6 +282,13 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     if (t_family == 2 && !rows_ok) return fail(BPK_ERR_SHAPE, "row-per-lane GEMV cannot serve this call");
     if (t_family == 3 && !mrow_ok) return fail(BPK_ERR_SHAPE, "matrix-core row kernel cannot serve this call");
     const bool stream_ok = kq::gemv_stream_supported(a);
+    const bool mtile_ok = kq::mtile_supported(a);
+    if (t_family == 6 && !mtile_ok) return fail(BPK_ERR_SHAPE, "16x16 tile kernel cannot serve this call");
+    if (t_family == 6 || (t_family == 0 && mtile_ok && M >= 3)) {
+        t_kernel = "mtile";
+        e = kq::launch_mtile(a, s);
+        return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+    }
     if (t_family == 5 && !stream_ok) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");
     if (t_family == 4) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
     // up to a few tens of thousands of rows the lanes-along-K kernel wins at M = 1

@@ -54,6 +54,10 @@ hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const G
 bool gemv_stream_supported(const MatmulArgs& a);
 hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStream_t s);
 
+// 16-row x 16-token MFMA tiles for M = 2..16 (dense): weights read once for all tokens.
+bool mtile_supported(const MatmulArgs& a);
+hipError_t launch_mtile(const MatmulArgs& a, hipStream_t s);
+
 // Row-per-lane matvec on the matrix cores, M <= 16 dense or grouped by expert.
 bool mrow_supported(const MatmulArgs& a);
 size_t mrow_scratch_floats(const MatmulArgs& a, const GemvTuning& t);

@@ -1,0 +1,438 @@
+// kq_mtile.hip — fused dequant-matmul for M = 2..16 tokens on the matrix cores,
+// tiles of 16 weight rows x 16 tokens (speculative-decode verify batches).
+//
+// v_mfma_f32_16x16x32_f16 multiplies a 16 x 32 block of activations (A, one
+// token per row) with a 32 x 16 block of weights (B, one weight row per column)
+// into a 16 x 16 fp32 tile.  Lane l of the wave holds, for both operands, eight
+// consecutive k (8*(l/16) .. +7) of token / weight row l%16, and of the result
+// the four tokens 4*(l/16) .. +3 of weight row l%16: a lane deals with a single
+// weight row, so block and sub-block scales are per-lane scalars.
+//
+// Weights.  The eight k of a lane are eight consecutive bytes of the block's
+// quants (one 64-bit load): their low nibbles belong to sub-block 2g, their
+// high nibbles to sub-block 2g+1.  A masked nibble left in the low mantissa
+// bits of an fp16 is the subnormal q * 2^-24 (q * 2^-20 four bits up), which
+// the matrix cores multiply exactly, so ten bit-ops per 8 bytes yield the B
+// operands of two sub-blocks.  Every weight byte is fetched once per launch and
+// used for all tokens.
+//
+// Activations.  fp32 X cannot go through fp16 unharmed, so a token's 256
+// elements of a superblock are scaled by a power of two that puts the largest
+// just below 2^15 and split into hi = fp16(x*s) and lo = fp16(x*s - hi), 22 bits
+// in all; each sub-block costs two MFMAs into the same accumulator.  The
+// workgroup converts a chunk of four superblocks of X at a time into LDS, in
+// operand order, together with the per-sub-block sums of x that the Q4_K minima
+// multiply.
+//
+// Q6_K.  Its scales cover 16 elements, half of one MFMA's k.  The token axis
+// pays for that: with at most 8 tokens, token m appears twice, as (m, first
+// half of k) in slot m and (m, second half) in slot m + 8, each with the other
+// half of its operand zeroed.  One MFMA then yields both 16-element sums, each
+// in lanes of its own that apply their own scale, and the two are added once
+// at the end.  (9..16 tokens are served as two calls of 8.)  The -32 offset of
+// the 6-bit values is applied against the sums of x over 16 elements.
+//
+// Work split.  A workgroup owns R tiles of 16 rows.  With R = NW every wave
+// owns a tile and walks all of K; with R = 1 (matrices of few rows) the waves of
+// the workgroup take different superblocks of the chunk and fold their partial
+// tiles through LDS at the end.  There is no fold across workgroups.
+#include "kq_format.h"
+#include "kq_kernels.h"
+
+namespace kq {
+
+typedef _Float16 t_half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 t_half2 __attribute__((ext_vector_type(2)));
+typedef float t_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t t_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t t_u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int MT_KC = 4;                       // superblocks of X staged at a time
+constexpr int MT_XA_BYTES = MT_KC * 8 * 2 * 1024;   // [block][sub-block][hi/lo][lane] 16 B
+constexpr int MT_XS_FLOATS = MT_KC * 8 * 16;        // [block][sub-block][token]
+constexpr int MT_INV_FLOATS = MT_KC * 16;           // [block][token]
+
+struct MtileParams {
+    const float* X;
+    const uint8_t* W;
+    const float* bias;
+    float* Y;
+    uint32_t M, N, K, n_blocks, row_stride_bytes, y_offset, ldy;
+    uint32_t tiles_per_wg;   // R == NW kernels: waves below this own a tile, the others only help convert X
+};
+
+// Conversion of a chunk's activations.  Thread (pair, sub) handles EPT
+// consecutive elements of one (token, superblock) pair; pairs are numbered
+// token-major, so a wave covers few tokens and waves whose tokens are all
+// beyond M have nothing to do after their slots were zeroed once.
+template <int NT, bool SPLIT16>
+struct MtileStager {
+    static constexpr int TPP = NT / (MT_KC * 16);   // threads per (token, block) pair
+    static constexpr int EPT = 256 / TPP;           // elements per thread: 64 or 32
+    static_assert(EPT == 64 || EPT == 32, "a thread converts one or two sub-blocks");
+    float4 v[EPT / 4];
+    uint32_t token, bb, sub;
+    bool live_token;
+
+    __device__ __forceinline__ void init(const MtileParams& p)
+    {
+        const uint32_t pair = threadIdx.x / TPP;
+        sub = threadIdx.x % TPP;
+        bb = pair % MT_KC;
+        token = pair / MT_KC;
+        live_token = token < p.M && (!SPLIT16 || token < 8u);
+    }
+    // requests the chunk's elements (nothing for tokens beyond M or superblocks beyond K)
+    __device__ __forceinline__ void fetch(const MtileParams& p, uint32_t c0)
+    {
+        const uint32_t b = c0 + bb;
+        const bool live = live_token && b < p.n_blocks;
+        const float4* src = (const float4*)(p.X + (size_t)(live ? token : 0u) * p.K + (size_t)(live ? b : 0u) * KQ_QK + sub * EPT);
+#pragma unroll
+        for (int i = 0; i < EPT / 4; ++i) v[i] = live ? src[i] : float4{0, 0, 0, 0};
+    }
+    // converts what fetch() brought and parks it in LDS (slots of tokens beyond M stay zero)
+    __device__ __forceinline__ void park(uint8_t* xa, float* xs, float* xinv)
+    {
+        if (!live_token) return;   // wave-uniform for whole waves of dead tokens
+        // largest magnitude of the pair's 256 elements, as float bits (orders like the floats)
+        uint32_t amax = 0;
+#pragma unroll
+        for (int i = 0; i < EPT / 4; ++i) {
+            amax = max(amax, __builtin_bit_cast(uint32_t, v[i].x) & 0x7FFFFFFFu);
+            amax = max(amax, __builtin_bit_cast(uint32_t, v[i].y) & 0x7FFFFFFFu);
+            amax = max(amax, __builtin_bit_cast(uint32_t, v[i].z) & 0x7FFFFFFFu);
+            amax = max(amax, __builtin_bit_cast(uint32_t, v[i].w) & 0x7FFFFFFFu);
+        }
+#pragma unroll
+        for (int off = 1; off < TPP; off <<= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, off, 64));
+        uint32_t e = amax >> 23;                  // biased exponent of the largest |x|
+        e = e < 15u ? 15u : (e > 253u ? 253u : e);
+        const float s = __builtin_bit_cast(float, (268u - e) << 23);     // 2^(141-e): amax*s in [2^14, 2^15)
+        const float inv = __builtin_bit_cast(float, (e - 14u) << 23);    // 2^(e-141)
+        if (sub == 0) {
+            xinv[bb * 16u + token] = inv;
+            if (SPLIT16) xinv[bb * 16u + token + 8u] = inv;
+        }
+        // groups of 8 consecutive k -> one operand slot: halves in the order k+0, k+2, k+1, k+3, k+4, k+6, k+5, k+7
+#pragma unroll
+        for (int g8 = 0; g8 < EPT / 8; ++g8) {
+            const float4 lo4 = v[2 * g8], hi4 = v[2 * g8 + 1];
+            const float a[8] = {lo4.x * s, lo4.y * s, lo4.z * s, lo4.w * s, hi4.x * s, hi4.y * s, hi4.z * s, hi4.w * s};
+            _Float16 h[8], l[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                h[i] = (_Float16)a[i];
+                l[i] = (_Float16)(a[i] - (float)h[i]);
+            }
+            const t_half8 hv = {h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+            const t_half8 lv = {l[0], l[2], l[1], l[3], l[4], l[6], l[5], l[7]};
+            const uint32_t k = sub * EPT + g8 * 8u;     // element of the superblock
+            const uint32_t sb = k >> 5, kq = (k >> 3) & 3u;
+            // SPLIT16: the first half of a 32-run goes to slot token, the second to slot token + 8
+            const uint32_t slot = SPLIT16 ? token + 8u * (kq >> 1) : token;
+            uint8_t* dst = xa + ((size_t)((bb * 8u + sb) * 2u) * 64u + slot + 16u * kq) * 16u;
+            *(t_half8*)dst = hv;
+            *(t_half8*)(dst + 1024) = lv;
+        }
+        // sums of the unscaled x over each run of 32 (or, SPLIT16, each half run of 16)
+#pragma unroll
+        for (int q = 0; q < EPT / 32; ++q) {
+            float h0 = 0.0f, h1 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                h0 += (v[8 * q + i].x + v[8 * q + i].y) + (v[8 * q + i].z + v[8 * q + i].w);
+                h1 += (v[8 * q + 4 + i].x + v[8 * q + 4 + i].y) + (v[8 * q + 4 + i].z + v[8 * q + 4 + i].w);
+            }
+            float* dst = xs + (bb * 8u + (sub * EPT) / 32u + q) * 16u + token;
+            if (SPLIT16) { dst[0] = h0; dst[8] = h1; }
+            else dst[0] = h0 + h1;
+        }
+    }
+};
+
+// One superblock of one 16-row tile: adds this block's contribution to tot[4]
+// (tokens 4*(lane/16) .. +3 of weight row lane%16).
+__device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2 (&w)[4], const uint8_t* xa_b,
+                                                const float* xs_b, const float* xinv_b, uint32_t lane,
+                                                t_f32x4& tot)
+{
+    const float d = half_bits_to_float(hdr.x & 0xFFFFu);
+    const float dmin = half_bits_to_float(hdr.x >> 16);
+    const uint32_t scA = hdr.y & 0x3F3F3F3Fu;
+    const uint32_t mnA = hdr.z & 0x3F3F3F3Fu;
+    const uint32_t scB = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    const uint32_t mnB = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    const uint32_t tq = lane >> 4;
+    t_f32x4 U = {0, 0, 0, 0}, V = {0, 0, 0, 0};
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const uint32_t d0 = w[g].x, d1 = w[g].y;
+        const uint32_t e0 = d0 >> 8, e1 = d1 >> 8;
+        const t_u32x4 blo = {d0 & 0x000F000Fu, e0 & 0x000F000Fu, d1 & 0x000F000Fu, e1 & 0x000F000Fu};
+        const t_u32x4 bhi = {d0 & 0x00F000F0u, e0 & 0x00F000F0u, d1 & 0x00F000F0u, e1 & 0x00F000F0u};
+#pragma unroll
+        for (int hn = 0; hn < 2; ++hn) {
+            const int sb = 2 * g + hn;
+            const uint8_t* ap = xa_b + ((size_t)(sb * 2) * 64u + lane) * 16u;
+            const t_half8 ahi = *(const t_half8*)ap;
+            const t_half8 alo = *(const t_half8*)(ap + 1024);
+            const t_half8 bq = __builtin_bit_cast(t_half8, hn ? bhi : blo);
+            t_f32x4 D = {0, 0, 0, 0};
+            D = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bq, D, 0, 0, 0);
+            D = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bq, D, 0, 0, 0);
+            const uint32_t scw = sb < 4 ? scA : scB, mnw = sb < 4 ? mnA : mnB;
+            // high nibbles sit four bits up: 1/16 goes into their scale
+            const float sc = (float)((scw >> (8 * (sb & 3))) & 255u) * (hn ? 0.0625f : 1.0f);
+            const float mn = (float)((mnw >> (8 * (sb & 3))) & 255u);
+            const float4 xsum = *(const float4*)(xs_b + sb * 16 + 4u * tq);
+            U.x = fmaf(sc, D.x, U.x); U.y = fmaf(sc, D.y, U.y); U.z = fmaf(sc, D.z, U.z); U.w = fmaf(sc, D.w, U.w);
+            V.x = fmaf(mn, xsum.x, V.x); V.y = fmaf(mn, xsum.y, V.y); V.z = fmaf(mn, xsum.z, V.z); V.w = fmaf(mn, xsum.w, V.w);
+        }
+    }
+    // D carries 2^-24 from the subnormal nibbles and the token's scale
+    const float4 inv = *(const float4*)(xinv_b + 4u * tq);
+    const float d24 = d * 16777216.0f;
+    tot.x += fmaf(d24 * inv.x, U.x, -(dmin * V.x));
+    tot.y += fmaf(d24 * inv.y, U.y, -(dmin * V.y));
+    tot.z += fmaf(d24 * inv.z, U.z, -(dmin * V.z));
+    tot.w += fmaf(d24 * inv.w, U.w, -(dmin * V.w));
+}
+
+// Q6_K: the weights of one superblock for one lane: 8 bytes of ql per (half, t&1), 8 of qh per half,
+// the 16 scales and d.
+struct Q6TileW {
+    t_u32x2 ql[2][2], qh[2];
+    t_u32x4 sc;
+    uint32_t d;
+};
+
+__device__ __forceinline__ void q6k_mtile_load(const uint8_t* blk, uint32_t kq, Q6TileW& w)
+{
+    // blocks are 210 bytes: these loads are 2-byte aligned, which the hardware accepts
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        __builtin_memcpy(&w.ql[h][0], blk + 64u * h + 8u * kq, 8);
+        __builtin_memcpy(&w.ql[h][1], blk + 64u * h + 32u + 8u * kq, 8);
+        __builtin_memcpy(&w.qh[h], blk + 128u + 32u * h + 8u * kq, 8);
+    }
+    __builtin_memcpy(&w.sc, blk + 192u, 16);
+    uint16_t d16;
+    __builtin_memcpy(&d16, blk + 208u, 2);
+    w.d = d16;
+}
+
+// One superblock of one 16-row tile, Q6_K.  Lanes 0..31 (tq < 2) hold the sums over the first
+// 16 elements of each run of 32 for tokens 4*tq .. +3, lanes 32..63 those over the second 16.
+__device__ __forceinline__ void q6k_mtile_block(const Q6TileW& w, const uint8_t* xa_b, const float* xs_b,
+                                                const float* xinv_b, uint32_t lane, t_f32x4& tot)
+{
+    const uint32_t tq = lane >> 4, u = tq >> 1;
+    t_f32x4 U = {0, 0, 0, 0}, V = {0, 0, 0, 0};
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        t_u32x4 bq[4];   // B operands of runs t = 0..3 of this half
+#pragma unroll
+        for (int wd = 0; wd < 2; ++wd) {
+            const uint32_t A = w.ql[h][0][wd], B = w.ql[h][1][wd], H = w.qh[h][wd];
+            const uint32_t A8 = A >> 8, B8 = B >> 8;
+            const uint32_t Hl4 = H << 4, Hl2 = H << 2, Hr4 = H >> 4, Hr6 = H >> 6;
+            // pair a: bytes 0, 2; pair b: bytes 1, 3 of the word
+            bq[0][2 * wd] = (A & 0x000F000Fu) | (Hl4 & 0x00300030u);
+            bq[0][2 * wd + 1] = (A8 & 0x000F000Fu) | (Hr4 & 0x00300030u);
+            bq[1][2 * wd] = (B & 0x000F000Fu) | (Hl2 & 0x00300030u);
+            bq[1][2 * wd + 1] = (B8 & 0x000F000Fu) | (Hr6 & 0x00300030u);
+            bq[2][2 * wd] = (A & 0x00F000F0u) | (Hl4 & 0x03000300u);
+            bq[2][2 * wd + 1] = (A8 & 0x00F000F0u) | (Hr4 & 0x03000300u);
+            bq[3][2 * wd] = (B & 0x00F000F0u) | (Hl2 & 0x03000300u);
+            bq[3][2 * wd + 1] = (B8 & 0x00F000F0u) | (Hr6 & 0x03000300u);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int run = 4 * h + t;
+            const uint8_t* ap = xa_b + ((size_t)(run * 2) * 64u + lane) * 16u;
+            const t_half8 ahi = *(const t_half8*)ap;
+            const t_half8 alo = *(const t_half8*)(ap + 1024);
+            const t_half8 b8 = __builtin_bit_cast(t_half8, bq[t]);
+            t_f32x4 D = {0, 0, 0, 0};
+            D = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, b8, D, 0, 0, 0);
+            D = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, b8, D, 0, 0, 0);
+            // scale of (half h, t, 16-element half u): byte 8h + 2t + u of the 16
+            const uint32_t word = w.sc[(8 * h + 2 * t) >> 2];
+            const uint32_t sh = 8u * ((2u * t) & 3u) + 8u * u;
+            const float scv = (float)(int)(int8_t)((word >> sh) & 255u);
+            const float sc = scv * (t >= 2 ? 0.0625f : 1.0f);   // t >= 2: the field sits four bits up
+            const float4 xsum = *(const float4*)(xs_b + run * 16 + 4u * tq);
+            U.x = fmaf(sc, D.x, U.x); U.y = fmaf(sc, D.y, U.y); U.z = fmaf(sc, D.z, U.z); U.w = fmaf(sc, D.w, U.w);
+            V.x = fmaf(scv, xsum.x, V.x); V.y = fmaf(scv, xsum.y, V.y); V.z = fmaf(scv, xsum.z, V.z); V.w = fmaf(scv, xsum.w, V.w);
+        }
+    }
+    const float4 inv = *(const float4*)(xinv_b + 4u * tq);
+    const float d = half_bits_to_float(w.d);
+    const float d24 = d * 16777216.0f, d32 = d * 32.0f;
+    tot.x += fmaf(d24 * inv.x, U.x, -(d32 * V.x));
+    tot.y += fmaf(d24 * inv.y, U.y, -(d32 * V.y));
+    tot.z += fmaf(d24 * inv.z, U.z, -(d32 * V.z));
+    tot.w += fmaf(d24 * inv.w, U.w, -(d32 * V.w));
+}
+
+template <int TYPE, int NW, int R>
+__global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
+{
+    static_assert(R == NW || R == 1, "a wave owns a tile, or all waves share one");
+    extern __shared__ __align__(16) uint8_t smem[];
+    uint8_t* xa = smem;
+    float* xs = (float*)(smem + MT_XA_BYTES);
+    float* xinv = xs + MT_XS_FLOATS;
+    float* red = (float*)smem;   // reused after the last chunk
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const bool has_tile = R == 1 || wave < p.tiles_per_wg;
+    const uint32_t tile = R == 1 ? blockIdx.x : blockIdx.x * p.tiles_per_wg + wave;
+    const uint32_t row = has_tile ? tile * 16u + (lane & 15u) : p.N;
+    const uint32_t kq = lane >> 4;
+    const uint8_t* wrow = p.W + (size_t)min(row, p.N - 1u) * p.row_stride_bytes;
+    // superblocks of a chunk this wave takes: all (R == NW), or wave, wave + NW, ... (R == 1)
+    constexpr int BPC = R == 1 ? (MT_KC + NW - 1) / NW : MT_KC;
+
+    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
+    constexpr uint32_t BB = Q6 ? KQ_Q6K_BYTES : KQ_Q4K_BYTES;
+    MtileStager<64 * NW, Q6> stager;
+    stager.init(p);
+    stager.fetch(p, 0);
+    // slots of tokens beyond M, and for Q6_K the halves that must read as zero, are cleared once
+    for (uint32_t i = threadIdx.x; i < (MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4) / 16; i += 64 * NW)
+        ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
+    __syncthreads();
+
+    t_f32x4 tot = {0, 0, 0, 0};
+    for (uint32_t c0 = 0; c0 < p.n_blocks; c0 += MT_KC) {
+        // the chunk's weights are requested first, so that their latency runs
+        // under the conversion of X
+        t_u32x4 hdr[BPC];
+        t_u32x2 w[BPC][4];
+        Q6TileW w6[BPC];
+#pragma unroll
+        for (int i = 0; i < BPC; ++i) {
+            const uint32_t bb = R == 1 ? wave + i * NW : i;
+            const uint32_t b = min(c0 + bb, p.n_blocks - 1u);
+            const uint8_t* blk = wrow + (size_t)b * BB;
+            if constexpr (Q6) {
+                q6k_mtile_load(blk, kq, w6[i]);
+            } else {
+                hdr[i] = *(const t_u32x4*)blk;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) w[i][g] = *(const t_u32x2*)(blk + 16u + 32u * g + 8u * kq);
+            }
+        }
+        stager.park(xa, xs, xinv);
+        __syncthreads();
+        // the next chunk of X travels while this one is multiplied
+        if (c0 + MT_KC < p.n_blocks) stager.fetch(p, c0 + MT_KC);
+        if (has_tile) {
+#pragma unroll
+            for (int i = 0; i < BPC; ++i) {
+                const uint32_t bb = R == 1 ? wave + i * NW : i;
+                if (bb < MT_KC && c0 + bb < p.n_blocks) {
+                    if constexpr (Q6)
+                        q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                    else
+                        q4k_mtile_block(hdr[i], w[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    if (R == 1) {
+        // fold the waves' partial tiles in wave order
+        *(t_f32x4*)(red + (wave * 64u + lane) * 4u) = tot;
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int w2 = 1; w2 < NW; ++w2) {
+            const t_f32x4 o = *(const t_f32x4*)(red + (w2 * 64u + lane) * 4u);
+            tot.x += o.x; tot.y += o.y; tot.z += o.z; tot.w += o.w;
+        }
+    }
+    if constexpr (Q6) {
+        // lanes l and l + 32 hold the two 16-element halves of tokens 4*(l/16) .. +3: add them
+        tot.x += __shfl_xor(tot.x, 32, 64);
+        tot.y += __shfl_xor(tot.y, 32, 64);
+        tot.z += __shfl_xor(tot.z, 32, 64);
+        tot.w += __shfl_xor(tot.w, 32, 64);
+    }
+    if (row < p.N && (!Q6 || kq < 2u)) {
+        const float bias = p.bias ? p.bias[row] : 0.0f;
+        const float t4[4] = {tot.x, tot.y, tot.z, tot.w};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t token = 4u * kq + r;
+            if (token < p.M) p.Y[(size_t)token * p.ldy + p.y_offset + row] = t4[r] + bias;
+        }
+    }
+}
+
+bool mtile_supported(const MatmulArgs& a)
+{
+    if (a.expert_idx) return false;
+    if (a.M < 1 || a.M > 16) return false;
+    if (((uintptr_t)a.X & 15u)) return false;
+    if (a.type == KQ_TYPE_Q4_K) return !(((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u));
+    if (a.type == KQ_TYPE_Q6_K) return !(((uintptr_t)a.W & 1u) || (a.row_stride_bytes & 1u));
+    return false;
+}
+
+template <int TYPE, int NW, int R>
+static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, hipStream_t s)
+{
+    constexpr size_t shmem = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * sizeof(float);
+    auto kern = mtile_kernel<TYPE, NW, R>;
+    static bool raised = false;   // per instantiation
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * NW), shmem, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_mtile(const MatmulArgs& a, hipStream_t s)
+{
+    const bool q6 = a.type == KQ_TYPE_Q6_K;
+    // Q6_K tiles hold 8 tokens: more are served in groups of 8, each reading the weights again
+    const uint32_t group = q6 ? 8u : 16u;
+    const uint32_t tiles = (a.N + 15u) / 16u;
+    for (uint32_t m0 = 0; m0 < a.M; m0 += group) {
+        MtileParams p;
+        p.X = (const float*)a.X + (size_t)m0 * a.K;
+        p.W = a.W;
+        p.bias = a.bias;
+        p.Y = a.Y + (size_t)m0 * a.ldy;
+        p.M = a.M - m0 < group ? a.M - m0 : group;
+        p.N = a.N; p.K = a.K;
+        p.n_blocks = a.n_blocks;
+        p.row_stride_bytes = a.row_stride_bytes;
+        p.y_offset = a.y_offset;
+        p.ldy = a.ldy;
+        p.tiles_per_wg = 1;
+        hipError_t e;
+        // a wave per tile once that still gives a couple of hundred workgroups; otherwise one tile per workgroup
+        if (tiles >= 7u * 200u) {
+            // 7 or 8 tiles per workgroup, whichever leaves the last round of workgroups fuller on 256 CUs
+            const uint32_t w7 = (tiles + 6u) / 7u, w8 = (tiles + 7u) / 8u;
+            const uint32_t fill7 = (w7 + 255u) / 256u * 256u - w7, fill8 = (w8 + 255u) / 256u * 256u - w8;
+            p.tiles_per_wg = fill7 * 7u < fill8 * 8u ? 7u : 8u;
+            const uint32_t wgs = (tiles + p.tiles_per_wg - 1u) / p.tiles_per_wg;
+            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8>(p, wgs, s) : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8>(p, wgs, s);
+        } else {
+            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 4, 1>(p, tiles, s) : launch_mtile_one<KQ_TYPE_Q4_K, 4, 1>(p, tiles, s);
+        }
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+}  // namespace kq

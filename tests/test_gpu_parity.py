@@ -91,6 +91,12 @@ def test_reference_recipe(gpu, kqo, name, family):
 
 
 # ---- matmul against the oracle ------------------------------------------------------
+# Extra distance from the exact contraction allowed on top of twice the CPU path's own, in
+# units of the output rms: VALU kernels accumulate like the CPU; the matrix-core kernels feed
+# activations as fp16 hi + lo (22 bits relative to the largest element of the token's
+# superblock) and the MFMA adds its products with about 2^-19 relative alignment loss.
+SLACK = {"mrow": 1e-5, "mrow_grouped": 1e-5, "mtile": 2e-5}
+
 SHAPES = [
     # type, M, N, K
     (Q4_K, 1, 4096, 4096),      # one decode projection (config 0)
@@ -114,11 +120,17 @@ SHAPES = [
     (Q4_K, 7, 300, 4096),
     (Q4_K, 12, 64, 768),
     (Q6_K, 3, 2048, 768),       # the MoE down projection: odd block count, 632-byte rows
+    (Q4_K, 16, 2000, 4096),     # tile kernel, one tile per workgroup, ragged last tile
+    (Q4_K, 9, 2300, 1280),      # ... with a partial last chunk of superblocks (5 blocks)
+    (Q6_K, 8, 2000, 4096),
+    (Q6_K, 13, 1800, 1536),     # Q6_K beyond 8 tokens: two groups; 6 blocks
+    (Q4_K, 16, 22500, 512),     # tile kernel, a wave per tile (7 or 8 tiles per workgroup), ragged last tile
+    (Q6_K, 5, 23001, 768),
 ]
 
 
 @pytest.mark.parametrize("type_,M,N,K", SHAPES)
-@pytest.mark.parametrize("family", [0, 1, 2, 3, 5])
+@pytest.mark.parametrize("family", [0, 1, 2, 3, 5, 6])
 def test_matmul_vs_oracle(gpu, kqo, type_, M, N, K, family):
     from backpack_amd import capi, kquant
     raw, packed, w = gpu.make_weight(type_, N, K, seed=N + K)
@@ -137,7 +149,7 @@ def test_matmul_vs_oracle(gpu, kqo, type_, M, N, K, family):
     finally:
         capi.force_kernel(0)
     r = gpu.check_matmul(kqo, type_, got, X, packed, N, K, bias=bias, label=f"{kern} {type_} {M}x{N}x{K}",
-                         slack=1e-5 if kern == "mrow" else 1e-6)
+                         slack=SLACK.get(kern, 1e-6))
     _say("   kernel", kern, r)
 
 
