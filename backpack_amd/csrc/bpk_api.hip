@@ -373,7 +373,19 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
     hipStream_t s = (hipStream_t)stream;
     const int sets = kq::moe_sets_for(T * k, n_experts);
     hipError_t e;
-    if (t_family != 1 && kq::mrow_supported(a) && n_experts <= 8192u &&
+    // two or more pairs per expert on average: records of 8 pairs on the 16x16 tile kernel
+    const bool tile_path = (t_family == 0 || t_family == 6) && kq::mtile_supported(a) && N >= 128u &&
+                           (uint64_t)T * k >= 2ull * n_experts && n_experts <= 8192u &&
+                           kq::moe_tiles_bound(T * k, n_experts, 4) <= 65535u &&
+                           kq::moe_tiles_words(T * k, n_experts, 4) <= kMoeWords;
+    if (tile_path) {
+        t_kernel = "mtile_grouped";
+        uint32_t* n_tiles = st->moe_tiles;
+        uint32_t* tiles = st->moe_tiles + 1;
+        e = kq::launch_moe_group(expert_idx, T * k, n_experts, 4, tiles, n_tiles, s);
+        if (e == hipSuccess)
+            e = kq::launch_mtile_grouped(a, tiles, n_tiles, kq::moe_tiles_bound(T * k, n_experts, 4), 8, s);
+    } else if (t_family != 1 && kq::mrow_supported(a) && n_experts <= 8192u &&
         kq::moe_tiles_bound(T * k, n_experts, sets) <= 65535u &&
         kq::moe_tiles_words(T * k, n_experts, sets) <= kMoeWords) {
         t_kernel = "mrow_grouped";
@@ -438,7 +450,20 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
     const bool fast = t_family != 1 && n_experts <= 8192u && bound <= 65535u && kq::mrow_supported(a) &&
                       kq::mrow_supported(d);
     hipError_t e = hipSuccess;
-    if (fast) {
+    const uint32_t bound8 = kq::moe_tiles_bound(P, n_experts, 4);
+    const bool tile_path = (t_family == 0 || t_family == 6) && n_experts <= 8192u && bound8 <= 65535u &&
+                           (uint64_t)P >= 2ull * n_experts && inter >= 128u && hidden >= 128u &&
+                           kq::mtile_supported(a) && kq::mtile_supported(d);
+    if (tile_path) {
+        // two or more pairs per expert on average: records of 8 pairs, every expert matrix read once per record
+        t_kernel = "moe_ffn_mtile";
+        e = kq::launch_moe_group(expert_idx, P, n_experts, 4, tiles, n_tiles, s);
+        if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, bound8, 8, s);
+        a.W = (const uint8_t*)up; a.Y = U;
+        if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, bound8, 8, s);
+        if (e == hipSuccess) e = kq::launch_moe_silu_mul(G, U, G, (size_t)P * inter, s);
+        if (e == hipSuccess) e = kq::launch_mtile_grouped(d, tiles, n_tiles, bound8, 8, s);
+    } else if (fast) {
         t_kernel = "moe_ffn_mrow";
         e = kq::launch_moe_group(expert_idx, P, n_experts, sets, tiles, n_tiles, s);
         if (e == hipSuccess) e = kq::launch_mrow(a, st->split, t_gemv, tiles, n_tiles, bound, sets, s);

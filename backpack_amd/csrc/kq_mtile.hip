@@ -59,6 +59,13 @@ struct MtileParams {
     float* Y;
     uint32_t M, N, K, n_blocks, row_stride_bytes, y_offset, ldy;
     uint32_t tiles_per_wg;   // R == NW kernels: waves below this own a tile, the others only help convert X
+    // grouped mode (tiles != nullptr): blockIdx.y walks records {expert, count, pair ids...} of up to
+    // 16 (Q4_K) / 8 (Q6_K) (token, slot) pairs that share an expert; N is the rows of one expert
+    const uint32_t* tiles;
+    const uint32_t* n_tiles;
+    uint32_t tile_stride;   // words per record
+    uint32_t k_slots;
+    int x_per_slot;         // X row of a pair: the pair itself (1) or its token, pair / k_slots (0)
 };
 
 // Conversion of a chunk's activations.  Thread (pair, sub) handles EPT
@@ -74,20 +81,26 @@ struct MtileStager {
     uint32_t token, bb, sub;
     bool live_token;
 
-    __device__ __forceinline__ void init(const MtileParams& p)
+    uint32_t xrow;   // row of X this thread converts
+    __device__ __forceinline__ void init(const MtileParams& p, const uint32_t* rec, uint32_t count)
     {
         const uint32_t pair = threadIdx.x / TPP;
         sub = threadIdx.x % TPP;
         bb = pair % MT_KC;
         token = pair / MT_KC;
-        live_token = token < p.M && (!SPLIT16 || token < 8u);
+        live_token = token < count && (!SPLIT16 || token < 8u);
+        xrow = token;
+        if (rec && live_token) {
+            const uint32_t pr = rec[2u + token];
+            xrow = p.x_per_slot ? pr : pr / p.k_slots;
+        }
     }
     // requests the chunk's elements (nothing for tokens beyond M or superblocks beyond K)
     __device__ __forceinline__ void fetch(const MtileParams& p, uint32_t c0)
     {
         const uint32_t b = c0 + bb;
         const bool live = live_token && b < p.n_blocks;
-        const float4* src = (const float4*)(p.X + (size_t)(live ? token : 0u) * p.K + (size_t)(live ? b : 0u) * KQ_QK + sub * EPT);
+        const float4* src = (const float4*)(p.X + (size_t)(live ? xrow : 0u) * p.K + (size_t)(live ? b : 0u) * KQ_QK + sub * EPT);
 #pragma unroll
         for (int i = 0; i < EPT / 4; ++i) v[i] = live ? src[i] : float4{0, 0, 0, 0};
     }
@@ -288,18 +301,28 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // grouped mode: this workgroup's tokens are the pairs of one record, its weights one expert's rows
+    const uint32_t* rec = nullptr;
+    uint32_t count = p.M;
+    const uint8_t* wmat = p.W;
+    if (p.tiles) {
+        if (blockIdx.y >= *p.n_tiles) return;   // whole workgroup
+        rec = p.tiles + (size_t)blockIdx.y * p.tile_stride;
+        count = rec[1];
+        wmat += (size_t)rec[0] * p.N * p.row_stride_bytes;
+    }
     const bool has_tile = R == 1 || wave < p.tiles_per_wg;
     const uint32_t tile = R == 1 ? blockIdx.x : blockIdx.x * p.tiles_per_wg + wave;
     const uint32_t row = has_tile ? tile * 16u + (lane & 15u) : p.N;
     const uint32_t kq = lane >> 4;
-    const uint8_t* wrow = p.W + (size_t)min(row, p.N - 1u) * p.row_stride_bytes;
+    const uint8_t* wrow = wmat + (size_t)min(row, p.N - 1u) * p.row_stride_bytes;
     // superblocks of a chunk this wave takes: all (R == NW), or wave, wave + NW, ... (R == 1)
     constexpr int BPC = R == 1 ? (MT_KC + NW - 1) / NW : MT_KC;
 
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
     constexpr uint32_t BB = Q6 ? KQ_Q6K_BYTES : KQ_Q4K_BYTES;
     MtileStager<64 * NW, Q6> stager;
-    stager.init(p);
+    stager.init(p, rec, count);
     stager.fetch(p, 0);
     // slots of tokens beyond M, and for Q6_K the halves that must read as zero, are cleared once
     for (uint32_t i = threadIdx.x; i < (MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4) / 16; i += 64 * NW)
@@ -369,15 +392,17 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const uint32_t token = 4u * kq + r;
-            if (token < p.M) p.Y[(size_t)token * p.ldy + p.y_offset + row] = t4[r] + bias;
+            if (token < count) {
+                const uint32_t yrow = rec ? rec[2u + token] : token;
+                p.Y[(size_t)yrow * p.ldy + p.y_offset + row] = t4[r] + bias;
+            }
         }
     }
 }
 
 bool mtile_supported(const MatmulArgs& a)
 {
-    if (a.expert_idx) return false;
-    if (a.M < 1 || a.M > 16) return false;
+    if (!a.expert_idx && (a.M < 1 || a.M > 16)) return false;   // grouped calls bring their tokens in records
     if (((uintptr_t)a.X & 15u)) return false;
     if (a.type == KQ_TYPE_Q4_K) return !(((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u));
     if (a.type == KQ_TYPE_Q6_K) return !(((uintptr_t)a.W & 1u) || (a.row_stride_bytes & 1u));
@@ -385,7 +410,7 @@ bool mtile_supported(const MatmulArgs& a)
 }
 
 template <int TYPE, int NW, int R>
-static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, hipStream_t s)
+static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s)
 {
     constexpr size_t shmem = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * sizeof(float);
     auto kern = mtile_kernel<TYPE, NW, R>;
@@ -395,8 +420,37 @@ static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, hipStream
         if (e != hipSuccess) return e;
         raised = true;
     }
-    hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * NW), shmem, s, p);
+    hipLaunchKernelGGL(kern, dim3(wgs, wgs_y), dim3(64 * NW), shmem, s, p);
     return hipGetLastError();
+}
+
+uint32_t mtile_group_cap(int type) { return type == KQ_TYPE_Q6_K ? 8u : 16u; }
+
+hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, const uint32_t* n_tiles,
+                                uint32_t tiles_bound, uint32_t cap, hipStream_t s)
+{
+    if (cap > mtile_group_cap(a.type) || tiles_bound == 0 || tiles_bound > 65535u) return hipErrorInvalidValue;
+    MtileParams p;
+    p.X = (const float*)a.X;
+    p.W = a.W;
+    p.bias = nullptr;
+    p.Y = a.Y;
+    p.M = cap; p.N = a.N; p.K = a.K;
+    p.n_blocks = a.n_blocks;
+    p.row_stride_bytes = a.row_stride_bytes;
+    p.y_offset = 0;
+    p.ldy = a.ldy;
+    p.tiles = tiles;
+    p.n_tiles = n_tiles;
+    p.tile_stride = 2u + cap;
+    p.k_slots = a.k_slots;
+    p.x_per_slot = a.x_per_slot;
+    // a wave per 16-row tile of the expert, 8 tiles per workgroup: X of the record is converted once per 128 rows
+    p.tiles_per_wg = 8;
+    const uint32_t row_tiles = (a.N + 15u) / 16u;
+    const uint32_t wgs = (row_tiles + 7u) / 8u;
+    return a.type == KQ_TYPE_Q6_K ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8>(p, wgs, tiles_bound, s)
+                                  : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8>(p, wgs, tiles_bound, s);
 }
 
 hipError_t launch_mtile(const MatmulArgs& a, hipStream_t s)
@@ -418,6 +472,7 @@ hipError_t launch_mtile(const MatmulArgs& a, hipStream_t s)
         p.y_offset = a.y_offset;
         p.ldy = a.ldy;
         p.tiles_per_wg = 1;
+        p.tiles = nullptr; p.n_tiles = nullptr; p.tile_stride = 0; p.k_slots = 1; p.x_per_slot = 0;
         hipError_t e;
         // a wave per tile once that still gives a couple of hundred workgroups; otherwise one tile per workgroup
         if (tiles >= 7u * 200u) {
@@ -426,9 +481,9 @@ hipError_t launch_mtile(const MatmulArgs& a, hipStream_t s)
             const uint32_t fill7 = (w7 + 255u) / 256u * 256u - w7, fill8 = (w8 + 255u) / 256u * 256u - w8;
             p.tiles_per_wg = fill7 * 7u < fill8 * 8u ? 7u : 8u;
             const uint32_t wgs = (tiles + p.tiles_per_wg - 1u) / p.tiles_per_wg;
-            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8>(p, wgs, s) : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8>(p, wgs, s);
+            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8>(p, wgs, 1, s) : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8>(p, wgs, 1, s);
         } else {
-            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 4, 1>(p, tiles, s) : launch_mtile_one<KQ_TYPE_Q4_K, 4, 1>(p, tiles, s);
+            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 4, 1>(p, tiles, 1, s) : launch_mtile_one<KQ_TYPE_Q4_K, 4, 1>(p, tiles, 1, s);
         }
         if (e != hipSuccess) return e;
     }

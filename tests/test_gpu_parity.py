@@ -348,9 +348,9 @@ def _routing(rng, T, E, k):
     return eidx, ew
 
 
-@pytest.mark.parametrize("family", [0, 1])
+@pytest.mark.parametrize("family", [0, 1, 3])
 @pytest.mark.parametrize("T,E,k,H,I", [(1, 8, 2, 512, 512), (5, 6, 3, 512, 768), (40, 16, 4, 512, 512),
-                                       (3, 4, 2, 512, 256)])
+                                       (3, 4, 2, 512, 256), (70, 5, 4, 768, 512)])
 def test_moe_ffn_vs_oracle(gpu, kqo, family, T, E, k, H, I):
     from backpack_amd import capi, kquant
     _say("moe_ffn", T, E, k, H, I, "family", family)
@@ -366,8 +366,15 @@ def test_moe_ffn_vs_oracle(gpu, kqo, family, T, E, k, H, I):
         kern = capi.last_kernel()
     finally:
         capi.force_kernel(0)
-    # a single-block Q6_K down projection (inter = 256) is outside the row kernel's reach
-    assert kern == ("moe_ffn_generic" if family == 1 or I == 256 else "moe_ffn_mrow")
+    # two or more pairs per expert on average go to the 16x16 tile kernel (family 3 keeps them on the
+    # row kernel); a single-block Q6_K down projection (inter = 256) is outside the row kernel's reach
+    if family == 1:
+        expect = "moe_ffn_generic"
+    elif family == 0 and T * k >= 2 * E:
+        expect = "moe_ffn_mtile"
+    else:
+        expect = "moe_ffn_generic" if I == 256 else "moe_ffn_mrow"
+    assert kern == expect, (kern, expect)
     want = kqo.moe_ffn(Q4_K, Q6_K, X, gp, up, dp, eidx, ew, H, I)
     rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
     err = np.abs(got - want)
@@ -394,7 +401,7 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
         X = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
         xd, ed, wd = gpu.dev(X), gpu.dev(eidx.view(np.int32)), gpu.dev(ew)
         got = kquant.moe_ffn(xd, gw, uw, dw, ed, wd, E).cpu().numpy()
-        assert capi.last_kernel() == "moe_ffn_mrow"
+        assert capi.last_kernel() == ("moe_ffn_mrow" if T == 1 else "moe_ffn_mtile")
         sel = np.arange(T) if T == 1 else np.array([0, 100, 101, 255])
         want = kqo.moe_ffn(Q4_K, Q6_K, X[sel], gp, up, dp, eidx[sel], ew[sel], H, I)
         rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
@@ -408,10 +415,18 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
             assert np.all(np.abs(got - ref) <= 1e-3 * rms + 1e-3 * np.abs(ref))
             again = kquant.moe_ffn(xd, gw, uw, dw, ed, wd, E).cpu().numpy()
             assert np.array_equal(got, again), "grouped path must not depend on bucket fill order"
+            capi.force_kernel(3)   # the row kernel's grouped mode on the same routing
+            try:
+                rowk = kquant.moe_ffn(xd, gw, uw, dw, ed, wd, E).cpu().numpy()
+                assert capi.last_kernel() == "moe_ffn_mrow"
+            finally:
+                capi.force_kernel(0)
+            assert np.all(np.abs(rowk - ref) <= 1e-3 * rms + 1e-3 * np.abs(ref))
 
 
+@pytest.mark.parametrize("family,kernel", [(0, "mtile_grouped"), (3, "mrow_grouped")])
 @pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True)])
-def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot):
+def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot, family, kernel):
     """Ragged lists: some experts get many pairs, some none; repeated experts inside a token."""
     from backpack_amd import capi, kquant
     E, T, k = 12, 37, 4
@@ -419,8 +434,12 @@ def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot):
     rng = np.random.default_rng(62)
     eidx = rng.choice([0, 1, 1, 1, 5, 5, 7, 11], size=(T, k)).astype(np.uint32)   # experts 2,3,4,6,8,9,10 idle
     X = rng.standard_normal((T * k if per_slot else T, K)).astype(np.float32)
-    got = kquant.moe_matmul(gpu.dev(X), w, gpu.dev(eidx.view(np.int32)), E, x_per_slot=per_slot).cpu().numpy()
-    assert capi.last_kernel() == "mrow_grouped"
+    capi.force_kernel(family)
+    try:
+        got = kquant.moe_matmul(gpu.dev(X), w, gpu.dev(eidx.view(np.int32)), E, x_per_slot=per_slot).cpu().numpy()
+        assert capi.last_kernel() == kernel
+    finally:
+        capi.force_kernel(0)
     want = kqo.moe_matmul(type_, X, packed, eidx, N, K, x_per_slot=per_slot)
     rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
     assert np.all(np.abs(got - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
