@@ -378,7 +378,13 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
                            (uint64_t)T * k >= 2ull * n_experts && n_experts <= 8192u &&
                            kq::moe_tiles_bound(T * k, n_experts, 4) <= 65535u &&
                            kq::moe_tiles_words(T * k, n_experts, 4) <= kMoeWords;
-    if (tile_path) {
+    // a handful of pairs (decode): one lanes-along-K matvec per pair, no grouping pass
+    const bool stream_path = (t_family == 0 || t_family == 5) && !tile_path && (uint64_t)T * k <= 64u &&
+                             kq::gemv_stream_supported(a);
+    if (stream_path) {
+        t_kernel = "stream_grouped";
+        e = kq::launch_gemv_stream(a, t_gemv, s);
+    } else if (tile_path) {
         t_kernel = "mtile_grouped";
         uint32_t* n_tiles = st->moe_tiles;
         uint32_t* tiles = st->moe_tiles + 1;
@@ -454,7 +460,17 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
     const bool tile_path = (t_family == 0 || t_family == 6) && n_experts <= 8192u && bound8 <= 65535u &&
                            (uint64_t)P >= 2ull * n_experts && inter >= 128u && hidden >= 128u &&
                            kq::mtile_supported(a) && kq::mtile_supported(d);
-    if (tile_path) {
+    const bool stream_path = (t_family == 0 || t_family == 5) && !tile_path && P <= 64u &&
+                             kq::gemv_stream_supported(a) && kq::gemv_stream_supported(d);
+    if (stream_path) {
+        // a handful of pairs (decode): one lanes-along-K matvec per pair, no grouping pass
+        t_kernel = "moe_ffn_stream";
+        e = kq::launch_gemv_stream(a, t_gemv, s);
+        a.W = (const uint8_t*)up; a.Y = U;
+        if (e == hipSuccess) e = kq::launch_gemv_stream(a, t_gemv, s);
+        if (e == hipSuccess) e = kq::launch_moe_silu_mul(G, U, G, (size_t)P * inter, s);
+        if (e == hipSuccess) e = kq::launch_gemv_stream(d, t_gemv, s);
+    } else if (tile_path) {
         // two or more pairs per expert on average: records of 8 pairs, every expert matrix read once per record
         t_kernel = "moe_ffn_mtile";
         e = kq::launch_moe_group(expert_idx, P, n_experts, 4, tiles, n_tiles, s);

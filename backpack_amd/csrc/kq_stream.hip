@@ -32,7 +32,22 @@ struct StreamParams {
     const float* bias;
     float* Y;
     uint32_t N, K, n_blocks, row_stride_bytes, y_offset;
+    // expert indirection (nullptr for the dense case): blockIdx.y is a (token, slot) pair that uses
+    // weight rows expert_idx[pair]*N .. +N-1, X row pair / k_slots (or pair, x_per_slot) and Y row pair
+    const uint32_t* expert_idx;
+    uint32_t k_slots, ldy;
+    int x_per_slot;
 };
+
+// Redirects the pointers of a grouped launch to the pair this workgroup serves.
+__device__ __forceinline__ void stream_select_pair(StreamParams& p)
+{
+    if (!p.expert_idx) return;
+    const uint32_t pair = blockIdx.y;
+    p.W += (size_t)p.expert_idx[pair] * p.N * p.row_stride_bytes;
+    p.X += (size_t)(p.x_per_slot ? pair : pair / p.k_slots) * p.K;
+    p.Y += (size_t)pair * p.ldy;
+}
 
 __device__ __forceinline__ float s_fma_h(_Float16 h, float x, float acc) { return __builtin_fmaf((float)h, x, acc); }
 
@@ -158,6 +173,7 @@ struct Q4Slot {
 template <int P, int NW, int D>
 __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
 {
+    stream_select_pair(p);
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t gw = blockIdx.x * NW + wave;
@@ -330,6 +346,7 @@ __device__ __forceinline__ float q6k_piece_dot(const Q6Piece& v, const float (&x
 template <int P, int KW, int D>
 __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
 {
+    stream_select_pair(p);
     __shared__ float part[KW > 1 ? KW : 1][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -432,8 +449,9 @@ static uint32_t stream_workgroups(uint32_t N, uint32_t per_cu, int rows_override
 
 bool gemv_stream_supported(const MatmulArgs& a)
 {
-    if (a.expert_idx) return false;
-    if (a.M != 1) return false;
+    // grouped calls: M counts (token, slot) pairs, each a matvec of its own
+    if (!a.expert_idx && a.M != 1) return false;
+    if (a.expert_idx && (a.M < 1 || a.M > 65535u || a.bias)) return false;
     if (((uintptr_t)a.X & 15u)) return false;
     if (a.n_blocks < 1) return false;
     if (a.type == KQ_TYPE_Q4_K) {
@@ -460,6 +478,11 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     p.n_blocks = a.n_blocks;
     p.row_stride_bytes = a.row_stride_bytes;
     p.y_offset = a.y_offset;
+    p.expert_idx = a.expert_idx;
+    p.k_slots = a.k_slots;
+    p.ldy = a.ldy;
+    p.x_per_slot = a.x_per_slot;
+    const uint32_t pairs = a.expert_idx ? a.M : 1u;   // grid.y
     // Measured on MI355X: these kernels run best with about 40 KB of weight loads
     // in flight per CU: 4 to 8 waves, two to four rows in flight each.  More waves
     // or deeper rings are slower.
@@ -468,13 +491,14 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
         const uint32_t nb = a.n_blocks;
         const int kw = nb <= 16u ? 1 : nb <= 32u ? 4 : 7;
         const int pp = nb <= 8u ? 1 : nb <= 16u ? 2 : nb <= 56u ? 1 : 2;
-        const uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 8u / (uint32_t)kw, t.splits);
+        uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 8u / (uint32_t)kw, t.splits);
+        wgs = (wgs + pairs - 1u) / pairs;   // the pairs of a grouped launch share the machine
         const int depth = t.depth > 0 ? t.depth : 2;
 #define KQ_STREAM6(P, KW) \
     do { \
-        if (depth <= 1) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 1>), dim3(wgs), dim3(64 * KW), 0, s, p); \
-        else if (depth <= 2) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 2>), dim3(wgs), dim3(64 * KW), 0, s, p); \
-        else hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 4>), dim3(wgs), dim3(64 * KW), 0, s, p); \
+        if (depth <= 1) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 1>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
+        else if (depth <= 2) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 2>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
+        else hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 4>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
     } while (0)
         if (kw == 1 && pp == 1) KQ_STREAM6(1, 1);
         else if (kw == 1) KQ_STREAM6(2, 1);
@@ -486,10 +510,11 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     }
     constexpr int NW = 4;
     // a Q4_K workgroup is NW independent waves, each with its own rows
-    const uint32_t wgs = t.splits > 0 ? ((a.N + (uint32_t)t.splits - 1u) / (uint32_t)t.splits + NW - 1u) / NW
-                                      : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
+    uint32_t wgs = t.splits > 0 ? ((a.N + (uint32_t)t.splits - 1u) / (uint32_t)t.splits + NW - 1u) / NW
+                                : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
+    wgs = (wgs + pairs - 1u) / pairs;
     const int depth = t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
-#define KQ_STREAM_LAUNCH(P, D) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D>), dim3(wgs), dim3(64 * NW), 0, s, p)
+#define KQ_STREAM_LAUNCH(P, D) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D>), dim3(wgs, pairs), dim3(64 * NW), 0, s, p)
     if (a.n_blocks <= 8u) {
         if (depth <= 1) KQ_STREAM_LAUNCH(1, 1);
         else if (depth <= 2) KQ_STREAM_LAUNCH(1, 2);

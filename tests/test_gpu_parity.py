@@ -372,6 +372,8 @@ def test_moe_ffn_vs_oracle(gpu, kqo, family, T, E, k, H, I):
         expect = "moe_ffn_generic"
     elif family == 0 and T * k >= 2 * E:
         expect = "moe_ffn_mtile"
+    elif family == 0:
+        expect = "moe_ffn_stream"     # a handful of pairs: one lanes-along-K matvec each
     else:
         expect = "moe_ffn_generic" if I == 256 else "moe_ffn_mrow"
     assert kern == expect, (kern, expect)
@@ -401,7 +403,7 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
         X = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
         xd, ed, wd = gpu.dev(X), gpu.dev(eidx.view(np.int32)), gpu.dev(ew)
         got = kquant.moe_ffn(xd, gw, uw, dw, ed, wd, E).cpu().numpy()
-        assert capi.last_kernel() == ("moe_ffn_mrow" if T == 1 else "moe_ffn_mtile")
+        assert capi.last_kernel() == ("moe_ffn_stream" if T == 1 else "moe_ffn_mtile")
         sel = np.arange(T) if T == 1 else np.array([0, 100, 101, 255])
         want = kqo.moe_ffn(Q4_K, Q6_K, X[sel], gp, up, dp, eidx[sel], ew[sel], H, I)
         rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
@@ -440,6 +442,22 @@ def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot, family, kern
         assert capi.last_kernel() == kernel
     finally:
         capi.force_kernel(0)
+    want = kqo.moe_matmul(type_, X, packed, eidx, N, K, x_per_slot=per_slot)
+    rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    assert np.all(np.abs(got - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
+
+
+@pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True), (Q6_K, 300, 4096, False)])
+def test_moe_matmul_few_pairs_stream(gpu, kqo, type_, N, K, per_slot):
+    """Decode-sized routing (fewer than two pairs per expert): one lanes-along-K matvec per pair."""
+    from backpack_amd import capi, kquant
+    E, T, k = 12, 3, 4
+    raw, packed, w = gpu.make_weight(type_, E * N, K, seed=71)
+    rng = np.random.default_rng(72)
+    eidx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.uint32)
+    X = rng.standard_normal((T * k if per_slot else T, K)).astype(np.float32)
+    got = kquant.moe_matmul(gpu.dev(X), w, gpu.dev(eidx.view(np.int32)), E, x_per_slot=per_slot).cpu().numpy()
+    assert capi.last_kernel() == "stream_grouped"
     want = kqo.moe_matmul(type_, X, packed, eidx, N, K, x_per_slot=per_slot)
     rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
     assert np.all(np.abs(got - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
