@@ -12,7 +12,7 @@ per-token command buffer (runtime/model_runner.cpp:5725-5759).
 
 Prints ONE JSON line.  `value` is weight+activation bytes of the step divided by
 wall time.  `roofline` covers the dominant kernel (the Q4_K GEMV on gate|up,
-48 % of the bytes), timed with HIP events on the launch stream over its own
+44 % of the bytes), timed with HIP events on the launch stream over its own
 region of 32 distinct matrices.  `cpu_baseline` times the reference's CPU path
 (dequantise to fp32, sequential fp32 dot) on a bounded sample on the host.
 """
@@ -32,10 +32,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 METRIC = "Q4_K M=1 matvec HBM GB/s (% of peak); M=2048 dequant-GEMM TFLOPS (% MFMA)"
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE (profiles/q4k_gemv_gate_up_hbm_traffic_pmc.txt): FETCH_SIZE 32601.0
-# x 2.000 KiB + WRITE_SIZE 112.0 x 1.000 KiB, the factors being what the same
+# WRITE_SIZE (profiles/decode_gemv_hbm_traffic_pmc.txt): FETCH_SIZE 32383.4
+# x 2.000 KiB + WRITE_SIZE 224.0 x 1.000 KiB, the factors being what the same
 # counters read for a 256 MiB copy kernel.
-MEASURED_TRAFFIC_BYTES = 66881536
+MEASURED_TRAFFIC_BYTES = 66550579
 
 
 def parse():
@@ -222,7 +222,7 @@ def main():
     dom_bytes = synth.weight_bytes(dom_w.type, dom_w.N, dom_w.K) + (dom_w.K + dom_w.N) * 4
     dom_gbs = dom_bytes / (dsec / launches) / 1e9
     roofline = {
-        "kernel": "kq::q4k_gemv_kernel<1, 8> (gate|up 28672x4096 Q4_K, M=1)",
+        "kernel": f"kq::q4k_stream_kernel<2, 4, 4> ({capi.last_kernel()}; gate|up 28672x4096 Q4_K, M=1)",
         "bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
         "bytes_per_launch": dom_bytes, "us_per_launch": round(dsec / launches * 1e6, 3),

@@ -180,16 +180,19 @@ BPK_API int bpk_kq_moe_ffn(int type_gu, int type_dn, const float *X,
 BPK_API const char *bpk_last_kernel(void);
 
 /* Force a kernel family for the next calls on this thread (testing only):
- * 0 = automatic, 1 = generic, 2 = row-per-lane GEMV, 3 = matrix-core small-M,
- * 4 = matrix-core tiled GEMM.  A forced family that cannot serve the call's
+ * 0 = automatic, 1 = generic, 2 = row-per-lane GEMV (M <= 4), 3 = row-per-lane
+ * kernel on the 4x4x4 matrix-core op (M <= 16), 4 = matrix-core tiled GEMM
+ * (bf16 X only), 5 = lanes-along-K GEMV (M = 1), 6 = 16-row x 16-token
+ * matrix-core tiles (M <= 16).  A forced family that cannot serve the call's
  * shape fails with BPK_ERR_SHAPE instead of falling back. */
 BPK_API int bpk_force_kernel(int family);
 
 /* Tuning knobs for experiments on this thread.  "gemv_splits": number of
- * K-range splits of the row-per-lane GEMV; "gemv_waves": its waves per
- * workgroup (2, 4 or 8); "gemv_depth": superblocks a wave keeps in flight
- * (1, 2 or 4); "gemm_tile": square workgroup tile of the bf16 GEMM
- * (128 or 256).  0 = automatic. */
+ * K-range splits of the row-per-lane GEMV, or rows per wave of the
+ * lanes-along-K GEMV; "gemv_waves": waves per workgroup of the row-per-lane
+ * kernels (2, 4 or 8); "gemv_depth": rows a wave of the lanes-along-K GEMV
+ * keeps in flight (1, 2 or 4); "gemm_tile": square workgroup tile of the bf16
+ * GEMM (128 or 256).  0 = automatic. */
 BPK_API int bpk_set_option(const char *name, int value);
 
 #ifdef __cplusplus
