@@ -245,10 +245,11 @@ def main():
         "metric": METRIC, "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "u8 weights, f32 activations and accumulation", "data": "synthetic",
+        "dtype": "f32", "data": "synthetic",
         "config": {"workload": "Llama-3-8B-shaped decode layer set, M=1, Q4_K_M mix "
                                f"({args.layers} layers x [qkv, o, gate_up, down] + lm_head)",
-                   "launches_per_step": len(mats), "weight_bytes": wb, "activation_bytes": act,
+                   "weights": "GGUF Q4_K / Q6_K superblocks, read as packed bytes", "activations": "f32",
+                   "accumulation": "f32", "launches_per_step": len(mats), "weight_bytes": wb, "activation_bytes": act,
                    "graph_replay": use_graph},
         "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 2),
         "tokens_per_s_equiv": round(args.steps / sec, 1),
