@@ -102,15 +102,18 @@ __device__ __forceinline__ void ring_load2(uint32_t& v, const uint8_t* ptr)
     asm volatile("global_load_ushort %0, %1, off" : "+v"(v) : "v"(ptr));
 }
 
-// One lane's share of one pass of a Q4_K row.
+// One lane's share of one pass of a Q4_K row, for MT tokens (the unpack is shared).
 //   hdr: the block's first 16 bytes; q: 16 quant bytes (piece j of the block)
 //   xlo/xhi: activations of the piece's 16 elements in the even / odd sub-block
 //   sel_hi: lane constant, j/2 >= 2;  sh: lane constant, 16 * ((j/2) & 1)
-__device__ __forceinline__ float q4k_piece_dot(const s_u32x4 hdr, const s_u32x4 q, const float (&xlo)[16],
-                                               const float (&xhi)[16], float xs_lo, float xs_hi, bool sel_hi,
-                                               uint32_t sh)
+template <int MT>
+__device__ __forceinline__ void q4k_piece_dot(const s_u32x4 hdr, const s_u32x4 q, const float (&xlo)[MT][16],
+                                              const float (&xhi)[MT][16], const float (&xs_lo)[MT],
+                                              const float (&xs_hi)[MT], bool sel_hi, uint32_t sh, float (&acc)[MT])
 {
-    float alo = 0.0f, ahi = 0.0f;
+    float alo[MT], ahi[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) { alo[t] = 0.0f; ahi[t] = 0.0f; }
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
         const uint32_t w = q[m];
@@ -119,14 +122,17 @@ __device__ __forceinline__ float q4k_piece_dot(const s_u32x4 hdr, const s_u32x4 
         const s_half2 b = __builtin_bit_cast(s_half2, w & 0x00F000F0u);     // high nibbles of bytes 0, 2 (x16)
         const s_half2 c = __builtin_bit_cast(s_half2, w8 & 0x000F000Fu);    // low nibbles of bytes 1, 3
         const s_half2 d = __builtin_bit_cast(s_half2, w8 & 0x00F000F0u);    // high nibbles of bytes 1, 3 (x16)
-        alo = s_fma_h(a.x, xlo[4 * m + 0], alo);
-        ahi = s_fma_h(b.x, xhi[4 * m + 0], ahi);
-        alo = s_fma_h(c.x, xlo[4 * m + 1], alo);
-        ahi = s_fma_h(d.x, xhi[4 * m + 1], ahi);
-        alo = s_fma_h(a.y, xlo[4 * m + 2], alo);
-        ahi = s_fma_h(b.y, xhi[4 * m + 2], ahi);
-        alo = s_fma_h(c.y, xlo[4 * m + 3], alo);
-        ahi = s_fma_h(d.y, xhi[4 * m + 3], ahi);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            alo[t] = s_fma_h(a.x, xlo[t][4 * m + 0], alo[t]);
+            ahi[t] = s_fma_h(b.x, xhi[t][4 * m + 0], ahi[t]);
+            alo[t] = s_fma_h(c.x, xlo[t][4 * m + 1], alo[t]);
+            ahi[t] = s_fma_h(d.x, xhi[t][4 * m + 1], ahi[t]);
+            alo[t] = s_fma_h(a.y, xlo[t][4 * m + 2], alo[t]);
+            ahi[t] = s_fma_h(b.y, xhi[t][4 * m + 2], ahi[t]);
+            alo[t] = s_fma_h(c.y, xlo[t][4 * m + 3], alo[t]);
+            ahi[t] = s_fma_h(d.y, xhi[t][4 * m + 3], ahi[t]);
+        }
     }
     // 6-bit scale and min of sub-blocks 2g and 2g+1: two adjacent bytes of each
     // scale word, at bit sh
@@ -136,14 +142,17 @@ __device__ __forceinline__ float q4k_piece_dot(const s_u32x4 hdr, const s_u32x4 
     const uint32_t mn_b = ((w2 >> 4) & 0x0F0Fu) | ((z2 >> 2) & 0x3030u);
     const uint32_t sc = sel_hi ? sc_b : sc_a;
     const uint32_t mn = sel_hi ? mn_b : mn_a;
-    const float sc0 = (float)(sc & 0xFFu), sc1 = (float)(sc >> 8);
+    const float sc0 = (float)(sc & 0xFFu), sc1 = (float)(sc >> 8) * 0.0625f;
     const float mn0 = (float)(mn & 0xFFu), mn1 = (float)(mn >> 8);
-    const float d = half_bits_to_float(hdr.x & 0xFFFFu);
+    const float d24 = half_bits_to_float(hdr.x & 0xFFFFu) * 16777216.0f;
     const float dmin = half_bits_to_float(hdr.x >> 16);
-    // alo carries 2^-24, ahi 2^-20
-    const float t = __builtin_fmaf(sc1 * 0.0625f, ahi, sc0 * alo);
-    const float u = __builtin_fmaf(mn1, xs_hi, mn0 * xs_lo);
-    return __builtin_fmaf(d * 16777216.0f, t, -(dmin * u));
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        // alo carries 2^-24, ahi 2^-20
+        const float tt = __builtin_fmaf(sc1, ahi[t], sc0 * alo[t]);
+        const float u = __builtin_fmaf(mn1, xs_hi[t], mn0 * xs_lo[t]);
+        acc[t] += __builtin_fmaf(d24, tt, -(dmin * u));
+    }
 }
 
 // One row in flight for the Q4_K kernel: P headers and P quant pieces per lane.
@@ -169,8 +178,8 @@ struct Q4Slot {
     }
 };
 
-// P passes of 8 superblocks cover a row (n_blocks <= 8 * P); D rows in flight.
-template <int P, int NW, int D>
+// P passes of 8 superblocks cover a row (n_blocks <= 8 * P); D rows in flight; MT tokens.
+template <int P, int NW, int D, int MT>
 __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
 {
     stream_select_pair(p);
@@ -186,7 +195,7 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
     const bool sel_hi = g >= 2u;
     const uint32_t sh = 16u * (g & 1u);
 
-    float xlo[P][16], xhi[P][16], xs_lo[P], xs_hi[P];
+    float xlo[P][MT][16], xhi[P][MT][16], xs_lo[P][MT], xs_hi[P][MT];
     uint32_t hoff[P];
 #pragma unroll
     for (int pass = 0; pass < P; ++pass) {
@@ -194,19 +203,22 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
         const bool valid = b < p.n_blocks;
         b = valid ? b : p.n_blocks - 1u;
         hoff[pass] = b * KQ_Q4K_BYTES;
-        const float4* xp = (const float4*)(p.X + (size_t)b * KQ_QK + 64u * g + 16u * h);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float4 lo = xp[i], hi = xp[8 + i];
-            if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
-            xlo[pass][4 * i + 0] = lo.x; xlo[pass][4 * i + 1] = lo.y; xlo[pass][4 * i + 2] = lo.z; xlo[pass][4 * i + 3] = lo.w;
-            xhi[pass][4 * i + 0] = hi.x; xhi[pass][4 * i + 1] = hi.y; xhi[pass][4 * i + 2] = hi.z; xhi[pass][4 * i + 3] = hi.w;
+        for (int t = 0; t < MT; ++t) {
+            const float4* xp = (const float4*)(p.X + (size_t)t * p.K + (size_t)b * KQ_QK + 64u * g + 16u * h);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float4 lo = xp[i], hi = xp[8 + i];
+                if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
+                xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
+                xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
+            }
+            float sl = 0.0f, sh_ = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
+            xs_lo[pass][t] = sl;
+            xs_hi[pass][t] = sh_;
         }
-        float sl = 0.0f, sh_ = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) { sl += xlo[pass][i]; sh_ += xhi[pass][i]; }
-        xs_lo[pass] = sl;
-        xs_hi[pass] = sh_;
     }
 
     // Ring of D rows in flight.  Slot d is refilled as soon as its row has been
@@ -219,29 +231,38 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
 #pragma unroll
     for (int d = 0; d < D; ++d)
         ring[d].fill(p.W + (size_t)(gw + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, hoff, j);
-    // Rows are taken 64 at a time: lane i keeps the sum of the chunk's row i, and the
+    // Rows are taken 64 at a time: lane i keeps the sums of the chunk's row i, and the
     // chunk is stored (bias added) after its last row.
     for (uint32_t c0 = 0; c0 < n_rows; c0 += 64u) {
         const uint32_t cnt = min(64u, n_rows - c0);
-        float res = 0.0f;
+        float res[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) res[t] = 0.0f;
         for (uint32_t i0 = 0; i0 < cnt; i0 += D) {
 #pragma unroll
             for (int d = 0; d < D; ++d) {
                 const uint32_t i = i0 + d;
                 ring[d].template wait<(D - 1) * SLOT_LOADS>();
-                float acc = 0.0f;
+                float acc[MT];
+#pragma unroll
+                for (int t = 0; t < MT; ++t) acc[t] = 0.0f;
 #pragma unroll
                 for (int pass = 0; pass < P; ++pass)
-                    acc += q4k_piece_dot(ring[d].hdr[pass], ring[d].q[pass], xlo[pass], xhi[pass], xs_lo[pass],
-                                         xs_hi[pass], sel_hi, sh);
+                    q4k_piece_dot<MT>(ring[d].hdr[pass], ring[d].q[pass], xlo[pass], xhi[pass], xs_lo[pass],
+                                      xs_hi[pass], sel_hi, sh, acc);
                 ring[d].fill(p.W + (size_t)(gw + min(c0 + i + D, n_rows - 1u) * stride) * p.row_stride_bytes, hoff, j);
-                const float tot = wave_sum(acc);
-                res = (lane == i && i < cnt) ? tot : res;
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    const float tot = wave_sum(acc[t]);
+                    res[t] = (lane == i && i < cnt) ? tot : res[t];
+                }
             }
         }
         if (lane < cnt) {
             const uint32_t r = gw + (c0 + lane) * stride;
-            p.Y[p.y_offset + r] = res + (p.bias ? p.bias[r] : 0.0f);
+            const float bias = p.bias ? p.bias[r] : 0.0f;
+#pragma unroll
+            for (int t = 0; t < MT; ++t) p.Y[(size_t)t * p.ldy + p.y_offset + r] = res[t] + bias;
         }
     }
     asm volatile("s_waitcnt vmcnt(0)");   // the ring's last refills land before the wave ends
@@ -293,11 +314,16 @@ struct Q6Slot {
     }
 };
 
-// x[k][i]: activation of element 128n + 32k + 8lg + i;  m32xs[k] = -32 * sum_i x[k][i]
-__device__ __forceinline__ float q6k_piece_dot(const Q6Piece& v, const float (&x)[4][8], const float (&m32xs)[4],
-                                               uint32_t sc_shift)
+// x[t][k][i]: activation of element 128n + 32k + 8lg + i of token t;  m32xs[t][k] = -32 * sum_i x[t][k][i]
+template <int MT>
+__device__ __forceinline__ void q6k_piece_dot(const Q6Piece& v, const float (&x)[MT][4][8], const float (&m32xs)[MT][4],
+                                              uint32_t sc_shift, float (&acc)[MT])
 {
-    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float a[MT][4];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) a[t][k] = 0.0f;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
         const uint32_t A = v.a[u], B = v.b[u], H = v.h[u];
@@ -313,41 +339,48 @@ __device__ __forceinline__ float q6k_piece_dot(const Q6Piece& v, const float (&x
         const s_half2 q1b = __builtin_bit_cast(s_half2, (B8 & 0x000F000Fu) | (Hr6 & 0x00300030u));
         const s_half2 q3b = __builtin_bit_cast(s_half2, (B8 & 0x00F000F0u) | (Hr6 & 0x03000300u));
         const int i = 4 * u;
-        a[0] = s_fma_h(q0a.x, x[0][i + 0], a[0]);
-        a[1] = s_fma_h(q1a.x, x[1][i + 0], a[1]);
-        a[2] = s_fma_h(q2a.x, x[2][i + 0], a[2]);
-        a[3] = s_fma_h(q3a.x, x[3][i + 0], a[3]);
-        a[0] = s_fma_h(q0b.x, x[0][i + 1], a[0]);
-        a[1] = s_fma_h(q1b.x, x[1][i + 1], a[1]);
-        a[2] = s_fma_h(q2b.x, x[2][i + 1], a[2]);
-        a[3] = s_fma_h(q3b.x, x[3][i + 1], a[3]);
-        a[0] = s_fma_h(q0a.y, x[0][i + 2], a[0]);
-        a[1] = s_fma_h(q1a.y, x[1][i + 2], a[1]);
-        a[2] = s_fma_h(q2a.y, x[2][i + 2], a[2]);
-        a[3] = s_fma_h(q3a.y, x[3][i + 2], a[3]);
-        a[0] = s_fma_h(q0b.y, x[0][i + 3], a[0]);
-        a[1] = s_fma_h(q1b.y, x[1][i + 3], a[1]);
-        a[2] = s_fma_h(q2b.y, x[2][i + 3], a[2]);
-        a[3] = s_fma_h(q3b.y, x[3][i + 3], a[3]);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            a[t][0] = s_fma_h(q0a.x, x[t][0][i + 0], a[t][0]);
+            a[t][1] = s_fma_h(q1a.x, x[t][1][i + 0], a[t][1]);
+            a[t][2] = s_fma_h(q2a.x, x[t][2][i + 0], a[t][2]);
+            a[t][3] = s_fma_h(q3a.x, x[t][3][i + 0], a[t][3]);
+            a[t][0] = s_fma_h(q0b.x, x[t][0][i + 1], a[t][0]);
+            a[t][1] = s_fma_h(q1b.x, x[t][1][i + 1], a[t][1]);
+            a[t][2] = s_fma_h(q2b.x, x[t][2][i + 1], a[t][2]);
+            a[t][3] = s_fma_h(q3b.x, x[t][3][i + 1], a[t][3]);
+            a[t][0] = s_fma_h(q0a.y, x[t][0][i + 2], a[t][0]);
+            a[t][1] = s_fma_h(q1a.y, x[t][1][i + 2], a[t][1]);
+            a[t][2] = s_fma_h(q2a.y, x[t][2][i + 2], a[t][2]);
+            a[t][3] = s_fma_h(q3a.y, x[t][3][i + 2], a[t][3]);
+            a[t][0] = s_fma_h(q0b.y, x[t][0][i + 3], a[t][0]);
+            a[t][1] = s_fma_h(q1b.y, x[t][1][i + 3], a[t][1]);
+            a[t][2] = s_fma_h(q2b.y, x[t][2][i + 3], a[t][2]);
+            a[t][3] = s_fma_h(q3b.y, x[t][3][i + 3], a[t][3]);
+        }
     }
     // scale of (half n, k, l/16) is byte 2k + l/16 of the half's eight: sc_shift = 8 * (l/16)
     const uint32_t s01 = v.sc.x >> sc_shift, s23 = v.sc.y >> sc_shift;
     const float sc0 = (float)(int)(int8_t)(s01 & 255u), sc1 = (float)(int)(int8_t)((s01 >> 16) & 255u);
     const float sc2 = (float)(int)(int8_t)(s23 & 255u), sc3 = (float)(int)(int8_t)((s23 >> 16) & 255u);
-    float tot = sc0 * __builtin_fmaf(a[0], 16777216.0f, m32xs[0]);
-    tot = __builtin_fmaf(sc1, __builtin_fmaf(a[1], 16777216.0f, m32xs[1]), tot);
-    tot = __builtin_fmaf(sc2, __builtin_fmaf(a[2], 1048576.0f, m32xs[2]), tot);
-    tot = __builtin_fmaf(sc3, __builtin_fmaf(a[3], 1048576.0f, m32xs[3]), tot);
-    return half_bits_to_float(v.d) * tot;
+    const float d = half_bits_to_float(v.d);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        float tot = sc0 * __builtin_fmaf(a[t][0], 16777216.0f, m32xs[t][0]);
+        tot = __builtin_fmaf(sc1, __builtin_fmaf(a[t][1], 16777216.0f, m32xs[t][1]), tot);
+        tot = __builtin_fmaf(sc2, __builtin_fmaf(a[t][2], 1048576.0f, m32xs[t][2]), tot);
+        tot = __builtin_fmaf(sc3, __builtin_fmaf(a[t][3], 1048576.0f, m32xs[t][3]), tot);
+        acc[t] += d * tot;
+    }
 }
 
 // Workgroup = KW waves, one K slice of 8*P superblocks each; the workgroup walks
 // rows blockIdx.x, + gridDim.x, ...; D rows in flight per wave.
-template <int P, int KW, int D>
+template <int P, int KW, int D, int MT>
 __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
 {
     stream_select_pair(p);
-    __shared__ float part[KW > 1 ? KW : 1][64];
+    __shared__ float part[KW > 1 ? KW : 1][MT][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t g = blockIdx.x, stride = gridDim.x;
@@ -355,7 +388,7 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
     const uint32_t bl = lane >> 3, t = lane & 7u, n = t >> 2, lg = t & 3u;
     const uint32_t sc_shift = 8u * (lg >> 1);
 
-    float x[P][4][8], m32xs[P][4];
+    float x[P][MT][4][8], m32xs[P][MT][4];
     uint32_t boff[P];
 #pragma unroll
     for (int pass = 0; pass < P; ++pass) {
@@ -363,17 +396,20 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
         const bool valid = b < p.n_blocks;
         b = valid ? b : p.n_blocks - 1u;
         boff[pass] = b * KQ_Q6K_BYTES;
-        const float4* xp = (const float4*)(p.X + (size_t)b * KQ_QK + 128u * n + 8u * lg);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            float4 lo = xp[8 * k], hi = xp[8 * k + 1];
-            if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
-            x[pass][k][0] = lo.x; x[pass][k][1] = lo.y; x[pass][k][2] = lo.z; x[pass][k][3] = lo.w;
-            x[pass][k][4] = hi.x; x[pass][k][5] = hi.y; x[pass][k][6] = hi.z; x[pass][k][7] = hi.w;
-            float sum = 0.0f;
+        for (int tk = 0; tk < MT; ++tk) {
+            const float4* xp = (const float4*)(p.X + (size_t)tk * p.K + (size_t)b * KQ_QK + 128u * n + 8u * lg);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) sum += x[pass][k][i];
-            m32xs[pass][k] = -32.0f * sum;
+            for (int k = 0; k < 4; ++k) {
+                float4 lo = xp[8 * k], hi = xp[8 * k + 1];
+                if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
+                x[pass][tk][k][0] = lo.x; x[pass][tk][k][1] = lo.y; x[pass][tk][k][2] = lo.z; x[pass][tk][k][3] = lo.w;
+                x[pass][tk][k][4] = hi.x; x[pass][tk][k][5] = hi.y; x[pass][tk][k][6] = hi.z; x[pass][tk][k][7] = hi.w;
+                float sum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sum += x[pass][tk][k][i];
+                m32xs[pass][tk][k] = -32.0f * sum;
+            }
         }
     }
 
@@ -383,39 +419,51 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
 #pragma unroll
     for (int d = 0; d < D; ++d)
         ring[d].fill(p.W + (size_t)(g + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, boff, n, lg);
-    // Rows are taken 64 at a time: lane i keeps the sum of the chunk's row i; the K
+    // Rows are taken 64 at a time: lane i keeps the sums of the chunk's row i; the K
     // slices are folded and the chunk stored after its last row.  The row loop is
     // the one of the Q4_K kernel.
     for (uint32_t c0 = 0; c0 < n_rows; c0 += 64u) {
         const uint32_t cnt = min(64u, n_rows - c0);
-        float res = 0.0f;
+        float res[MT];
+#pragma unroll
+        for (int tk = 0; tk < MT; ++tk) res[tk] = 0.0f;
         for (uint32_t i0 = 0; i0 < cnt; i0 += D) {
 #pragma unroll
             for (int d = 0; d < D; ++d) {
                 const uint32_t i = i0 + d;
                 ring[d].template wait<(D - 1) * SLOT_LOADS>();
-                float acc = 0.0f;
+                float acc[MT];
+#pragma unroll
+                for (int tk = 0; tk < MT; ++tk) acc[tk] = 0.0f;
 #pragma unroll
                 for (int pass = 0; pass < P; ++pass)
-                    acc += q6k_piece_dot(ring[d].v[pass], x[pass], m32xs[pass], sc_shift);
+                    q6k_piece_dot<MT>(ring[d].v[pass], x[pass], m32xs[pass], sc_shift, acc);
                 ring[d].fill(p.W + (size_t)(g + min(c0 + i + D, n_rows - 1u) * stride) * p.row_stride_bytes, boff, n, lg);
-                const float tot = wave_sum(acc);
-                res = (lane == i && i < cnt) ? tot : res;
+#pragma unroll
+                for (int tk = 0; tk < MT; ++tk) {
+                    const float tot = wave_sum(acc[tk]);
+                    res[tk] = (lane == i && i < cnt) ? tot : res[tk];
+                }
             }
         }
         if (KW > 1) {
-            part[wave][lane] = res;
+#pragma unroll
+            for (int tk = 0; tk < MT; ++tk) part[wave][tk][lane] = res[tk];
             __syncthreads();
         }
         if (wave == 0 && lane < cnt) {
-            float y = res;
-            if (KW > 1) {
-                y = part[0][lane];
-#pragma unroll
-                for (int w = 1; w < KW; ++w) y += part[w][lane];
-            }
             const uint32_t r = g + (c0 + lane) * stride;
-            p.Y[p.y_offset + r] = y + (p.bias ? p.bias[r] : 0.0f);
+            const float bias = p.bias ? p.bias[r] : 0.0f;
+#pragma unroll
+            for (int tk = 0; tk < MT; ++tk) {
+                float y = res[tk];
+                if (KW > 1) {
+                    y = part[0][tk][lane];
+#pragma unroll
+                    for (int w = 1; w < KW; ++w) y += part[w][tk][lane];
+                }
+                p.Y[(size_t)tk * p.ldy + p.y_offset + r] = y + bias;
+            }
         }
         if (KW > 1) __syncthreads();
     }
@@ -450,7 +498,7 @@ static uint32_t stream_workgroups(uint32_t N, uint32_t per_cu, int rows_override
 bool gemv_stream_supported(const MatmulArgs& a)
 {
     // grouped calls: M counts (token, slot) pairs, each a matvec of its own
-    if (!a.expert_idx && a.M != 1) return false;
+    if (!a.expert_idx && (a.M < 1 || a.M > 2)) return false;
     if (a.expert_idx && (a.M < 1 || a.M > 65535u || a.bias)) return false;
     if (((uintptr_t)a.X & 15u)) return false;
     if (a.n_blocks < 1) return false;
@@ -483,6 +531,7 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     p.ldy = a.ldy;
     p.x_per_slot = a.x_per_slot;
     const uint32_t pairs = a.expert_idx ? a.M : 1u;   // grid.y
+    const bool two = !a.expert_idx && a.M == 2;       // two tokens share every weight load
     // Measured on MI355X: these kernels run best with about 40 KB of weight loads
     // in flight per CU: 4 to 8 waves, two to four rows in flight each.  More waves
     // or deeper rings are slower.
@@ -494,11 +543,16 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
         uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 8u / (uint32_t)kw, t.splits);
         wgs = (wgs + pairs - 1u) / pairs;   // the pairs of a grouped launch share the machine
         const int depth = t.depth > 0 ? t.depth : 2;
+#define KQ_STREAM6_MT(P, KW, MT) \
+    do { \
+        if (depth <= 1) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 1, MT>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
+        else if (depth <= 2) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 2, MT>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
+        else hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 4, MT>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
+    } while (0)
 #define KQ_STREAM6(P, KW) \
     do { \
-        if (depth <= 1) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 1>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
-        else if (depth <= 2) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 2>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
-        else hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 4>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
+        if (two) KQ_STREAM6_MT(P, KW, 2); \
+        else KQ_STREAM6_MT(P, KW, 1); \
     } while (0)
         if (kw == 1 && pp == 1) KQ_STREAM6(1, 1);
         else if (kw == 1) KQ_STREAM6(2, 1);
@@ -506,6 +560,7 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
         else if (pp == 1) KQ_STREAM6(1, 7);
         else KQ_STREAM6(2, 7);
 #undef KQ_STREAM6
+#undef KQ_STREAM6_MT
         return hipGetLastError();
     }
     constexpr int NW = 4;
@@ -514,7 +569,11 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
                                 : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
     wgs = (wgs + pairs - 1u) / pairs;
     const int depth = t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
-#define KQ_STREAM_LAUNCH(P, D) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D>), dim3(wgs, pairs), dim3(64 * NW), 0, s, p)
+#define KQ_STREAM_LAUNCH(P, D) \
+    do { \
+        if (two) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, 2>), dim3(wgs, pairs), dim3(64 * NW), 0, s, p); \
+        else hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, 1>), dim3(wgs, pairs), dim3(64 * NW), 0, s, p); \
+    } while (0)
     if (a.n_blocks <= 8u) {
         if (depth <= 1) KQ_STREAM_LAUNCH(1, 1);
         else if (depth <= 2) KQ_STREAM_LAUNCH(1, 2);

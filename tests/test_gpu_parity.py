@@ -190,18 +190,21 @@ STREAM_SHAPES = [
 @pytest.mark.parametrize("type_,N,K", STREAM_SHAPES)
 @pytest.mark.parametrize("depth", [1, 2, 4])
 @pytest.mark.parametrize("rows_per_wave", [1, 3, 100])
-def test_gemv_stream_shapes(gpu, kqo, type_, N, K, depth, rows_per_wave):
+@pytest.mark.parametrize("M", [1, 2])
+def test_gemv_stream_shapes(gpu, kqo, type_, N, K, depth, rows_per_wave, M):
     """The lanes-along-K kernel over its tuning space: rows in flight per wave,
     rows per wave (1 = every wave a single row, 100 = more than the 64 rows a
     wave folds at a time), every pass / K-slice configuration, ragged last
-    pass, with a y offset and bias."""
+    pass, one and two tokens, with a y offset and bias."""
     import torch
     from backpack_amd import capi, kquant
     raw, packed, w = gpu.make_weight(type_, N, K, seed=N)
     rng = np.random.default_rng(depth * 100 + rows_per_wave)
-    X = rng.standard_normal((1, K)).astype(np.float32)
+    X = rng.standard_normal((M, K)).astype(np.float32)
     bias = rng.standard_normal(N).astype(np.float32)
-    out = torch.full((1, N + 7), 123.0, device="cuda")
+    out = torch.full((M, N), 123.0, device="cuda")
+    if M == 1:
+        out = torch.full((1, N + 7), 123.0, device="cuda")   # room for a y offset
     capi.set_option("gemv_depth", depth)
     capi.set_option("gemv_splits", rows_per_wave)
     capi.force_kernel(5)
@@ -209,15 +212,17 @@ def test_gemv_stream_shapes(gpu, kqo, type_, N, K, depth, rows_per_wave):
         _say("stream", type_, N, K, depth, rows_per_wave)
         xd, bd = gpu.dev(X), gpu.dev(bias)      # named: the buffers must outlive the call
         capi.check(capi.lib().bpk_kq_matmul(type_, xd.data_ptr(), w.data.data_ptr(), bd.data_ptr(),
-                                            out.data_ptr(), 1, N, K, w.n_blocks, w.row_stride_words, 7, None))
+                                            out.data_ptr(), M, N, K, w.n_blocks, w.row_stride_words, 7 if M == 1 else 0, None))
         assert capi.last_kernel() == "gemv_stream"
     finally:
         capi.force_kernel(0)
         capi.set_option("gemv_depth", 0)
         capi.set_option("gemv_splits", 0)
     got = out.cpu().numpy()
-    assert np.all(got[:, :7] == 123.0), "wrote before y_offset"
-    gpu.check_matmul(kqo, type_, got[:, 7:], X, packed, N, K, bias=bias,
+    if M == 1:
+        assert np.all(got[:, :7] == 123.0), "wrote before y_offset"
+        got = got[:, 7:]
+    gpu.check_matmul(kqo, type_, got, X, packed, N, K, bias=bias,
                      label=f"stream {type_} {N}x{K} d{depth} r{rows_per_wave}")
 
 
