@@ -259,6 +259,8 @@ def main():
         "roofline": roofline,
         "per_shape": shapes,
     }
+    if args.all:
+        out["config0"] = config0_leg()
     if args.verify or args.all:
         out["verify"] = verify_leg(mats, wb, use_graph)
     if args.moe or args.all:
@@ -271,6 +273,33 @@ def main():
         torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
+
+
+def config0_leg():
+    """One Q4_K matvec, M=1, K=N=4096 (a decode projection): cold = 64 distinct
+    matrices per pass (604 MB, beyond the last-level cache), hot = one matrix
+    launched back to back; graph replay, HIP events around each pass."""
+    import torch
+    from backpack_amd import kquant, synth
+    N = K = 4096
+    mk = lambda seed: kquant.KQuantPacked(synth.make_packed_device(synth.Q4_K, N, K, seed=seed), synth.Q4_K, N, K,
+                                          synth.row_stride_words(synth.Q4_K, K), synth.n_blocks(K))
+    ws = [mk(1000 + i) for i in range(64)]
+    x = torch.randn(1, K, device="cuda", generator=torch.Generator(device="cuda").manual_seed(0))
+    y = torch.empty(1, N, device="cuda")
+    nbytes = synth.weight_bytes(synth.Q4_K, N, K) + (K + N) * 4
+    res = {}
+    for label, mats in (("cold", ws), ("hot", [ws[0]] * 64)):
+        sel = [("m", w, x, y) for w in mats]
+        times = []
+        for _ in range(5):
+            s, _ = run_region(sel, 4, 1, True)
+            times.append(s / (4 * len(sel)))
+        times.sort()
+        res[label] = {"us_min": round(times[0] * 1e6, 2), "us_median": round(times[len(times) // 2] * 1e6, 2),
+                      "GBps": round(nbytes / times[len(times) // 2] / 1e9, 1), "launches_timed": 5 * 4 * len(sel)}
+    res["bytes_per_launch"] = nbytes
+    return res
 
 
 def verify_leg(mats, wb, use_graph):

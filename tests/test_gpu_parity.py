@@ -124,6 +124,8 @@ SHAPES = [
     (Q4_K, 9, 2300, 1280),      # ... with a partial last chunk of superblocks (5 blocks)
     (Q6_K, 8, 2000, 4096),
     (Q6_K, 13, 1800, 1536),     # Q6_K beyond 8 tokens: two groups; 6 blocks
+    (Q4_K, 37, 300, 1024),      # fp32 X beyond 16 tokens: groups of 16 (Q4_K) / 8 (Q6_K) on the tile kernel
+    (Q6_K, 21, 200, 1024),
     (Q4_K, 16, 22500, 512),     # tile kernel, a wave per tile (7 or 8 tiles per workgroup), ragged last tile
     (Q6_K, 5, 23001, 768),
 ]
