@@ -26,6 +26,7 @@ thread_local const char* t_kernel = "";
 thread_local int t_family = 0;
 thread_local kq::GemvTuning t_gemv;
 thread_local int t_gemm_tile = 0;
+thread_local int t_gemm_split = 0;
 
 int fail(int code, const char* fmt, ...)
 {
@@ -143,6 +144,11 @@ int bpk_set_option(const char* name, int value)
     if (!strcmp(name, "gemm_tile")) {
         if (value != 0 && value != 128 && value != 256) return fail(BPK_ERR_SHAPE, "gemm_tile must be 0, 128 or 256");
         t_gemm_tile = value;
+        return BPK_OK;
+    }
+    if (!strcmp(name, "gemm_split")) {
+        if (value < 0 || value > 2) return fail(BPK_ERR_SHAPE, "gemm_split must be 0, 1 or 2");
+        t_gemm_split = value;
         return BPK_OK;
     }
     return fail(BPK_ERR_SHAPE, "unknown option '%s'", name);
@@ -331,7 +337,7 @@ int bpk_kq_matmul_bf16(int type, const uint16_t* X, const void* W, const float* 
     if (!kq::gemm_bf16_supported(a))
         return fail(BPK_ERR_ALIGN, "bf16 GEMM needs 16-byte aligned X and (for Q4_K) 16-byte aligned W rows");
     t_kernel = "gemm_bf16";
-    hipError_t e = kq::launch_gemm_bf16(a, t_gemm_tile, (hipStream_t)stream);
+    hipError_t e = kq::launch_gemm_bf16(a, t_gemm_tile, t_gemm_split, (hipStream_t)stream);
     return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
 }
 

@@ -8,14 +8,18 @@
 // v_mfma_f32_32x32x16_bf16, fp32 accumulation in registers.  LDS is
 // double-buffered with one barrier per step.
 //
-// The 256 x 256 tile runs 8 waves (2 x 4, 128 x 64 each), two per SIMD, in two
-// phases: waves 0..3 issue the global loads of step t+1, run the MFMAs of step
-// t and then dequantise step t+1; waves 4..7 first dequantise step t+1 from
-// registers loaded a step earlier, issue the loads of step t+2, then run the
-// MFMAs of step t.  On every SIMD one wave's conversion arithmetic therefore
-// overlaps the other wave's matrix work.  The 128 x 128 tile runs 4 waves
-// (2 x 2) and fits twice on a CU, which gives the same overlap between
-// workgroups.
+// Two kernels:
+//  - 256 x 256 tile, 8 waves (2 x 4, 128 x 64 each, two per SIMD), persistent.  Every wave runs the same
+//    software-pipelined schedule: a step is four k slices of 16; in a slice the wave issues the LDS operand
+//    reads of the next slice, the 8 matrix instructions of this slice and, between them, a quarter of its
+//    share of the next tile (X piece copied, 8 weights dequantised, the global loads that refill the
+//    registers just freed).  The step's barrier sits before the last slice, whose operands are already in
+//    registers, so the matrix cores have work the moment the barrier opens.  The walk over (tile, k step)
+//    units is either one tile per workgroup or cut into equal shares per CU ("stream-K"): a tile cut
+//    between workgroups is summed into Y with fp32 atomics after a small kernel has cleared it (two
+//    addends per element in the common case, so the sum does not depend on their order).
+//  - 128 x 128 tile, 4 waves (2 x 2), two workgroups per CU: for shapes whose 256-tiles would leave half
+//    the CUs idle and whose K is too short to be worth cutting.
 //
 // LDS rows are 64 bf16 + 16 bytes of padding (144 B = an odd number of 16-byte
 // slots), which makes the 128-bit fragment reads of 32 consecutive rows
@@ -26,6 +30,7 @@
 // 32 consecutive floats of one Y row.
 #include "kq_format.h"
 #include "kq_kernels.h"
+#include <type_traits>
 
 namespace kq {
 
@@ -44,6 +49,9 @@ struct GemmParams {
     const float* bias;
     float* Y;
     uint32_t M, N, K, n_blocks, row_stride_bytes, ldy;
+    // walk of the persistent kernel: units = k steps (of 64) of all 256 x 256 tiles, tile after tile
+    // (tiles of one token block next to each other), cut into equal shares
+    uint32_t tiles_n, units, units_per_wg;
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
@@ -149,6 +157,43 @@ __device__ __forceinline__ void q6k_expand(const Q6Raw& r, uint32_t kc, uint32_t
     }
 }
 
+// Epilogue of both kernels.  Accumulator register r of lane l of a 32 x 32 block: token row
+// 8*(r/4) + 4*(l/32) + r%4, weight row l%32, so a register's 32 lanes store 128 contiguous bytes of one Y
+// row.  A wave whose rows all exist stores without per-row branches: a branch per store would make every
+// store wait for the one before it (the bias load keeps the memory counter ambiguous at each join).
+template <int TM, int TN, bool ATOMIC = false>
+__device__ __forceinline__ void store_acc(const GemmParams& p, const f32x16 (&acc)[TM][TN], uint32_t m_base, uint32_t n_base,
+                                          uint32_t lane, bool with_bias = true)
+{
+    const bool full = m_base + TM * 32u <= p.M;   // wave-uniform
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const uint32_t n = n_base + j * 32u + (lane & 31u);
+        if (n >= p.N) continue;
+        const float bias = (p.bias && with_bias) ? p.bias[n] : 0.0f;
+        float* y = p.Y + (size_t)(m_base + 4u * (lane >> 5)) * p.ldy + n;
+        auto put = [&](float* dst, float v) {
+            if (ATOMIC) __builtin_amdgcn_global_atomic_fadd_f32(dst, v);   // no return value: fire and forget
+            else *dst = v;
+        };
+        if (full) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    put(y + (size_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * p.ldy, acc[i][j][r] + bias);
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t dm = i * 32 + 8 * (r >> 2) + (r & 3);
+                    if (m_base + 4u * (lane >> 5) + dm < p.M) put(y + (size_t)dm * p.ldy, acc[i][j][r] + bias);
+                }
+        }
+    }
+}
+
 template <int TYPE, int BM, int BN, int NWAVES>
 __global__ __launch_bounds__(64 * NWAVES) void gemm_bf16_kernel(GemmParams p)
 {
@@ -160,7 +205,6 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm_bf16_kernel(GemmParams p)
     constexpr int XROWS = NT / 8;         // X rows per pass: 8 threads x 16 bytes per row
     constexpr int XP = BM / XROWS;        // X passes
     constexpr int WI = BN * 2 / NT;       // W items (row, 32-element run) per thread
-    constexpr bool PHASED = NWAVES == 8;  // second half of the waves converts before it multiplies
     uint8_t* As = smem;
     uint8_t* Bs = smem + 2 * A_BYTES;
 
@@ -169,7 +213,6 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm_bf16_kernel(GemmParams p)
     const uint32_t wm = wave / WAVES_N, wn = wave % WAVES_N;
     const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const uint32_t nk = p.K / GEMM_BK;
-    const bool convert_first = PHASED && wave >= NWAVES / 2;   // wave-uniform
 
     // X: thread -> (row tid/8 of each pass, 16-byte column tid%8)
     const uint8_t* xsrc[XP];
@@ -243,38 +286,274 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm_bf16_kernel(GemmParams p)
 
     load_tile(0);
     store_tile(0, 0);
-    if (convert_first && nk > 1) load_tile(1);
     __syncthreads();
 
     for (uint32_t kt = 0; kt < nk; ++kt) {
         const uint32_t buf = kt & 1u;
-        if (convert_first) {
-            if (kt + 1 < nk) store_tile(kt + 1, buf ^ 1u);
-            if (kt + 2 < nk) load_tile(kt + 2);
-        } else {
-            if (kt + 1 < nk) load_tile(kt + 1);
-        }
+        if (kt + 1 < nk) load_tile(kt + 1);
         multiply(buf);
-        if (!convert_first && kt + 1 < nk) store_tile(kt + 1, buf ^ 1u);
+        if (kt + 1 < nk) store_tile(kt + 1, buf ^ 1u);
         __syncthreads();
     }
 
-    // accumulator register r of lane l: token row 8*(r/4) + 4*(l/32) + r%4, weight row l%32
+    store_acc<TM, TN>(p, acc, m0 + wm * WM, n0 + wn * WN, lane);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Persistent 256 x 256 x 64 kernel.  A thread owns one (weight row, run of 32 k) item of the W tile and four
+// 16-byte pieces of the X tile per step; their raw bytes live in registers one step ahead of their use.
+struct RawQ4 { u32x4 h, q0, q1; };
+struct RawQ6 { u32x4 a0, a1, b0, b1; uint32_t sc2, d16; };
+
+__device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, uint32_t, RawQ4& r)
+{
+    r.h = *(const u32x4*)(row + (size_t)(kc >> 2) * KQ_Q4K_BYTES);
+}
+__device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint32_t, int half, RawQ4& r)
+{
+    const u32x4* q = (const u32x4*)(row + (size_t)(kc >> 2) * KQ_Q4K_BYTES + 16 + (kc & 3u) * 32u);
+    if (half == 0) r.q0 = q[0]; else r.q1 = q[1];
+}
+__device__ __forceinline__ void il_scales(const RawQ4& r, uint32_t kc, uint32_t hf, float& s0, float& s1, float& nb)
+{
+    const float d = half_bits_to_float(r.h.x & 0xFFFFu);
+    const float dmin = half_bits_to_float(r.h.x >> 16);
+    uint32_t sc, mn;
+    q4k_scale_min(r.h.y, r.h.z, r.h.w, (int)((kc & 3u) * 2u + hf), sc, mn);
+    // the high nibble is converted in place (16 q), so its scale carries the 1/16
+    s0 = d * (float)sc * (hf ? 0.0625f : 1.0f);
+    s1 = s0;
+    nb = -(dmin * (float)mn);
+}
+// 8 weights (piece v of the thread's run of 32) -> 16 bytes of bf16
+__device__ __forceinline__ u32x4 il_expand(const RawQ4& r, uint32_t, uint32_t hf, int v, float s0, float, float nb)
+{
+    const u32x4 src = v < 2 ? r.q0 : r.q1;
+    const uint32_t mask = hf ? 0xF0F0F0F0u : 0x0F0F0F0Fu;
+    u32x4 out;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const uint32_t n = n0 + wn * WN + j * 32u + (lane & 31u);
-        if (n >= p.N) continue;
-        const float bias = p.bias ? p.bias[n] : 0.0f;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint32_t m = m0 + wm * WM + i * 32u + 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
-                if (m < p.M) p.Y[(size_t)m * p.ldy + n] = acc[i][j][r] + bias;
-            }
-        }
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t w = src[(v & 1) * 2 + j] & mask;
+        const float f0 = fmaf(s0, (float)(w & 255u), nb);
+        const float f1 = fmaf(s0, (float)((w >> 8) & 255u), nb);
+        const float f2 = fmaf(s0, (float)((w >> 16) & 255u), nb);
+        const float f3 = fmaf(s0, (float)(w >> 24), nb);
+        out[j * 2] = pack_bf16(f0, f1);
+        out[j * 2 + 1] = pack_bf16(f2, f3);
+    }
+    return out;
+}
+
+__device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, uint32_t hf, RawQ6& r)
+{
+    const uint32_t c = kc & 3u, h = c >> 1, t = (c & 1u) * 2u + hf;
+    const uint8_t* blk = row + (size_t)(kc >> 2) * KQ_Q6K_BYTES;
+    uint16_t s2, d2;
+    __builtin_memcpy(&s2, blk + 192u + 8u * h + 2u * t, 2);
+    __builtin_memcpy(&d2, blk + 208u, 2);
+    r.sc2 = s2;
+    r.d16 = d2;
+}
+__device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint32_t hf, int half, RawQ6& r)
+{
+    const uint32_t c = kc & 3u, h = c >> 1, t = (c & 1u) * 2u + hf;
+    const uint8_t* blk = row + (size_t)(kc >> 2) * KQ_Q6K_BYTES;
+    // blocks are 2-byte aligned; the hardware takes unaligned 128-bit loads as they are
+    if (half == 0) {
+        __builtin_memcpy(&r.a0, blk + 64u * h + 32u * (t & 1u), 16);
+        __builtin_memcpy(&r.b0, blk + 128u + 32u * h, 16);
+    } else {
+        __builtin_memcpy(&r.a1, blk + 64u * h + 32u * (t & 1u) + 16u, 16);
+        __builtin_memcpy(&r.b1, blk + 128u + 32u * h + 16u, 16);
     }
 }
+__device__ __forceinline__ void il_scales(const RawQ6& r, uint32_t, uint32_t, float& s0, float& s1, float& nb)
+{
+    const float d = half_bits_to_float(r.d16);
+    s0 = d * (float)(int)(int8_t)(r.sc2 & 255u);
+    s1 = d * (float)(int)(int8_t)(r.sc2 >> 8);
+    nb = 0.0f;
+}
+__device__ __forceinline__ u32x4 il_expand(const RawQ6& r, uint32_t kc, uint32_t hf, int v, float s0, float s1, float)
+{
+    const uint32_t t = ((kc & 3u) & 1u) * 2u + hf;
+    const uint32_t lsh = (t & 2u) ? 4u : 0u;
+    const float s = v < 2 ? s0 : s1;
+    const float off = -32.0f * s;
+    const u32x4 ql = v < 2 ? r.a0 : r.a1, qh = v < 2 ? r.b0 : r.b1;
+    u32x4 out;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t lo = (ql[(v & 1) * 2 + j] >> lsh) & 0x0F0F0F0Fu;
+        const uint32_t hi = ((qh[(v & 1) * 2 + j] >> (2u * t)) & 0x03030303u) << 4;
+        const uint32_t q = lo | hi;   // four 6-bit stored values
+        const float f0 = fmaf(s, (float)(q & 255u), off);
+        const float f1 = fmaf(s, (float)((q >> 8) & 255u), off);
+        const float f2 = fmaf(s, (float)((q >> 16) & 255u), off);
+        const float f3 = fmaf(s, (float)(q >> 24), off);
+        out[j * 2] = pack_bf16(f0, f1);
+        out[j * 2 + 1] = pack_bf16(f2, f3);
+    }
+    return out;
+}
+
+template <int TYPE>
+__global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
+{
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int BM = 256, BN = 256, WAVES_N = 4, WM = 128, WN = 64, TM = 4, TN = 2;
+    constexpr int A_BYTES = BM * GEMM_LD, B_BYTES = BN * GEMM_LD;
+    constexpr int XROWS = 64;   // X rows per piece: 8 threads x 16 bytes per row, 4 pieces
+    using Raw = typename std::conditional<TYPE == KQ_TYPE_Q4_K, RawQ4, RawQ6>::type;
+    uint8_t* As = smem;
+    uint8_t* Bs = smem + 2 * A_BYTES;
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const uint32_t nk_all = p.K / GEMM_BK;
+    const uint32_t x_dst = (tid >> 3) * GEMM_LD + (tid & 7u) * 16u;
+    const uint32_t wrow = tid >> 1, whf = tid & 1u;
+    const uint32_t w_dst = wrow * GEMM_LD + whf * 64u;
+    const uint32_t a_src = (wm * WM + (lane & 31u)) * GEMM_LD + (lane >> 5) * 16u;
+    const uint32_t b_src = (wn * WN + (lane & 31u)) * GEMM_LD + (lane >> 5) * 16u;
+
+    // this workgroup's share of the walk: units [u, u_end), a unit = one k step of one tile
+    uint32_t u = blockIdx.x * p.units_per_wg;
+    const uint32_t u_end = min(u + p.units_per_wg, p.units);
+    while (u < u_end) {
+    const uint32_t tile = u / nk_all, k_first = u - tile * nk_all;
+    const uint32_t nk = min(nk_all - k_first, u_end - u);   // k steps of this segment
+    u += nk;
+        const uint32_t m0 = (tile / p.tiles_n) * BM, n0 = (tile % p.tiles_n) * BN;
+
+    const uint8_t* xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t m = min(m0 + i * XROWS + (tid >> 3), p.M - 1u);
+        xsrc[i] = (const uint8_t*)p.X + (size_t)m * p.K * 2u + (tid & 7u) * 16u;
+    }
+    const uint8_t* wsrc = p.W + (size_t)min(n0 + wrow, p.N - 1u) * p.row_stride_bytes;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // Raw registers: piece v of xr / w holds tile T(v) of the k walk.  Piece 0 runs one tile ahead of
+    // pieces 1..3 (it is converted in the slice after the barrier, the others in the three slices before).
+    u32x4 xr[4];
+    Raw w;
+    float s0, s1, nb;   // scales of the tile being converted
+    auto tile_at = [&](uint32_t t) { return k_first + min(t, nk - 1u); };   // k step t of the segment, clamped
+    auto load_x = [&](uint32_t t, int i) { xr[i] = *(const u32x4*)(xsrc[i] + (size_t)tile_at(t) * (GEMM_BK * 2)); };
+    auto read_ops = [&](uint32_t buf, int s, bf16x8 (&af)[TM], bf16x8 (&bfr)[TN]) {
+        const uint8_t* a = As + buf * A_BYTES + a_src + s * 32;
+        const uint8_t* b = Bs + buf * B_BYTES + b_src + s * 32;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[i] = *(const bf16x8*)(a + i * 32 * GEMM_LD);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bfr[j] = *(const bf16x8*)(b + j * 32 * GEMM_LD);
+    };
+    auto mfma_ops = [&](const bf16x8 (&af)[TM], const bf16x8 (&bfr)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    };
+    // piece v of tile t: X copy and 8 dequantised weights into LDS buffer t&1, then the registers of the
+    // piece are refilled from tile t+1 (a full step before they are converted)
+    auto convert_piece = [&](uint32_t t, int v) {
+        const uint32_t buf = t & 1u;
+        *(u32x4*)(As + buf * A_BYTES + x_dst + v * XROWS * GEMM_LD) = xr[v];
+        *(u32x4*)(Bs + buf * B_BYTES + w_dst + v * 16) = il_expand(w, tile_at(t), whf, v, s0, s1, nb);
+        load_x(t + 1u, v);
+        if (v == 1) il_load_q(wsrc, tile_at(t + 1u), whf, 0, w);
+        if (v == 3) il_load_q(wsrc, tile_at(t + 1u), whf, 1, w);
+    };
+    // the matrix instructions of a slice take turns with the conversion arithmetic; LDS reads go first
+    auto slice_schedule = [&]() {
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+#pragma unroll
+        for (int g = 0; g < TM * TN; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // prologue: tile 0 whole and piece 0 of tile 1 into LDS; registers end up holding pieces 1..3 of tile 1,
+    // piece 0 of tile 2 and the scales of tile 1
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_x(0, i);
+    il_load_head(wsrc, tile_at(0), whf, w);
+    il_load_q(wsrc, tile_at(0), whf, 0, w);
+    il_load_q(wsrc, tile_at(0), whf, 1, w);
+    il_scales(w, tile_at(0), whf, s0, s1, nb);
+    il_load_head(wsrc, tile_at(1), whf, w);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) convert_piece(0, v);
+    il_scales(w, tile_at(1), whf, s0, s1, nb);
+    il_load_head(wsrc, tile_at(2), whf, w);
+    convert_piece(1, 0);
+    __syncthreads();
+
+    bf16x8 af[2][TM], bfr[2][TN];
+    read_ops(0, 0, af[0], bfr[0]);
+    for (uint32_t kt = 0; kt < nk; ++kt) {
+        const uint32_t buf = kt & 1u;
+        // slices 0..2 of tile kt; pieces 1..3 of tile kt+1 go to the other buffer
+#pragma unroll
+        for (int s = 0; s < 3; ++s) {
+            read_ops(buf, s + 1, af[(s + 1) & 1], bfr[(s + 1) & 1]);
+            mfma_ops(af[s & 1], bfr[s & 1]);
+            convert_piece(kt + 1u, s + 1);
+            slice_schedule();
+        }
+        // every wave has now read all of tile kt and written its part of tile kt+1
+        __syncthreads();
+        // slice 3 of tile kt needs no LDS: its operands are in registers.  Behind it the first operands of
+        // tile kt+1 are fetched and piece 0 of tile kt+2 replaces tile kt in LDS.
+        read_ops(buf ^ 1u, 0, af[0], bfr[0]);
+        mfma_ops(af[1], bfr[1]);
+        il_scales(w, tile_at(kt + 2u), whf, s0, s1, nb);
+        il_load_head(wsrc, tile_at(kt + 3u), whf, w);
+        convert_piece(kt + 2u, 0);
+        slice_schedule();
+    }
+
+    // a tile walked in one piece is stored; a tile cut between workgroups is summed into Y, which the
+    // launcher cleared for exactly those tiles (the bias goes in with the segment that starts at k = 0)
+    if (nk == nk_all) store_acc<TM, TN, false>(p, acc, m0 + wm * WM, n0 + wn * WN, lane);
+    else store_acc<TM, TN, true>(p, acc, m0 + wm * WM, n0 + wn * WN, lane, k_first == 0u);
+    __syncthreads();   // the next segment's prologue overwrites LDS
+    }
+}
+
+// Clears the tiles of Y that the persistent kernel's cut points split: block b looks at the boundary
+// between workgroups b and b+1.
+__global__ __launch_bounds__(256) void gemm_clear_split_tiles_kernel(GemmParams p)
+{
+    const uint32_t nk_all = p.K / GEMM_BK;
+    const uint32_t cut = (blockIdx.x + 1u) * p.units_per_wg;
+    if (cut >= p.units || cut % nk_all == 0u) return;
+    const uint32_t tile = cut / nk_all;
+        const uint32_t m0 = (tile / p.tiles_n) * 256u, n0 = (tile % p.tiles_n) * 256u;
+    const uint32_t col = (threadIdx.x & 63u) * 4u, row0 = threadIdx.x >> 6;
+    for (uint32_t r = row0; r < 256u; r += 4u) {
+        const uint32_t m = m0 + r;
+        if (m >= p.M) break;
+        float* y = p.Y + (size_t)m * p.ldy + n0 + col;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (n0 + col + c < p.N) y[c] = 0.0f;
+    }
+}
+
 
 bool gemm_bf16_supported(const MatmulArgs& a)
 {
@@ -304,9 +583,34 @@ static hipError_t launch_gemm(const GemmParams& p, hipStream_t s)
     return hipGetLastError();
 }
 
-hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, hipStream_t s)
+// 256-tile kernel.  even_shares: cut the walk into one equal share per CU; else one tile per workgroup.
+template <int TYPE>
+static hipError_t launch_gemm_persistent(GemmParams p, bool even_shares, hipStream_t s)
 {
-    GemmParams p;
+    constexpr size_t shmem = 2 * (size_t)(256 + 256) * GEMM_LD;
+    auto kern = gemm_bf16_sk_kernel<TYPE>;
+    static bool raised = false;   // per instantiation
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    const uint32_t nk = p.K / GEMM_BK;
+    p.tiles_n = (p.N + 255u) / 256u;
+    const uint32_t tiles = ((p.M + 255u) / 256u) * p.tiles_n;
+    p.units = tiles * nk;
+    const uint32_t cus = device_cu_count();
+    p.units_per_wg = even_shares ? (p.units + cus - 1u) / cus : nk;
+    const uint32_t wgs = (p.units + p.units_per_wg - 1u) / p.units_per_wg;
+    if (wgs > 1u && p.units_per_wg % nk != 0u)
+        hipLaunchKernelGGL(gemm_clear_split_tiles_kernel, dim3(wgs - 1u), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(kern, dim3(wgs), dim3(512), shmem, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, hipStream_t s)
+{
+    GemmParams p{};
     p.X = (const uint16_t*)a.X;
     p.W = a.W;
     p.bias = a.bias;
@@ -315,11 +619,20 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, hipStream_t s)
     p.n_blocks = a.n_blocks;
     p.row_stride_bytes = a.row_stride_bytes;
     p.ldy = a.ldy;
-    // big tiles when they still give every CU work, else 128 x 128
-    const uint64_t big = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 255u) / 256u);
-    const bool use_big = tile == 256 || (tile == 0 && big >= 256u);
     const bool q4 = a.type == KQ_TYPE_Q4_K;
-    if (use_big) return q4 ? launch_gemm<KQ_TYPE_Q4_K, 256, 256, 8>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 256, 256, 8>(p, s);
+    // Measured on M = 2048: 256-tiles win once they occupy more than half the CUs.  Below that, a long K is
+    // worth cutting (the epilogue of a cut tile costs about 15 k steps), a short one runs on 128-tiles, two
+    // workgroups per CU.  With many tiles per CU, equal shares also remove the ragged last round.
+    const uint32_t cus = device_cu_count(), nk = a.K / GEMM_BK;
+    const uint64_t big = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 255u) / 256u);
+    bool use_big, even;
+    if (big * 2u > cus) { use_big = true; even = big >= 8ull * cus; }
+    else { use_big = nk >= 128u && big * nk >= 16ull * cus; even = true; }
+    if (tile == 256) use_big = true;
+    if (tile == 128) use_big = false;
+    if (split == 1) even = false;
+    if (split == 2) even = true;
+    if (use_big) return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, even, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, even, s);
     return q4 ? launch_gemm<KQ_TYPE_Q4_K, 128, 128, 4>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 128, 128, 4>(p, s);
 }
 

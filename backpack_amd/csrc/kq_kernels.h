@@ -81,8 +81,23 @@ hipError_t launch_moe_combine(const float* down, const float* wt, float* out, ui
                               hipStream_t s);
 
 // Prefill GEMM on the matrix cores: X bf16 [M,K], Y f32.  tile = 0 (automatic),
-// 128 or 256 (square workgroup tile).
+// 128 or 256 (square workgroup tile); split (256-tile only) = 0 (automatic),
+// 1 (one tile per workgroup) or 2 (the walk cut into equal shares per CU).
 bool gemm_bf16_supported(const MatmulArgs& a);
-hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, hipStream_t s);
+hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, hipStream_t s);
+
+// Compute units of the current device (cached per device id).
+inline uint32_t device_cu_count()
+{
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256u;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return (uint32_t)cached[dev];
+}
 
 }  // namespace kq

@@ -470,19 +470,7 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
     asm volatile("s_waitcnt vmcnt(0)");   // the ring's last refills land before the wave ends
 }
 
-// Compute units of the current device (cached per device id).
-static uint32_t cu_count()
-{
-    static int cached[64];
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256u;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n;
-    }
-    return (uint32_t)cached[dev];
-}
+static uint32_t cu_count() { return device_cu_count(); }
 
 // Workgroups for a kernel whose workgroups walk rows g, g + wgs, ...: a whole
 // multiple of the CU count, so that every CU gets the same number of workgroups,

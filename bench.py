@@ -52,6 +52,10 @@ def parse():
     ap.add_argument("--moe", action="store_true",
                     help="also time the Qwen3-30B-A3B-shaped routed-expert FFN at T = 1 and T = 256")
     ap.add_argument("--all", action="store_true", help="--prefill --verify --moe")
+    ap.add_argument("--gemm-tile", type=int, default=0,
+                    help="force the prefill GEMM tile (0 = the library's own choice)")
+    ap.add_argument("--gemm-split", type=int, default=0,
+                    help="256-tile prefill GEMM: 1 = one tile per workgroup, 2 = equal shares per CU (0 = automatic)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the M=2048 prefill GEMM leg and print its figures (for profiling)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -203,6 +207,10 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
+    if args.gemm_tile:
+        capi.set_option("gemm_tile", args.gemm_tile)
+    if args.gemm_split:
+        capi.set_option("gemm_split", args.gemm_split)
     if args.prefill_only:
         print(json.dumps({"prefill": prefill_leg()}))
         return

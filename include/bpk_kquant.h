@@ -192,7 +192,10 @@ BPK_API int bpk_force_kernel(int family);
  * lanes-along-K GEMV; "gemv_waves": waves per workgroup of the row-per-lane
  * kernels (2, 4 or 8); "gemv_depth": rows a wave of the lanes-along-K GEMV
  * keeps in flight (1, 2 or 4); "gemm_tile": square workgroup tile of the bf16
- * GEMM (128 or 256).  0 = automatic. */
+ * GEMM (128 or 256); "gemm_split": how the 256-tile GEMM hands out work
+ * (1 = one tile per workgroup, 2 = the walk over tiles and k steps cut into
+ * equal shares per compute unit, tiles cut between workgroups are summed with
+ * fp32 atomics).  0 = automatic. */
 BPK_API int bpk_set_option(const char *name, int value);
 
 #ifdef __cplusplus

@@ -300,6 +300,17 @@ GEMM_SHAPES = [
     (Q6_K, 256, 256, 768, 256),      # odd block count: rows only 8-byte aligned
     (Q6_K, 190, 260, 1024, 128),
     (Q6_K, 512, 512, 4096, 0),
+    # 256-tile with the walk cut into equal shares per CU (tiles summed with atomics)
+    (Q4_K, 256, 256, 256, 258),
+    (Q4_K, 300, 520, 768, 258),
+    (Q4_K, 512, 1024, 4096, 258),
+    (Q4_K, 2048, 1024, 1024, 258),   # 32 tiles x 16 steps on 256 CUs: two steps per workgroup
+    (Q6_K, 256, 256, 768, 258),
+    (Q6_K, 190, 260, 1024, 258),
+    (Q6_K, 512, 512, 4096, 258),
+    # 256-tile, one tile per workgroup
+    (Q4_K, 512, 1024, 4096, 257),
+    (Q6_K, 300, 520, 768, 257),
 ]
 
 
@@ -319,13 +330,15 @@ def test_gemm_bf16_vs_oracle(gpu, kqo, type_, M, N, K, tile):
     bits = _bf16_bits(X)
     bias = rng.standard_normal(N).astype(np.float32)
     xd = torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
-    capi.set_option("gemm_tile", tile)
+    capi.set_option("gemm_tile", min(tile, 256))
+    capi.set_option("gemm_split", max(tile - 256, 0))   # 257 / 258: the 256-tile with split 1 / 2
     try:
         _say("gemm", type_, M, N, K, tile)
         got = kquant.matmul(xd, w, bias=gpu.dev(bias)).cpu().numpy()
         assert capi.last_kernel() == "gemm_bf16"
     finally:
         capi.set_option("gemm_tile", 0)
+        capi.set_option("gemm_split", 0)
     Xw = (bits.astype(np.uint32) << 16).view(np.float32)
     cpu = kqo.matmul(type_, Xw, packed, N, K, bias=bias)        # the reference's fp32 CPU path
     err = np.abs(got.astype(np.float64) - cpu)
