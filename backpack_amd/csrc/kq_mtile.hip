@@ -47,6 +47,14 @@ typedef float t_f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t t_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t t_u32x2 __attribute__((ext_vector_type(2)));
 
+// Orders a wave's own LDS traffic (writes of a staging pass against the reads around it); no s_barrier.
+__device__ __forceinline__ void wave_window_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 constexpr int MT_KC = 4;                       // superblocks of X staged at a time
 constexpr int MT_XA_BYTES = MT_KC * 8 * 2 * 1024;   // [block][sub-block][hi/lo][lane] 16 B
 constexpr int MT_XS_FLOATS = MT_KC * 8 * 16;        // [block][sub-block][token]
@@ -95,14 +103,15 @@ struct MtileStager {
             xrow = p.x_per_slot ? pr : pr / p.k_slots;
         }
     }
-    // requests the chunk's elements (nothing for tokens beyond M or superblocks beyond K)
+    // requests the chunk's elements (nothing for tokens beyond M; superblocks beyond K re-read the last
+    // one, which is parked but never multiplied)
     __device__ __forceinline__ void fetch(const MtileParams& p, uint32_t c0)
     {
-        const uint32_t b = c0 + bb;
-        const bool live = live_token && b < p.n_blocks;
-        const float4* src = (const float4*)(p.X + (size_t)(live ? xrow : 0u) * p.K + (size_t)(live ? b : 0u) * KQ_QK + sub * EPT);
+        if (!live_token) return;   // wave-uniform for whole waves of dead tokens
+        const uint32_t b = min(c0 + bb, p.n_blocks - 1u);
+        const float4* src = (const float4*)(p.X + (size_t)xrow * p.K + (size_t)b * KQ_QK + sub * EPT);
 #pragma unroll
-        for (int i = 0; i < EPT / 4; ++i) v[i] = live ? src[i] : float4{0, 0, 0, 0};
+        for (int i = 0; i < EPT / 4; ++i) v[i] = src[i];
     }
     // converts what fetch() brought and parks it in LDS (slots of tokens beyond M stay zero)
     __device__ __forceinline__ void park(uint8_t* xa, float* xs, float* xinv)
@@ -289,6 +298,46 @@ __device__ __forceinline__ void q6k_mtile_block(const Q6TileW& w, const uint8_t*
     tot.w += fmaf(d24 * inv.w, U.w, -(d32 * V.w));
 }
 
+// Weights travel HBM -> registers -> LDS in 16-byte units that are consecutive along a row, so every cache
+// line is fetched once and whole (a lane fetching only the 8-byte pieces its operands need makes each line
+// cross the L2 -> L1 path five times).  A wave stages SPAN bytes of each of its 16 rows in a private LDS
+// window (row pitch PITCH, chosen so that the 16 rows start in different banks) and then reads its operand
+// pieces from there.
+template <int SPAN, int PITCH>
+struct MtileWStage {
+    static constexpr int UPR = (SPAN + 15) / 16;            // units per row
+    static constexpr int NU = (16 * UPR + 63) / 64;         // units per lane
+    const uint8_t* src[NU];
+    uint32_t dst[NU], col[NU];
+    t_u32x4 raw[NU];
+    __device__ __forceinline__ void init(const uint8_t* wmat, uint32_t row0, uint32_t N, uint32_t row_stride, uint32_t lane)
+    {
+#pragma unroll
+        for (int i = 0; i < NU; ++i) {
+            const uint32_t u = min((uint32_t)i * 64u + lane, 16u * UPR - 1u);   // spare lanes repeat the last unit
+            const uint32_t r = u / UPR, c = u - r * UPR;
+            src[i] = wmat + (size_t)min(row0 + r, N - 1u) * row_stride;
+            col[i] = c * 16u;
+            dst[i] = r * PITCH + c * 16u;
+        }
+    }
+    // requests bytes [off, off + SPAN) of every row; a unit that would start at or beyond row_bytes reads
+    // the row's last 16 bytes instead (it belongs to superblocks that do not exist and are not multiplied)
+    __device__ __forceinline__ void load(uint32_t off, uint32_t row_bytes)
+    {
+#pragma unroll
+        for (int i = 0; i < NU; ++i) {
+            const uint32_t o = off + col[i];
+            __builtin_memcpy(&raw[i], src[i] + (o < row_bytes ? o : row_bytes - 16u), 16);
+        }
+    }
+    __device__ __forceinline__ void store(uint8_t* window) const
+    {
+#pragma unroll
+        for (int i = 0; i < NU; ++i) *(t_u32x4*)(window + dst[i]) = raw[i];
+    }
+};
+
 template <int TYPE, int NW, int R>
 __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
 {
@@ -315,15 +364,30 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
     const uint32_t tile = R == 1 ? blockIdx.x : blockIdx.x * p.tiles_per_wg + wave;
     const uint32_t row = has_tile ? tile * 16u + (lane & 15u) : p.N;
     const uint32_t kq = lane >> 4;
-    const uint8_t* wrow = wmat + (size_t)min(row, p.N - 1u) * p.row_stride_bytes;
-    // superblocks of a chunk this wave takes: all (R == NW), or wave, wave + NW, ... (R == 1)
-    constexpr int BPC = R == 1 ? (MT_KC + NW - 1) / NW : MT_KC;
 
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
     constexpr uint32_t BB = Q6 ? KQ_Q6K_BYTES : KQ_Q4K_BYTES;
+    // A wave with a tile of its own stages two superblocks of its 16 rows at a time (two passes per chunk);
+    // waves that share a tile stage the one superblock of the chunk that is theirs.
+    constexpr int HB = R == 1 ? 1 : 2;                        // superblocks per staging pass
+    constexpr int SPAN = HB * BB;
+    constexpr int PITCH = Q6 ? (HB == 1 ? 240 : 464) : (HB == 1 ? 160 : 304);
+    constexpr int PASSES = R == 1 ? 1 : MT_KC / HB;
+    using WStage = MtileWStage<SPAN, PITCH>;
+    static_assert(PITCH >= WStage::UPR * 16 && PITCH % 16 == 0, "window row holds the staged units");
+    uint8_t* wwin = smem + MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4 + wave * (16 * PITCH);
+    const uint32_t row_bytes = p.n_blocks * BB;
+    WStage ws[PASSES];
+#pragma unroll
+    for (int h = 0; h < PASSES; ++h) ws[h].init(wmat, has_tile ? tile * 16u : 0u, p.N, p.row_stride_bytes, lane);
+    // first superblock of staging pass h of the chunk at c0
+    auto pass_block = [&](uint32_t c0, int h) { return c0 + (R == 1 ? wave : (uint32_t)h * HB); };
+
     MtileStager<64 * NW, Q6> stager;
     stager.init(p, rec, count);
     stager.fetch(p, 0);
+#pragma unroll
+    for (int h = 0; h < PASSES; ++h) ws[h].load(pass_block(0, h) * BB, row_bytes);
     // slots of tokens beyond M, and for Q6_K the halves that must read as zero, are cleared once
     for (uint32_t i = threadIdx.x; i < (MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4) / 16; i += 64 * NW)
         ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
@@ -331,37 +395,36 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
 
     t_f32x4 tot = {0, 0, 0, 0};
     for (uint32_t c0 = 0; c0 < p.n_blocks; c0 += MT_KC) {
-        // the chunk's weights are requested first, so that their latency runs
-        // under the conversion of X
-        t_u32x4 hdr[BPC];
-        t_u32x2 w[BPC][4];
-        Q6TileW w6[BPC];
-#pragma unroll
-        for (int i = 0; i < BPC; ++i) {
-            const uint32_t bb = R == 1 ? wave + i * NW : i;
-            const uint32_t b = min(c0 + bb, p.n_blocks - 1u);
-            const uint8_t* blk = wrow + (size_t)b * BB;
-            if constexpr (Q6) {
-                q6k_mtile_load(blk, kq, w6[i]);
-            } else {
-                hdr[i] = *(const t_u32x4*)blk;
-#pragma unroll
-                for (int g = 0; g < 4; ++g) w[i][g] = *(const t_u32x2*)(blk + 16u + 32u * g + 8u * kq);
-            }
-        }
         stager.park(xa, xs, xinv);
+        ws[0].store(wwin);
         __syncthreads();
-        // the next chunk of X travels while this one is multiplied
-        if (c0 + MT_KC < p.n_blocks) stager.fetch(p, c0 + MT_KC);
-        if (has_tile) {
+        // the next chunk of X and of the weights travels while this one is multiplied
+        stager.fetch(p, c0 + MT_KC);
+        ws[0].load(pass_block(c0 + MT_KC, 0) * BB, row_bytes);
 #pragma unroll
-            for (int i = 0; i < BPC; ++i) {
-                const uint32_t bb = R == 1 ? wave + i * NW : i;
-                if (bb < MT_KC && c0 + bb < p.n_blocks) {
-                    if constexpr (Q6)
-                        q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
-                    else
-                        q4k_mtile_block(hdr[i], w[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+        for (int h = 0; h < PASSES; ++h) {
+            if (h > 0) {
+                wave_window_fence();          // this wave's reads of the previous pass are done
+                ws[h].store(wwin);
+                ws[h].load(pass_block(c0 + MT_KC, h) * BB, row_bytes);
+                wave_window_fence();
+            }
+#pragma unroll
+            for (int i = 0; i < HB; ++i) {
+                const uint32_t bb = R == 1 ? wave : (uint32_t)(h * HB + i);
+                if (has_tile && bb < MT_KC && c0 + bb < p.n_blocks) {
+                    const uint8_t* blk = wwin + (lane & 15u) * PITCH + i * BB;
+                    if constexpr (Q6) {
+                        Q6TileW w6;
+                        q6k_mtile_load(blk, kq, w6);
+                        q6k_mtile_block(w6, xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                    } else {
+                        const t_u32x4 hdr = *(const t_u32x4*)blk;
+                        t_u32x2 w[4];
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) w[g] = *(const t_u32x2*)(blk + 16u + 32u * g + 8u * kq);
+                        q4k_mtile_block(hdr, w, xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                    }
                 }
             }
         }
@@ -414,7 +477,9 @@ bool mtile_supported(const MatmulArgs& a)
 template <int TYPE, int NW, int R>
 static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s)
 {
-    constexpr size_t shmem = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * sizeof(float);
+    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
+    constexpr int PITCH = Q6 ? (R == 1 ? 240 : 464) : (R == 1 ? 160 : 304);   // as in the kernel
+    constexpr size_t shmem = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * sizeof(float) + (size_t)NW * 16 * PITCH;
     auto kern = mtile_kernel<TYPE, NW, R>;
     static bool raised = false;   // per instantiation
     if (!raised) {
