@@ -292,7 +292,7 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     if (t_family == 6 && !mtile_ok) return fail(BPK_ERR_SHAPE, "16x16 tile kernel cannot serve this call");
     if (t_family == 6 || (t_family == 0 && mtile_ok && M >= 3 && M <= 255)) {
         t_kernel = "mtile";
-        e = kq::launch_mtile(a, s);
+        e = kq::launch_mtile(a, st->split, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
     }
     if (t_family == 5 && !stream_ok) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");

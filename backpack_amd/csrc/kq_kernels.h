@@ -56,7 +56,7 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
 
 // 16-row x 16-token MFMA tiles for M = 2..16 (dense): weights read once for all tokens.
 bool mtile_supported(const MatmulArgs& a);
-hipError_t launch_mtile(const MatmulArgs& a, hipStream_t s);
+hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s);
 // grouped by expert: records {expert, count, pair ids...} of up to cap pairs, as launch_moe_group
 // writes them with sets = cap / 2; cap at most mtile_group_cap(type)
 uint32_t mtile_group_cap(int type);

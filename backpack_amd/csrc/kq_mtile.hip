@@ -67,6 +67,12 @@ struct MtileParams {
     float* Y;
     uint32_t M, N, K, n_blocks, row_stride_bytes, y_offset, ldy;
     uint32_t tiles_per_wg;   // R == NW kernels: waves below this own a tile, the others only help convert X
+    // K split over blockIdx.z (dense calls): split z walks chunks [z * chunks_per_split, ...); each split
+    // leaves its partial tile in partial[z][token][tile row], the last workgroup of a row group to arrive
+    // adds them in split order
+    uint32_t n_splits, chunks_per_split;
+    float* partial;
+    uint32_t* counters;      // one per blockIdx.x, zero between launches
     // grouped mode (tiles != nullptr): blockIdx.y walks records {expert, count, pair ids...} of up to
     // 16 (Q4_K) / 8 (Q6_K) (token, slot) pairs that share an expert; N is the rows of one expert
     const uint32_t* tiles;
@@ -383,18 +389,21 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
     // first superblock of staging pass h of the chunk at c0
     auto pass_block = [&](uint32_t c0, int h) { return c0 + (R == 1 ? wave : (uint32_t)h * HB); };
 
+    const uint32_t c_begin = blockIdx.z * p.chunks_per_split * MT_KC;
+    const uint32_t c_end = min(p.n_blocks, c_begin + p.chunks_per_split * MT_KC);
+
     MtileStager<64 * NW, Q6> stager;
     stager.init(p, rec, count);
-    stager.fetch(p, 0);
+    stager.fetch(p, c_begin);
 #pragma unroll
-    for (int h = 0; h < PASSES; ++h) ws[h].load(pass_block(0, h) * BB, row_bytes);
+    for (int h = 0; h < PASSES; ++h) ws[h].load(pass_block(c_begin, h) * BB, row_bytes);
     // slots of tokens beyond M, and for Q6_K the halves that must read as zero, are cleared once
     for (uint32_t i = threadIdx.x; i < (MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4) / 16; i += 64 * NW)
         ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
     __syncthreads();
 
     t_f32x4 tot = {0, 0, 0, 0};
-    for (uint32_t c0 = 0; c0 < p.n_blocks; c0 += MT_KC) {
+    for (uint32_t c0 = c_begin; c0 < c_end; c0 += MT_KC) {
         stager.park(xa, xs, xinv);
         ws[0].store(wwin);
         __syncthreads();
@@ -412,7 +421,7 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
 #pragma unroll
             for (int i = 0; i < HB; ++i) {
                 const uint32_t bb = R == 1 ? wave : (uint32_t)(h * HB + i);
-                if (has_tile && bb < MT_KC && c0 + bb < p.n_blocks) {
+                if (has_tile && bb < MT_KC && c0 + bb < c_end) {
                     const uint8_t* blk = wwin + (lane & 15u) * PITCH + i * BB;
                     if constexpr (Q6) {
                         Q6TileW w6;
@@ -449,6 +458,38 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
         tot.z += __shfl_xor(tot.z, 32, 64);
         tot.w += __shfl_xor(tot.w, 32, 64);
     }
+    if (R == NW && p.n_splits > 1) {   // (only the wave-per-tile kernels are launched with splits)
+        // Same hand-over as the split GEMV: partial sums go out as agent-scope stores, the workgroup takes a
+        // ticket once they are acknowledged, and the last one in reads all of them back past the
+        // non-coherent cache levels and adds them in split order.
+        const size_t plane = (size_t)gridDim.x * p.tiles_per_wg * 16u;   // rows of all tiles
+        const bool mine = has_tile && (!Q6 || kq < 2u);
+        const uint32_t prow = tile * 16u + (lane & 15u);
+        if (mine) {
+            const float t4[4] = {tot.x, tot.y, tot.z, tot.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                __hip_atomic_store(p.partial + ((size_t)blockIdx.z * 16u + 4u * kq + r) * plane + prow, t4[r], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        uint32_t* ticket = (uint32_t*)(smem + 16);
+        if (threadIdx.x == 0)
+            *ticket = __hip_atomic_fetch_add(&p.counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*ticket != p.n_splits - 1u) return;   // whole workgroup
+        if (mine) {
+            float t4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (uint32_t z = 0; z < p.n_splits; ++z)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    t4[r] += __hip_atomic_load(p.partial + ((size_t)z * 16u + 4u * kq + r) * plane + prow, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+            tot = t_f32x4{t4[0], t4[1], t4[2], t4[3]};
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(&p.counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     if (row < p.N && (!Q6 || kq < 2u)) {
         const float bias = p.bias ? p.bias[row] : 0.0f;
         const float t4[4] = {tot.x, tot.y, tot.z, tot.w};
@@ -475,7 +516,7 @@ bool mtile_supported(const MatmulArgs& a)
 }
 
 template <int TYPE, int NW, int R>
-static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s)
+static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s, uint32_t wgs_z = 1)
 {
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
     constexpr int PITCH = Q6 ? (R == 1 ? 240 : 464) : (R == 1 ? 160 : 304);   // as in the kernel
@@ -487,7 +528,7 @@ static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t 
         if (e != hipSuccess) return e;
         raised = true;
     }
-    hipLaunchKernelGGL(kern, dim3(wgs, wgs_y), dim3(64 * NW), shmem, s, p);
+    hipLaunchKernelGGL(kern, dim3(wgs, wgs_y, wgs_z), dim3(64 * NW), shmem, s, p);
     return hipGetLastError();
 }
 
@@ -510,6 +551,7 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
     p.tiles = tiles;
     p.n_tiles = n_tiles;
     p.tile_stride = 2u + cap;
+    p.n_splits = 1; p.chunks_per_split = (a.n_blocks + MT_KC - 1) / MT_KC; p.partial = nullptr; p.counters = nullptr;
     p.k_slots = a.k_slots;
     p.x_per_slot = a.x_per_slot;
     // a wave per 16-row tile of the expert, 8 tiles per workgroup: X of the record is converted once per 128 rows
@@ -520,12 +562,38 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
                                   : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8>(p, wgs, tiles_bound, s);
 }
 
-hipError_t launch_mtile(const MatmulArgs& a, hipStream_t s)
+hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s)
 {
     const bool q6 = a.type == KQ_TYPE_Q6_K;
     // Q6_K tiles hold 8 tokens: more are served in groups of 8, each reading the weights again
     const uint32_t group = q6 ? 8u : 16u;
     const uint32_t tiles = (a.N + 15u) / 16u;
+    const uint32_t n_chunks = (a.n_blocks + MT_KC - 1) / MT_KC;
+    const uint32_t cus = device_cu_count();
+
+    // Work split.  A wave per tile, tpw tiles per workgroup (they share the conversion of X), and K cut into
+    // n_splits runs of whole chunks when the rows alone give too few workgroups.  Candidates are priced as
+    // rounds x (chunks walked + 1.5 for launch, prologue and fold), a partly idle last round costing half its
+    // idle share extra; one tile per workgroup with the waves taking different superblocks is the fallback
+    // for matrices of a few rows.
+    uint32_t best_tpw = 0, best_splits = 1, best_cps = n_chunks;
+    float best_cost = 1e30f;
+    for (uint32_t tpw = 8; tpw >= 4; --tpw) {
+        const uint32_t groups = (tiles + tpw - 1u) / tpw;
+        for (uint32_t splits = 1; splits <= n_chunks && splits <= 16u; ++splits) {
+            const uint32_t cps = (n_chunks + splits - 1u) / splits;
+            if ((splits - 1u) * cps >= n_chunks) continue;   // a split would be empty
+            if (splits > 1u && ((size_t)splits * 16u * groups * tpw * 16u > sc.capacity_floats || groups > sc.n_counters)) continue;
+            const uint32_t wgs = groups * splits, rounds = (wgs + cus - 1u) / cus;
+            const float idle = 1.0f - (float)wgs / (float)(rounds * cus);
+            const float cost = (float)rounds * ((float)cps + 1.5f) * (1.0f + 0.5f * idle);
+            if (cost < best_cost) { best_cost = cost; best_tpw = tpw; best_splits = splits; best_cps = cps; }
+        }
+    }
+    // one tile per workgroup of 4 waves, two workgroups per CU: every workgroup converts all of X itself
+    const float shared_rounds = (float)((tiles + 2u * cus - 1u) / (2u * cus));
+    const bool shared_tile = shared_rounds * ((float)n_chunks * 1.25f + 1.5f) < best_cost;
+
     for (uint32_t m0 = 0; m0 < a.M; m0 += group) {
         MtileParams p;
         p.X = (const float*)a.X + (size_t)m0 * a.K;
@@ -540,17 +608,17 @@ hipError_t launch_mtile(const MatmulArgs& a, hipStream_t s)
         p.ldy = a.ldy;
         p.tiles_per_wg = 1;
         p.tiles = nullptr; p.n_tiles = nullptr; p.tile_stride = 0; p.k_slots = 1; p.x_per_slot = 0;
+        p.n_splits = 1; p.chunks_per_split = n_chunks; p.partial = sc.partial; p.counters = sc.counters;
         hipError_t e;
-        // a wave per tile once that still gives a couple of hundred workgroups; otherwise one tile per workgroup
-        if (tiles >= 7u * 200u) {
-            // 7 or 8 tiles per workgroup, whichever leaves the last round of workgroups fuller on 256 CUs
-            const uint32_t w7 = (tiles + 6u) / 7u, w8 = (tiles + 7u) / 8u;
-            const uint32_t fill7 = (w7 + 255u) / 256u * 256u - w7, fill8 = (w8 + 255u) / 256u * 256u - w8;
-            p.tiles_per_wg = fill7 * 7u < fill8 * 8u ? 7u : 8u;
-            const uint32_t wgs = (tiles + p.tiles_per_wg - 1u) / p.tiles_per_wg;
-            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8>(p, wgs, 1, s) : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8>(p, wgs, 1, s);
-        } else {
+        if (shared_tile) {
             e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 4, 1>(p, tiles, 1, s) : launch_mtile_one<KQ_TYPE_Q4_K, 4, 1>(p, tiles, 1, s);
+        } else {
+            p.tiles_per_wg = best_tpw;
+            p.n_splits = best_splits;
+            p.chunks_per_split = best_cps;
+            const uint32_t wgs = (tiles + best_tpw - 1u) / best_tpw;
+            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8>(p, wgs, 1, s, best_splits)
+                   : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8>(p, wgs, 1, s, best_splits);
         }
         if (e != hipSuccess) return e;
     }

@@ -128,6 +128,10 @@ SHAPES = [
     (Q6_K, 21, 200, 1024),
     (Q4_K, 16, 22500, 512),     # tile kernel, a wave per tile (7 or 8 tiles per workgroup), ragged last tile
     (Q6_K, 5, 23001, 768),
+    (Q4_K, 16, 6144, 4096),     # tile kernel with K cut over workgroups (4 runs of one chunk), partials folded by the last
+    (Q4_K, 6, 4100, 5376),      # ... 21 superblocks: runs of unequal length, the last with a partial chunk
+    (Q6_K, 5, 4096, 14336),     # ... 7 runs of two chunks
+    (Q6_K, 12, 1000, 7168),     # ... two token groups through the same scratch
 ]
 
 
