@@ -542,18 +542,18 @@ __global__ __launch_bounds__(256) void gemm_clear_split_tiles_kernel(GemmParams 
     const uint32_t cut = (blockIdx.x + 1u) * p.units_per_wg;
     if (cut >= p.units || cut % nk_all == 0u) return;
     const uint32_t tile = cut / nk_all;
-        const uint32_t m0 = (tile / p.tiles_n) * 256u, n0 = (tile % p.tiles_n) * 256u;
-    const uint32_t col = (threadIdx.x & 63u) * 4u, row0 = threadIdx.x >> 6;
-    for (uint32_t r = row0; r < 256u; r += 4u) {
-        const uint32_t m = m0 + r;
-        if (m >= p.M) break;
-        float* y = p.Y + (size_t)m * p.ldy + n0 + col;
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-            if (n0 + col + c < p.N) y[c] = 0.0f;
+    const uint32_t m0 = (tile / p.tiles_n) * 256u, n0 = (tile % p.tiles_n) * 256u;
+    const uint32_t rows = min(256u, p.M - m0);
+    if (n0 + 256u <= p.N && (((uintptr_t)p.Y | ((uintptr_t)p.ldy * 4u)) & 15u) == 0u) {
+        // whole 1 KB rows, 16 bytes per lane: a wave clears a row per store
+        float4* y = (float4*)(p.Y + (size_t)m0 * p.ldy + n0) + (threadIdx.x & 63u);
+        for (uint32_t r = threadIdx.x >> 6; r < rows; r += 4u) y[(size_t)r * (p.ldy / 4u)] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+    } else {
+        const uint32_t n = n0 + threadIdx.x;
+        if (n < p.N)
+            for (uint32_t r = 0; r < rows; ++r) p.Y[(size_t)(m0 + r) * p.ldy + n] = 0.0f;
     }
 }
-
 
 bool gemm_bf16_supported(const MatmulArgs& a)
 {
