@@ -111,7 +111,9 @@ BPK_API int bpk_weight_destroy(bpk_weight *w);
  *   Y[m*N + y_offset + n] = bias[n] + sum_k X[m*K + k] * dequant(W)[n, k]
  *
  * X: f32 [M,K] (device).  W: packed rows (device, 4-byte aligned; 16-byte
- * aligned rows take the fast kernels).  bias: f32 [N] or NULL (= zeros).
+ * aligned rows take the fast kernels).  Q6_K blocks are 210 bytes and are
+ * fetched in 16-byte pieces: the buffer must stay readable for 16 bytes past
+ * the end of the last row (bpk_weight_create allocates them).  bias: f32 [N] or NULL (= zeros).
  * Y: f32, caller-owned, not cleared.  fp32 accumulation throughout. */
 BPK_API int bpk_kq_matmul(int type, const float *X, const void *W,
                           const float *bias, float *Y, uint32_t M, uint32_t N,
