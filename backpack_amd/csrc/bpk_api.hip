@@ -470,21 +470,25 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
                              kq::gemv_stream_supported(a) && kq::gemv_stream_supported(d);
     if (stream_path) {
         // a handful of pairs (decode): one lanes-along-K matvec per pair, no grouping pass
+        // gate and up in one launch (they read the same x), the activation folded into down's load of x
         t_kernel = "moe_ffn_stream";
+        a.W2 = (const uint8_t*)up; a.Y2 = U;
         e = kq::launch_gemv_stream(a, t_gemv, s);
-        a.W = (const uint8_t*)up; a.Y = U;
-        if (e == hipSuccess) e = kq::launch_gemv_stream(a, t_gemv, s);
-        if (e == hipSuccess) e = kq::launch_moe_silu_mul(G, U, G, (size_t)P * inter, s);
+        d.X2 = U;
         if (e == hipSuccess) e = kq::launch_gemv_stream(d, t_gemv, s);
     } else if (tile_path) {
-        // two or more pairs per expert on average: records of 8 pairs, every expert matrix read once per record
+        // two or more pairs per expert on average: records of 8 pairs (16 from four pairs per expert on),
+        // every expert matrix read once per record (Q6_K: once per 8 pairs of it)
         t_kernel = "moe_ffn_mtile";
-        e = kq::launch_moe_group(expert_idx, P, n_experts, 4, tiles, n_tiles, s);
-        if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, bound8, 8, s);
+        const bool wide = (uint64_t)P >= 4ull * n_experts && kq::moe_tiles_bound(P, n_experts, 8) <= 65535u;
+        const int rsets = wide ? 8 : 4;
+        const uint32_t rbound = kq::moe_tiles_bound(P, n_experts, rsets), rcap = 2u * (uint32_t)rsets;
+        e = kq::launch_moe_group(expert_idx, P, n_experts, rsets, tiles, n_tiles, s);
+        if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, rbound, rcap, s);
         a.W = (const uint8_t*)up; a.Y = U;
-        if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, bound8, 8, s);
+        if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, rbound, rcap, s);
         if (e == hipSuccess) e = kq::launch_moe_silu_mul(G, U, G, (size_t)P * inter, s);
-        if (e == hipSuccess) e = kq::launch_mtile_grouped(d, tiles, n_tiles, bound8, 8, s);
+        if (e == hipSuccess) e = kq::launch_mtile_grouped(d, tiles, n_tiles, rbound, rcap, s);
     } else if (fast) {
         t_kernel = "moe_ffn_mrow";
         e = kq::launch_moe_group(expert_idx, P, n_experts, sets, tiles, n_tiles, s);

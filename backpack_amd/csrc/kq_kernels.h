@@ -21,6 +21,11 @@ struct MatmulArgs {
     const uint32_t* expert_idx;
     uint32_t k_slots;
     int x_per_slot;
+    // fusions of the MoE FFN, honoured by the grouped lanes-along-K launch only: a twin matrix W2 of the
+    // same shape whose products go to Y2 (gate and up in one launch), and X2: x = silu(X) * X2
+    const uint8_t* W2;
+    float* Y2;
+    const float* X2;
 };
 
 // Per-device scratch for split-K partial sums and arrival counters.

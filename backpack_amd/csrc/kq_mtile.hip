@@ -344,8 +344,12 @@ struct MtileWStage {
     }
 };
 
-template <int TYPE, int NW, int R>
-__global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
+// STAGED: weights through the LDS windows described above (dense calls).  Grouped calls walk one or two
+// chunks per workgroup and run thousands of workgroups: there the windows' LDS (one workgroup per CU instead
+// of two) costs more than the line re-fetches, so they load each lane's pieces straight from global memory.
+// (the grouped Q4_K kernel is held to 128 registers so that two of its workgroups share a CU)
+template <int TYPE, int NW, int R, bool STAGED>
+__global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1) void mtile_kernel(MtileParams p)
 {
     static_assert(R == NW || R == 1, "a wave owns a tile, or all waves share one");
     extern __shared__ __align__(16) uint8_t smem[];
@@ -363,8 +367,13 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
     if (p.tiles) {
         if (blockIdx.y >= *p.n_tiles) return;   // whole workgroup
         rec = p.tiles + (size_t)blockIdx.y * p.tile_stride;
-        count = rec[1];
+        // a record may hold more pairs than a pass of this kernel has token slots: blockIdx.z takes a slice
+        const uint32_t slots = TYPE == KQ_TYPE_Q6_K ? 8u : 16u;
+        const uint32_t first = blockIdx.z * slots;
+        if (first >= rec[1]) return;            // whole workgroup
+        count = min(rec[1] - first, slots);
         wmat += (size_t)rec[0] * p.N * p.row_stride_bytes;
+        rec += first;                           // rec[2 + token] is now the slice's pair
     }
     const bool has_tile = R == 1 || wave < p.tiles_per_wg;
     const uint32_t tile = R == 1 ? blockIdx.x : blockIdx.x * p.tiles_per_wg + wave;
@@ -389,12 +398,14 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
     // first superblock of staging pass h of the chunk at c0
     auto pass_block = [&](uint32_t c0, int h) { return c0 + (R == 1 ? wave : (uint32_t)h * HB); };
 
-    const uint32_t c_begin = blockIdx.z * p.chunks_per_split * MT_KC;
+    const uint32_t c_begin = (p.tiles ? 0u : blockIdx.z) * p.chunks_per_split * MT_KC;
     const uint32_t c_end = min(p.n_blocks, c_begin + p.chunks_per_split * MT_KC);
 
     MtileStager<64 * NW, Q6> stager;
     stager.init(p, rec, count);
     stager.fetch(p, c_begin);
+    t_f32x4 tot = {0, 0, 0, 0};
+    if constexpr (STAGED) {
 #pragma unroll
     for (int h = 0; h < PASSES; ++h) ws[h].load(pass_block(c_begin, h) * BB, row_bytes);
     // slots of tokens beyond M, and for Q6_K the halves that must read as zero, are cleared once
@@ -402,7 +413,6 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
         ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
     __syncthreads();
 
-    t_f32x4 tot = {0, 0, 0, 0};
     for (uint32_t c0 = c_begin; c0 < c_end; c0 += MT_KC) {
         stager.park(xa, xs, xinv);
         ws[0].store(wwin);
@@ -438,6 +448,48 @@ __global__ __launch_bounds__(64 * NW) void mtile_kernel(MtileParams p)
             }
         }
         __syncthreads();
+    }
+    } else {
+    for (uint32_t i = threadIdx.x; i < (MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4) / 16; i += 64 * NW)
+        ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
+    __syncthreads();
+    const uint8_t* wrow = wmat + (size_t)min(row, p.N - 1u) * p.row_stride_bytes;
+    constexpr int BPC = R == 1 ? (MT_KC + NW - 1) / NW : MT_KC;   // superblocks of a chunk this wave takes
+    for (uint32_t c0 = c_begin; c0 < c_end; c0 += MT_KC) {
+        // the chunk's weights are requested first, so that their latency runs under the conversion of X
+        t_u32x4 hdr[BPC];
+        t_u32x2 w[BPC][4];
+        Q6TileW w6[BPC];
+#pragma unroll
+        for (int i = 0; i < BPC; ++i) {
+            const uint32_t bb = R == 1 ? wave + i * NW : i;
+            const uint32_t b = min(c0 + bb, p.n_blocks - 1u);
+            const uint8_t* blk = wrow + (size_t)b * BB;
+            if constexpr (Q6) {
+                q6k_mtile_load(blk, kq, w6[i]);
+            } else {
+                hdr[i] = *(const t_u32x4*)blk;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) w[i][g] = *(const t_u32x2*)(blk + 16u + 32u * g + 8u * kq);
+            }
+        }
+        stager.park(xa, xs, xinv);
+        __syncthreads();
+        if (c0 + MT_KC < c_end) stager.fetch(p, c0 + MT_KC);   // the next chunk of X travels while this one is multiplied
+        if (has_tile) {
+#pragma unroll
+            for (int i = 0; i < BPC; ++i) {
+                const uint32_t bb = R == 1 ? wave + i * NW : i;
+                if (bb < MT_KC && c0 + bb < c_end) {
+                    if constexpr (Q6)
+                        q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                    else
+                        q4k_mtile_block(hdr[i], w[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                }
+            }
+        }
+        __syncthreads();
+    }
     }
 
     if (R == 1) {
@@ -515,13 +567,13 @@ bool mtile_supported(const MatmulArgs& a)
     return false;
 }
 
-template <int TYPE, int NW, int R>
+template <int TYPE, int NW, int R, bool STAGED = true>
 static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s, uint32_t wgs_z = 1)
 {
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
     constexpr int PITCH = Q6 ? (R == 1 ? 240 : 464) : (R == 1 ? 160 : 304);   // as in the kernel
-    constexpr size_t shmem = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * sizeof(float) + (size_t)NW * 16 * PITCH;
-    auto kern = mtile_kernel<TYPE, NW, R>;
+    constexpr size_t shmem = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * sizeof(float) + (STAGED ? (size_t)NW * 16 * PITCH : 0);
+    auto kern = mtile_kernel<TYPE, NW, R, STAGED>;
     static bool raised = false;   // per instantiation
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -537,7 +589,9 @@ uint32_t mtile_group_cap(int type) { return type == KQ_TYPE_Q6_K ? 8u : 16u; }
 hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, const uint32_t* n_tiles,
                                 uint32_t tiles_bound, uint32_t cap, hipStream_t s)
 {
-    if (cap > mtile_group_cap(a.type) || tiles_bound == 0 || tiles_bound > 65535u) return hipErrorInvalidValue;
+    // records of up to cap pairs; a record beyond the kernel's token slots (Q6_K: 8) is served in slices
+    const uint32_t slices = (cap + mtile_group_cap(a.type) - 1u) / mtile_group_cap(a.type);
+    if (cap == 0 || cap > 16u || tiles_bound == 0 || tiles_bound > 65535u) return hipErrorInvalidValue;
     MtileParams p;
     p.X = (const float*)a.X;
     p.W = a.W;
@@ -558,8 +612,8 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
     p.tiles_per_wg = 8;
     const uint32_t row_tiles = (a.N + 15u) / 16u;
     const uint32_t wgs = (row_tiles + 7u) / 8u;
-    return a.type == KQ_TYPE_Q6_K ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8>(p, wgs, tiles_bound, s)
-                                  : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8>(p, wgs, tiles_bound, s);
+    return a.type == KQ_TYPE_Q6_K ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, false>(p, wgs, tiles_bound, s, slices)
+                                  : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, false>(p, wgs, tiles_bound, s, slices);
 }
 
 hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s)

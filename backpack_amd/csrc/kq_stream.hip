@@ -37,16 +37,39 @@ struct StreamParams {
     const uint32_t* expert_idx;
     uint32_t k_slots, ldy;
     int x_per_slot;
+    // MoE FFN fusions (grouped launches): a twin matrix of the same shape served by blockIdx.z == 1
+    // (gate and up read the same x), and an activation input: x = silu(X) * X2 (down reads gate and up)
+    const uint8_t* W2;
+    float* Y2;
+    const float* X2;
 };
 
 // Redirects the pointers of a grouped launch to the pair this workgroup serves.
 __device__ __forceinline__ void stream_select_pair(StreamParams& p)
 {
     if (!p.expert_idx) return;
+    if (blockIdx.z) { p.W = p.W2; p.Y = p.Y2; }
     const uint32_t pair = blockIdx.y;
     p.W += (size_t)p.expert_idx[pair] * p.N * p.row_stride_bytes;
-    p.X += (size_t)(p.x_per_slot ? pair : pair / p.k_slots) * p.K;
+    const size_t xrow = (size_t)(p.x_per_slot ? pair : pair / p.k_slots) * p.K;
+    p.X += xrow;
+    if (p.X2) p.X2 += xrow;
     p.Y += (size_t)pair * p.ldy;
+}
+
+// Four activations: X as it is, or silu(X) * X2 with silu(g) = g / (exp(-g) + 1) (the formula of
+// moe_silu_mul_kernel, so that the fused and the separate form agree to the bit).
+__device__ __forceinline__ float4 stream_x4(const StreamParams& p, const float4* xp)
+{
+    float4 v = *xp;
+    if (p.X2) {
+        const float4 u = *(const float4*)((const float*)xp - p.X + p.X2);
+        v.x = v.x / (expf(-v.x) + 1.0f) * u.x;
+        v.y = v.y / (expf(-v.y) + 1.0f) * u.y;
+        v.z = v.z / (expf(-v.z) + 1.0f) * u.z;
+        v.w = v.w / (expf(-v.w) + 1.0f) * u.w;
+    }
+    return v;
 }
 
 __device__ __forceinline__ float s_fma_h(_Float16 h, float x, float acc) { return __builtin_fmaf((float)h, x, acc); }
@@ -208,7 +231,7 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
             const float4* xp = (const float4*)(p.X + (size_t)t * p.K + (size_t)b * KQ_QK + 64u * g + 16u * h);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float4 lo = xp[i], hi = xp[8 + i];
+                float4 lo = stream_x4(p, xp + i), hi = stream_x4(p, xp + 8 + i);
                 if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
                 xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
                 xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
@@ -401,7 +424,7 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
             const float4* xp = (const float4*)(p.X + (size_t)tk * p.K + (size_t)b * KQ_QK + 128u * n + 8u * lg);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                float4 lo = xp[8 * k], hi = xp[8 * k + 1];
+                float4 lo = stream_x4(p, xp + 8 * k), hi = stream_x4(p, xp + 8 * k + 1);
                 if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
                 x[pass][tk][k][0] = lo.x; x[pass][tk][k][1] = lo.y; x[pass][tk][k][2] = lo.z; x[pass][tk][k][3] = lo.w;
                 x[pass][tk][k][4] = hi.x; x[pass][tk][k][5] = hi.y; x[pass][tk][k][6] = hi.z; x[pass][tk][k][7] = hi.w;
@@ -518,6 +541,10 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     p.k_slots = a.k_slots;
     p.ldy = a.ldy;
     p.x_per_slot = a.x_per_slot;
+    p.W2 = a.expert_idx ? a.W2 : nullptr;
+    p.Y2 = a.Y2;
+    p.X2 = a.expert_idx ? a.X2 : nullptr;
+    const uint32_t twins = p.W2 ? 2u : 1u;            // grid.z
     const uint32_t pairs = a.expert_idx ? a.M : 1u;   // grid.y
     const bool two = !a.expert_idx && a.M == 2;       // two tokens share every weight load
     // Measured on MI355X: these kernels run best with about 40 KB of weight loads
@@ -529,13 +556,13 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
         const int kw = nb <= 16u ? 1 : nb <= 32u ? 4 : 7;
         const int pp = nb <= 8u ? 1 : nb <= 16u ? 2 : nb <= 56u ? 1 : 2;
         uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 8u / (uint32_t)kw, t.splits);
-        wgs = (wgs + pairs - 1u) / pairs;   // the pairs of a grouped launch share the machine
+        wgs = (wgs + pairs * twins - 1u) / (pairs * twins);   // the pairs of a grouped launch share the machine
         const int depth = t.depth > 0 ? t.depth : 2;
 #define KQ_STREAM6_MT(P, KW, MT) \
     do { \
-        if (depth <= 1) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 1, MT>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
-        else if (depth <= 2) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 2, MT>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
-        else hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 4, MT>), dim3(wgs, pairs), dim3(64 * KW), 0, s, p); \
+        if (depth <= 1) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 1, MT>), dim3(wgs, pairs, twins), dim3(64 * KW), 0, s, p); \
+        else if (depth <= 2) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 2, MT>), dim3(wgs, pairs, twins), dim3(64 * KW), 0, s, p); \
+        else hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 4, MT>), dim3(wgs, pairs, twins), dim3(64 * KW), 0, s, p); \
     } while (0)
 #define KQ_STREAM6(P, KW) \
     do { \
@@ -555,12 +582,12 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     // a Q4_K workgroup is NW independent waves, each with its own rows
     uint32_t wgs = t.splits > 0 ? ((a.N + (uint32_t)t.splits - 1u) / (uint32_t)t.splits + NW - 1u) / NW
                                 : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
-    wgs = (wgs + pairs - 1u) / pairs;
+    wgs = (wgs + pairs * twins - 1u) / (pairs * twins);
     const int depth = t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
 #define KQ_STREAM_LAUNCH(P, D) \
     do { \
-        if (two) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, 2>), dim3(wgs, pairs), dim3(64 * NW), 0, s, p); \
-        else hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, 1>), dim3(wgs, pairs), dim3(64 * NW), 0, s, p); \
+        if (two) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, 2>), dim3(wgs, pairs, twins), dim3(64 * NW), 0, s, p); \
+        else hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, 1>), dim3(wgs, pairs, twins), dim3(64 * NW), 0, s, p); \
     } while (0)
     if (a.n_blocks <= 8u) {
         if (depth <= 1) KQ_STREAM_LAUNCH(1, 1);
