@@ -608,12 +608,16 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
     p.n_splits = 1; p.chunks_per_split = (a.n_blocks + MT_KC - 1) / MT_KC; p.partial = nullptr; p.counters = nullptr;
     p.k_slots = a.k_slots;
     p.x_per_slot = a.x_per_slot;
-    // a wave per 16-row tile of the expert, 8 tiles per workgroup: X of the record is converted once per 128 rows
-    p.tiles_per_wg = 8;
+    // a wave per 16-row tile of the expert, X of the record converted once per workgroup.  These workgroups walk
+    // one or two chunks and are bound by their latencies, so two must share a CU: Q4_K runs 8 tiles per
+    // workgroup at 128 registers, Q6_K (160 registers) 4 tiles per workgroup of 4 waves.
     const uint32_t row_tiles = (a.N + 15u) / 16u;
-    const uint32_t wgs = (row_tiles + 7u) / 8u;
-    return a.type == KQ_TYPE_Q6_K ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, false>(p, wgs, tiles_bound, s, slices)
-                                  : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, false>(p, wgs, tiles_bound, s, slices);
+    if (a.type == KQ_TYPE_Q6_K) {
+        p.tiles_per_wg = 4;
+        return launch_mtile_one<KQ_TYPE_Q6_K, 4, 4, false>(p, (row_tiles + 3u) / 4u, tiles_bound, s, slices);
+    }
+    p.tiles_per_wg = 8;
+    return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, false>(p, (row_tiles + 7u) / 8u, tiles_bound, s, slices);
 }
 
 hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s)
