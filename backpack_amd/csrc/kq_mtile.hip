@@ -86,11 +86,13 @@ struct MtileParams {
 // consecutive elements of one (token, superblock) pair; pairs are numbered
 // token-major, so a wave covers few tokens and waves whose tokens are all
 // beyond M have nothing to do after their slots were zeroed once.
-template <int NT, bool SPLIT16>
+// TOK = 16 or 8 (4 works too): the tokens the workgroup's threads are spread over; a launch with few tokens takes a
+// small TOK so that every wave converts a share instead of the first waves converting everything.
+template <int NT, bool SPLIT16, int TOK>
 struct MtileStager {
-    static constexpr int TPP = NT / (MT_KC * 16);   // threads per (token, block) pair
-    static constexpr int EPT = 256 / TPP;           // elements per thread: 64 or 32
-    static_assert(EPT == 64 || EPT == 32, "a thread converts one or two sub-blocks");
+    static constexpr int TPP = NT / (MT_KC * TOK);  // threads per (token, block) pair
+    static constexpr int EPT = 256 / TPP;           // elements per thread
+    static_assert(TPP <= 64 && (EPT == 64 || EPT == 32 || EPT == 16 || EPT == 8), "a pair is converted inside one wave");
     float4 v[EPT / 4];
     uint32_t token, bb, sub;
     bool live_token;
@@ -164,24 +166,114 @@ struct MtileStager {
             *(t_half8*)(dst + 1024) = lv;
         }
         // sums of the unscaled x over each run of 32 (or, SPLIT16, each half run of 16)
+        if constexpr (EPT >= 32) {
 #pragma unroll
-        for (int q = 0; q < EPT / 32; ++q) {
-            float h0 = 0.0f, h1 = 0.0f;
+            for (int q = 0; q < EPT / 32; ++q) {
+                float h0 = 0.0f, h1 = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                h0 += (v[8 * q + i].x + v[8 * q + i].y) + (v[8 * q + i].z + v[8 * q + i].w);
-                h1 += (v[8 * q + 4 + i].x + v[8 * q + 4 + i].y) + (v[8 * q + 4 + i].z + v[8 * q + 4 + i].w);
+                for (int i = 0; i < 4; ++i) {
+                    h0 += (v[8 * q + i].x + v[8 * q + i].y) + (v[8 * q + i].z + v[8 * q + i].w);
+                    h1 += (v[8 * q + 4 + i].x + v[8 * q + 4 + i].y) + (v[8 * q + 4 + i].z + v[8 * q + 4 + i].w);
+                }
+                float* dst = xs + (bb * 8u + (sub * EPT) / 32u + q) * 16u + token;
+                if (SPLIT16) { dst[0] = h0; dst[8] = h1; }
+                else dst[0] = h0 + h1;
             }
-            float* dst = xs + (bb * 8u + (sub * EPT) / 32u + q) * 16u + token;
-            if (SPLIT16) { dst[0] = h0; dst[8] = h1; }
-            else dst[0] = h0 + h1;
+        } else {
+            // the run is spread over 32 / EPT neighbouring threads: partial sums meet by lane exchange
+            float h = 0.0f;
+#pragma unroll
+            for (int i = 0; i < EPT / 4; ++i) h += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+            constexpr int PER16 = 16 / EPT;   // threads per half run: 1 (EPT 16) or 2 (EPT 8)
+            if (PER16 == 2) h += __shfl_xor(h, 1, 64);
+            const uint32_t half = (sub / PER16) & 1u, run = sub / (2u * PER16);
+            float* dst = xs + (bb * 8u + run) * 16u + token;
+            if (SPLIT16) {
+                if (sub % PER16 == 0u) dst[8u * half] = h;
+            } else {
+                h += __shfl_xor(h, PER16, 64);
+                if (sub % (2u * PER16) == 0u) dst[0] = h;
+            }
         }
     }
 };
 
 // One superblock of one 16-row tile: adds this block's contribution to tot[4]
-// (tokens 4*(lane/16) .. +3 of weight row lane%16).
+// (tokens 4*(lane/16) .. +3 of weight row lane%16).  The LDS operands of sub-block s+1 are requested
+// before the matrix instructions of sub-block s, and the scale arithmetic on a result runs one sub-block
+// behind the instructions that produce it, so neither latency is waited for.
+struct MtileA {
+    t_half8 hi, lo;
+    float4 xsum;
+};
+__device__ __forceinline__ MtileA mtile_read_a(const uint8_t* xa_b, const float* xs_b, int sb, uint32_t lane)
+{
+    const uint8_t* ap = xa_b + ((size_t)(sb * 2) * 64u + lane) * 16u;
+    MtileA a;
+    a.hi = *(const t_half8*)ap;
+    a.lo = *(const t_half8*)(ap + 1024);
+    a.xsum = *(const float4*)(xs_b + sb * 16 + 4u * (lane >> 4));
+    return a;
+}
+
 __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2 (&w)[4], const uint8_t* xa_b,
+                                                const float* xs_b, const float* xinv_b, uint32_t lane,
+                                                t_f32x4& tot)
+{
+    const float d = half_bits_to_float(hdr.x & 0xFFFFu);
+    const float dmin = half_bits_to_float(hdr.x >> 16);
+    const uint32_t scA = hdr.y & 0x3F3F3F3Fu;
+    const uint32_t mnA = hdr.z & 0x3F3F3F3Fu;
+    const uint32_t scB = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    const uint32_t mnB = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    const uint32_t tq = lane >> 4;
+    t_f32x4 U = {0, 0, 0, 0}, V = {0, 0, 0, 0};
+    MtileA a_cur = mtile_read_a(xa_b, xs_b, 0, lane);
+    t_f32x4 D_prev = {0, 0, 0, 0};
+    float4 xsum_prev = {0, 0, 0, 0};
+    t_u32x4 blo = {0, 0, 0, 0}, bhi = {0, 0, 0, 0};
+    auto scale_in = [&](int sb, const t_f32x4& D, const float4& xsum) {
+        const uint32_t scw = sb < 4 ? scA : scB, mnw = sb < 4 ? mnA : mnB;
+        // high nibbles sit four bits up: 1/16 goes into their scale
+        const float sc = (float)((scw >> (8 * (sb & 3))) & 255u) * ((sb & 1) ? 0.0625f : 1.0f);
+        const float mn = (float)((mnw >> (8 * (sb & 3))) & 255u);
+        U.x = fmaf(sc, D.x, U.x); U.y = fmaf(sc, D.y, U.y); U.z = fmaf(sc, D.z, U.z); U.w = fmaf(sc, D.w, U.w);
+        V.x = fmaf(mn, xsum.x, V.x); V.y = fmaf(mn, xsum.y, V.y); V.z = fmaf(mn, xsum.z, V.z); V.w = fmaf(mn, xsum.w, V.w);
+    };
+#pragma unroll
+    for (int sb = 0; sb < 8; ++sb) {
+        MtileA a_next = a_cur;
+        if (sb < 7) a_next = mtile_read_a(xa_b, xs_b, sb + 1, lane);
+        if ((sb & 1) == 0) {
+            const uint32_t d0 = w[sb >> 1].x, d1 = w[sb >> 1].y;
+            const uint32_t e0 = d0 >> 8, e1 = d1 >> 8;
+            blo = t_u32x4{d0 & 0x000F000Fu, e0 & 0x000F000Fu, d1 & 0x000F000Fu, e1 & 0x000F000Fu};
+            bhi = t_u32x4{d0 & 0x00F000F0u, e0 & 0x00F000F0u, d1 & 0x00F000F0u, e1 & 0x00F000F0u};
+        }
+        const t_half8 bq = __builtin_bit_cast(t_half8, (sb & 1) ? bhi : blo);
+        t_f32x4 D = {0, 0, 0, 0};
+        D = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur.hi, bq, D, 0, 0, 0);
+        D = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur.lo, bq, D, 0, 0, 0);
+        if (sb > 0) scale_in(sb - 1, D_prev, xsum_prev);
+        __builtin_amdgcn_sched_barrier(0);   // keeps the three stages of this step together
+        D_prev = D;
+        xsum_prev = a_cur.xsum;
+        a_cur = a_next;
+    }
+    scale_in(7, D_prev, xsum_prev);
+    (void)tq;
+    // D carries 2^-24 from the subnormal nibbles and the token's scale
+    const float4 inv = *(const float4*)(xinv_b + 4u * (lane >> 4));
+    const float d24 = d * 16777216.0f;
+    tot.x += fmaf(d24 * inv.x, U.x, -(dmin * V.x));
+    tot.y += fmaf(d24 * inv.y, U.y, -(dmin * V.y));
+    tot.z += fmaf(d24 * inv.z, U.z, -(dmin * V.z));
+    tot.w += fmaf(d24 * inv.w, U.w, -(dmin * V.w));
+}
+
+// The same arithmetic with every operand read where it is used: fewer registers (the grouped kernel is held
+// to 128 so that two of its workgroups share a CU).
+__device__ __forceinline__ void q4k_mtile_block_compact(const t_u32x4 hdr, const t_u32x2 (&w)[4], const uint8_t* xa_b,
                                                 const float* xs_b, const float* xinv_b, uint32_t lane,
                                                 t_f32x4& tot)
 {
@@ -348,7 +440,7 @@ struct MtileWStage {
 // chunks per workgroup and run thousands of workgroups: there the windows' LDS (one workgroup per CU instead
 // of two) costs more than the line re-fetches, so they load each lane's pieces straight from global memory.
 // (the grouped Q4_K kernel is held to 128 registers so that two of its workgroups share a CU)
-template <int TYPE, int NW, int R, bool STAGED>
+template <int TYPE, int NW, int R, bool STAGED, int TOK>
 __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1) void mtile_kernel(MtileParams p)
 {
     static_assert(R == NW || R == 1, "a wave owns a tile, or all waves share one");
@@ -401,7 +493,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     const uint32_t c_begin = (p.tiles ? 0u : blockIdx.z) * p.chunks_per_split * MT_KC;
     const uint32_t c_end = min(p.n_blocks, c_begin + p.chunks_per_split * MT_KC);
 
-    MtileStager<64 * NW, Q6> stager;
+    MtileStager<64 * NW, Q6, TOK> stager;
     stager.init(p, rec, count);
     stager.fetch(p, c_begin);
     t_f32x4 tot = {0, 0, 0, 0};
@@ -484,7 +576,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                     if constexpr (Q6)
                         q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
                     else
-                        q4k_mtile_block(hdr[i], w[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                        q4k_mtile_block_compact(hdr[i], w[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
                 }
             }
         }
@@ -567,13 +659,13 @@ bool mtile_supported(const MatmulArgs& a)
     return false;
 }
 
-template <int TYPE, int NW, int R, bool STAGED = true>
+template <int TYPE, int NW, int R, bool STAGED = true, int TOK = 16>
 static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s, uint32_t wgs_z = 1)
 {
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
     constexpr int PITCH = Q6 ? (R == 1 ? 240 : 464) : (R == 1 ? 160 : 304);   // as in the kernel
     constexpr size_t shmem = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * sizeof(float) + (STAGED ? (size_t)NW * 16 * PITCH : 0);
-    auto kern = mtile_kernel<TYPE, NW, R, STAGED>;
+    auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK>;
     static bool raised = false;   // per instantiation
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -675,8 +767,14 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
             p.n_splits = best_splits;
             p.chunks_per_split = best_cps;
             const uint32_t wgs = (tiles + best_tpw - 1u) / best_tpw;
-            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8>(p, wgs, 1, s, best_splits)
-                   : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8>(p, wgs, 1, s, best_splits);
+            // 5..8 tokens: the conversion of X is spread over twice the threads per (token, superblock), so
+            // that all waves take part (measured +2-3 %; with 4 tokens or fewer the wider exchange costs more)
+            if (p.M > 4u && p.M <= 8u)
+                e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits)
+                       : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits);
+            else
+                e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits)
+                       : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits);
         }
         if (e != hipSuccess) return e;
     }

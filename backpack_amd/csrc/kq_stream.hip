@@ -20,6 +20,7 @@
 // its 16 activations, a per-lane constant.
 #include "kq_format.h"
 #include "kq_kernels.h"
+#include <type_traits>
 
 namespace kq {
 
@@ -59,10 +60,11 @@ __device__ __forceinline__ void stream_select_pair(StreamParams& p)
 
 // Four activations: X as it is, or silu(X) * X2 with silu(g) = g / (exp(-g) + 1) (the formula of
 // moe_silu_mul_kernel, so that the fused and the separate form agree to the bit).
+template <bool ACT>
 __device__ __forceinline__ float4 stream_x4(const StreamParams& p, const float4* xp)
 {
     float4 v = *xp;
-    if (p.X2) {
+    if constexpr (ACT) {
         const float4 u = *(const float4*)((const float*)xp - p.X + p.X2);
         v.x = v.x / (expf(-v.x) + 1.0f) * u.x;
         v.y = v.y / (expf(-v.y) + 1.0f) * u.y;
@@ -220,6 +222,9 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
 
     float xlo[P][MT][16], xhi[P][MT][16], xs_lo[P][MT], xs_hi[P][MT];
     uint32_t hoff[P];
+    // (one branch around the whole prologue, so that either form issues its loads back to back)
+    auto load_x = [&](auto act) {
+        constexpr bool ACT = decltype(act)::value;
 #pragma unroll
     for (int pass = 0; pass < P; ++pass) {
         uint32_t b = pass * 8u + bl;
@@ -231,7 +236,7 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
             const float4* xp = (const float4*)(p.X + (size_t)t * p.K + (size_t)b * KQ_QK + 64u * g + 16u * h);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float4 lo = stream_x4(p, xp + i), hi = stream_x4(p, xp + 8 + i);
+                float4 lo = stream_x4<ACT>(p, xp + i), hi = stream_x4<ACT>(p, xp + 8 + i);
                 if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
                 xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
                 xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
@@ -243,6 +248,10 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
             xs_hi[pass][t] = sh_;
         }
     }
+
+    };
+    if (p.X2) load_x(std::true_type{});
+    else load_x(std::false_type{});
 
     // Ring of D rows in flight.  Slot d is refilled as soon as its row has been
     // consumed; the wait before a slot's arithmetic leaves the (D-1) younger
@@ -413,6 +422,8 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
 
     float x[P][MT][4][8], m32xs[P][MT][4];
     uint32_t boff[P];
+    auto load_x = [&](auto act) {
+        constexpr bool ACT = decltype(act)::value;
 #pragma unroll
     for (int pass = 0; pass < P; ++pass) {
         uint32_t b = (wave * P + pass) * 8u + bl;
@@ -424,7 +435,7 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
             const float4* xp = (const float4*)(p.X + (size_t)tk * p.K + (size_t)b * KQ_QK + 128u * n + 8u * lg);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                float4 lo = stream_x4(p, xp + 8 * k), hi = stream_x4(p, xp + 8 * k + 1);
+                float4 lo = stream_x4<ACT>(p, xp + 8 * k), hi = stream_x4<ACT>(p, xp + 8 * k + 1);
                 if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
                 x[pass][tk][k][0] = lo.x; x[pass][tk][k][1] = lo.y; x[pass][tk][k][2] = lo.z; x[pass][tk][k][3] = lo.w;
                 x[pass][tk][k][4] = hi.x; x[pass][tk][k][5] = hi.y; x[pass][tk][k][6] = hi.z; x[pass][tk][k][7] = hi.w;
@@ -435,6 +446,10 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
             }
         }
     }
+
+    };
+    if (p.X2) load_x(std::true_type{});
+    else load_x(std::false_type{});
 
     if (n_rows == 0) return;   // whole workgroup
     constexpr int SLOT_LOADS = 5 * P;
