@@ -59,6 +59,8 @@ constexpr int MT_KC = 4;                       // superblocks of X staged at a t
 constexpr int MT_XA_BYTES = MT_KC * 8 * 2 * 1024;   // [block][sub-block][hi/lo][lane] 16 B
 constexpr int MT_XS_FLOATS = MT_KC * 8 * 16;        // [block][sub-block][token]
 constexpr int MT_INV_FLOATS = MT_KC * 16;           // [block][token]
+constexpr int MT_XV_BYTES = MT_KC * 2 * 1024;       // [block][hi/lo][lane] 16 B: the sub-block sums as an A operand (Q4_K)
+constexpr int MT_STAGE_BYTES = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4 + MT_XV_BYTES;
 
 struct MtileParams {
     const float* X;
@@ -88,7 +90,8 @@ struct MtileParams {
 // beyond M have nothing to do after their slots were zeroed once.
 // TOK = 16 or 8 (4 works too): the tokens the workgroup's threads are spread over; a launch with few tokens takes a
 // small TOK so that every wave converts a share instead of the first waves converting everything.
-template <int NT, bool SPLIT16, int TOK>
+// XV: also stage the sub-block sums as an A operand (the Q4_K kernels that put the minima on the matrix cores).
+template <int NT, bool SPLIT16, int TOK, bool XV>
 struct MtileStager {
     static constexpr int TPP = NT / (MT_KC * TOK);  // threads per (token, block) pair
     static constexpr int EPT = 256 / TPP;           // elements per thread
@@ -122,7 +125,7 @@ struct MtileStager {
         for (int i = 0; i < EPT / 4; ++i) v[i] = src[i];
     }
     // converts what fetch() brought and parks it in LDS (slots of tokens beyond M stay zero)
-    __device__ __forceinline__ void park(uint8_t* xa, float* xs, float* xinv)
+    __device__ __forceinline__ void park(uint8_t* xa, float* xs, float* xinv, uint8_t* xv)
     {
         if (!live_token) return;   // wave-uniform for whole waves of dead tokens
         // largest magnitude of the pair's 256 elements, as float bits (orders like the floats)
@@ -144,6 +147,17 @@ struct MtileStager {
             xinv[bb * 16u + token] = inv;
             if (SPLIT16) xinv[bb * 16u + token + 8u] = inv;
         }
+        // Q4_K: the sum over sub-block sb also goes out as element sb of an A operand (lane = token, the
+        // lanes of k >= 8 stay zero), scaled by s / 32 so that 32 elements of at most 2^15 fit an fp16
+        auto put_sum = [&](uint32_t sb, float sum) {
+            if (!XV) return;
+            const float a = sum * (s * 0.03125f);
+            const _Float16 h = (_Float16)a;
+            const _Float16 l = (_Float16)(a - (float)h);
+            _Float16* dst = (_Float16*)(xv + ((size_t)(bb * 2u) * 64u + token) * 16u) + sb;
+            dst[0] = h;
+            dst[512] = l;   // the lo operand: 1024 bytes on
+        };
         // groups of 8 consecutive k -> one operand slot: halves in the order k+0, k+2, k+1, k+3, k+4, k+6, k+5, k+7
 #pragma unroll
         for (int g8 = 0; g8 < EPT / 8; ++g8) {
@@ -177,7 +191,7 @@ struct MtileStager {
                 }
                 float* dst = xs + (bb * 8u + (sub * EPT) / 32u + q) * 16u + token;
                 if (SPLIT16) { dst[0] = h0; dst[8] = h1; }
-                else dst[0] = h0 + h1;
+                else { dst[0] = h0 + h1; put_sum((sub * EPT) / 32u + q, h0 + h1); }
             }
         } else {
             // the run is spread over 32 / EPT neighbouring threads: partial sums meet by lane exchange
@@ -192,7 +206,7 @@ struct MtileStager {
                 if (sub % PER16 == 0u) dst[8u * half] = h;
             } else {
                 h += __shfl_xor(h, PER16, 64);
-                if (sub % (2u * PER16) == 0u) dst[0] = h;
+                if (sub % (2u * PER16) == 0u) { dst[0] = h; put_sum(run, h); }
             }
         }
     }
@@ -204,20 +218,21 @@ struct MtileStager {
 // behind the instructions that produce it, so neither latency is waited for.
 struct MtileA {
     t_half8 hi, lo;
-    float4 xsum;
 };
-__device__ __forceinline__ MtileA mtile_read_a(const uint8_t* xa_b, const float* xs_b, int sb, uint32_t lane)
+__device__ __forceinline__ MtileA mtile_read_a(const uint8_t* xa_b, int sb, uint32_t lane)
 {
     const uint8_t* ap = xa_b + ((size_t)(sb * 2) * 64u + lane) * 16u;
     MtileA a;
     a.hi = *(const t_half8*)ap;
     a.lo = *(const t_half8*)(ap + 1024);
-    a.xsum = *(const float4*)(xs_b + sb * 16 + 4u * (lane >> 4));
     return a;
 }
 
+// The minima ride on the matrix cores as well: sum over sub-blocks of mn[row][sb] * xsum[token][sb] is one more
+// product with k = sub-block (8 of the 32 k used): A = the staged sums (xv_b), B = the eight 6-bit minima of
+// the lane's row as subnormals.  B's lanes of k >= 8 hold the same finite values; A is zero there.
 __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2 (&w)[4], const uint8_t* xa_b,
-                                                const float* xs_b, const float* xinv_b, uint32_t lane,
+                                                const uint8_t* xv_b, const float* xinv_b, uint32_t lane,
                                                 t_f32x4& tot)
 {
     const float d = half_bits_to_float(hdr.x & 0xFFFFu);
@@ -226,24 +241,22 @@ __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2
     const uint32_t mnA = hdr.z & 0x3F3F3F3Fu;
     const uint32_t scB = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
     const uint32_t mnB = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
-    const uint32_t tq = lane >> 4;
-    t_f32x4 U = {0, 0, 0, 0}, V = {0, 0, 0, 0};
-    MtileA a_cur = mtile_read_a(xa_b, xs_b, 0, lane);
+    t_f32x4 U = {0, 0, 0, 0};
+    MtileA a_cur = mtile_read_a(xa_b, 0, lane);
+    const t_half8 vhi = *(const t_half8*)(xv_b + (size_t)lane * 16u);
+    const t_half8 vlo = *(const t_half8*)(xv_b + 1024 + (size_t)lane * 16u);
     t_f32x4 D_prev = {0, 0, 0, 0};
-    float4 xsum_prev = {0, 0, 0, 0};
     t_u32x4 blo = {0, 0, 0, 0}, bhi = {0, 0, 0, 0};
-    auto scale_in = [&](int sb, const t_f32x4& D, const float4& xsum) {
-        const uint32_t scw = sb < 4 ? scA : scB, mnw = sb < 4 ? mnA : mnB;
+    auto scale_in = [&](int sb, const t_f32x4& D) {
+        const uint32_t scw = sb < 4 ? scA : scB;
         // high nibbles sit four bits up: 1/16 goes into their scale
         const float sc = (float)((scw >> (8 * (sb & 3))) & 255u) * ((sb & 1) ? 0.0625f : 1.0f);
-        const float mn = (float)((mnw >> (8 * (sb & 3))) & 255u);
         U.x = fmaf(sc, D.x, U.x); U.y = fmaf(sc, D.y, U.y); U.z = fmaf(sc, D.z, U.z); U.w = fmaf(sc, D.w, U.w);
-        V.x = fmaf(mn, xsum.x, V.x); V.y = fmaf(mn, xsum.y, V.y); V.z = fmaf(mn, xsum.z, V.z); V.w = fmaf(mn, xsum.w, V.w);
     };
 #pragma unroll
     for (int sb = 0; sb < 8; ++sb) {
         MtileA a_next = a_cur;
-        if (sb < 7) a_next = mtile_read_a(xa_b, xs_b, sb + 1, lane);
+        if (sb < 7) a_next = mtile_read_a(xa_b, sb + 1, lane);
         if ((sb & 1) == 0) {
             const uint32_t d0 = w[sb >> 1].x, d1 = w[sb >> 1].y;
             const uint32_t e0 = d0 >> 8, e1 = d1 >> 8;
@@ -254,21 +267,26 @@ __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2
         t_f32x4 D = {0, 0, 0, 0};
         D = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur.hi, bq, D, 0, 0, 0);
         D = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur.lo, bq, D, 0, 0, 0);
-        if (sb > 0) scale_in(sb - 1, D_prev, xsum_prev);
+        if (sb > 0) scale_in(sb - 1, D_prev);
         __builtin_amdgcn_sched_barrier(0);   // keeps the three stages of this step together
         D_prev = D;
-        xsum_prev = a_cur.xsum;
         a_cur = a_next;
     }
-    scale_in(7, D_prev, xsum_prev);
-    (void)tq;
-    // D carries 2^-24 from the subnormal nibbles and the token's scale
+    // bytes of mnA / mnB -> fp16 subnormals mn * 2^-24, element sb in position sb
+    const t_u32x4 bm = {__builtin_amdgcn_perm(0u, mnA, 0x0c010c00u), __builtin_amdgcn_perm(0u, mnA, 0x0c030c02u),
+                        __builtin_amdgcn_perm(0u, mnB, 0x0c010c00u), __builtin_amdgcn_perm(0u, mnB, 0x0c030c02u)};
+    const t_half8 bmn = __builtin_bit_cast(t_half8, bm);
+    t_f32x4 V = {0, 0, 0, 0};
+    V = __builtin_amdgcn_mfma_f32_16x16x32_f16(vhi, bmn, V, 0, 0, 0);
+    V = __builtin_amdgcn_mfma_f32_16x16x32_f16(vlo, bmn, V, 0, 0, 0);
+    scale_in(7, D_prev);
+    // U carries 2^-24 from the subnormal nibbles and the token's scale s; V carries 2^-24 and s / 32
     const float4 inv = *(const float4*)(xinv_b + 4u * (lane >> 4));
-    const float d24 = d * 16777216.0f;
-    tot.x += fmaf(d24 * inv.x, U.x, -(dmin * V.x));
-    tot.y += fmaf(d24 * inv.y, U.y, -(dmin * V.y));
-    tot.z += fmaf(d24 * inv.z, U.z, -(dmin * V.z));
-    tot.w += fmaf(d24 * inv.w, U.w, -(dmin * V.w));
+    const float d24 = d * 16777216.0f, m24 = dmin * (16777216.0f * 32.0f);
+    tot.x += inv.x * fmaf(d24, U.x, -(m24 * V.x));
+    tot.y += inv.y * fmaf(d24, U.y, -(m24 * V.y));
+    tot.z += inv.z * fmaf(d24, U.z, -(m24 * V.z));
+    tot.w += inv.w * fmaf(d24, U.w, -(m24 * V.w));
 }
 
 // The same arithmetic with every operand read where it is used: fewer registers (the grouped kernel is held
@@ -448,6 +466,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     uint8_t* xa = smem;
     float* xs = (float*)(smem + MT_XA_BYTES);
     float* xinv = xs + MT_XS_FLOATS;
+    uint8_t* xv = (uint8_t*)(xinv + MT_INV_FLOATS);
     float* red = (float*)smem;   // reused after the last chunk
 
     const uint32_t lane = threadIdx.x & 63u;
@@ -482,7 +501,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     constexpr int PASSES = R == 1 ? 1 : MT_KC / HB;
     using WStage = MtileWStage<SPAN, PITCH>;
     static_assert(PITCH >= WStage::UPR * 16 && PITCH % 16 == 0, "window row holds the staged units");
-    uint8_t* wwin = smem + MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4 + wave * (16 * PITCH);
+    uint8_t* wwin = smem + MT_STAGE_BYTES + wave * (16 * PITCH);
     const uint32_t row_bytes = p.n_blocks * BB;
     WStage ws[PASSES];
 #pragma unroll
@@ -493,7 +512,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     const uint32_t c_begin = (p.tiles ? 0u : blockIdx.z) * p.chunks_per_split * MT_KC;
     const uint32_t c_end = min(p.n_blocks, c_begin + p.chunks_per_split * MT_KC);
 
-    MtileStager<64 * NW, Q6, TOK> stager;
+    MtileStager<64 * NW, Q6, TOK, STAGED && !Q6> stager;
     stager.init(p, rec, count);
     stager.fetch(p, c_begin);
     t_f32x4 tot = {0, 0, 0, 0};
@@ -501,12 +520,12 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
 #pragma unroll
     for (int h = 0; h < PASSES; ++h) ws[h].load(pass_block(c_begin, h) * BB, row_bytes);
     // slots of tokens beyond M, and for Q6_K the halves that must read as zero, are cleared once
-    for (uint32_t i = threadIdx.x; i < (MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4) / 16; i += 64 * NW)
+    for (uint32_t i = threadIdx.x; i < MT_STAGE_BYTES / 16; i += 64 * NW)
         ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
     __syncthreads();
 
     for (uint32_t c0 = c_begin; c0 < c_end; c0 += MT_KC) {
-        stager.park(xa, xs, xinv);
+        stager.park(xa, xs, xinv, xv);
         ws[0].store(wwin);
         __syncthreads();
         // the next chunk of X and of the weights travels while this one is multiplied
@@ -534,7 +553,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                         t_u32x2 w[4];
 #pragma unroll
                         for (int g = 0; g < 4; ++g) w[g] = *(const t_u32x2*)(blk + 16u + 32u * g + 8u * kq);
-                        q4k_mtile_block(hdr, w, xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                        q4k_mtile_block(hdr, w, xa + (size_t)bb * (8 * 2 * 1024), xv + (size_t)bb * 2048, xinv + bb * 16, lane, tot);
                     }
                 }
             }
@@ -542,7 +561,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         __syncthreads();
     }
     } else {
-    for (uint32_t i = threadIdx.x; i < (MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4) / 16; i += 64 * NW)
+    for (uint32_t i = threadIdx.x; i < MT_STAGE_BYTES / 16; i += 64 * NW)
         ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
     __syncthreads();
     const uint8_t* wrow = wmat + (size_t)min(row, p.N - 1u) * p.row_stride_bytes;
@@ -565,7 +584,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                 for (int g = 0; g < 4; ++g) w[i][g] = *(const t_u32x2*)(blk + 16u + 32u * g + 8u * kq);
             }
         }
-        stager.park(xa, xs, xinv);
+        stager.park(xa, xs, xinv, xv);
         __syncthreads();
         if (c0 + MT_KC < c_end) stager.fetch(p, c0 + MT_KC);   // the next chunk of X travels while this one is multiplied
         if (has_tile) {
@@ -664,7 +683,7 @@ static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t 
 {
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
     constexpr int PITCH = Q6 ? (R == 1 ? 240 : 464) : (R == 1 ? 160 : 304);   // as in the kernel
-    constexpr size_t shmem = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * sizeof(float) + (STAGED ? (size_t)NW * 16 * PITCH : 0);
+    constexpr size_t shmem = MT_STAGE_BYTES + (STAGED ? (size_t)NW * 16 * PITCH : 0);
     auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK>;
     static bool raised = false;   // per instantiation
     if (!raised) {
