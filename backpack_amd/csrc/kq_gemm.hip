@@ -583,9 +583,10 @@ static hipError_t launch_gemm(const GemmParams& p, hipStream_t s)
     return hipGetLastError();
 }
 
-// 256-tile kernel.  even_shares: cut the walk into one equal share per CU; else one tile per workgroup.
+// 256-tile kernel.  share = k steps per workgroup: nk for one tile per workgroup, otherwise the walk over all
+// (tile, k step) units is cut into runs of that length.
 template <int TYPE>
-static hipError_t launch_gemm_persistent(GemmParams p, bool even_shares, hipStream_t s)
+static hipError_t launch_gemm_persistent(GemmParams p, uint32_t share, hipStream_t s)
 {
     constexpr size_t shmem = 2 * (size_t)(256 + 256) * GEMM_LD;
     auto kern = gemm_bf16_sk_kernel<TYPE>;
@@ -599,8 +600,7 @@ static hipError_t launch_gemm_persistent(GemmParams p, bool even_shares, hipStre
     p.tiles_n = (p.N + 255u) / 256u;
     const uint32_t tiles = ((p.M + 255u) / 256u) * p.tiles_n;
     p.units = tiles * nk;
-    const uint32_t cus = device_cu_count();
-    p.units_per_wg = even_shares ? (p.units + cus - 1u) / cus : nk;
+    p.units_per_wg = share;
     const uint32_t wgs = (p.units + p.units_per_wg - 1u) / p.units_per_wg;
     if (wgs > 1u && p.units_per_wg % nk != 0u)
         hipLaunchKernelGGL(gemm_clear_split_tiles_kernel, dim3(wgs - 1u), dim3(256), 0, s, p);
@@ -625,14 +625,24 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, hipStream_
     // workgroups per CU.  With many tiles per CU, equal shares also remove the ragged last round.
     const uint32_t cus = device_cu_count(), nk = a.K / GEMM_BK;
     const uint64_t big = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 255u) / 256u);
-    bool use_big, even;
-    if (big * 2u > cus) { use_big = true; even = big >= 8ull * cus; }
-    else { use_big = nk >= 128u && big * nk >= 16ull * cus; even = true; }
+    // A cut tile is summed with atomics, which is order-independent for two addends only: the automatic
+    // choices never cut a tile into more than two runs.
+    const uint32_t one_per_cu = (uint32_t)((big * nk + cus - 1u) / cus);   // equal shares over all CUs
+    bool use_big;
+    uint32_t share = nk;
+    if (big * 2u > cus) {
+        use_big = true;
+        if (big >= 8ull * cus) share = one_per_cu;   // >= 8 tiles each: at most one cut per tile
+    } else {
+        use_big = nk >= 128u && big * nk >= 16ull * cus;
+        share = nk / 2u;                             // every tile in two halves (nk is a multiple of 4)
+    }
     if (tile == 256) use_big = true;
     if (tile == 128) use_big = false;
-    if (split == 1) even = false;
-    if (split == 2) even = true;
-    if (use_big) return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, even, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, even, s);
+    if (split == 1) share = nk;
+    if (split == 2) share = one_per_cu;              // forced: any number of runs per tile
+    (void)cus;
+    if (use_big) return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, share, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, share, s);
     return q4 ? launch_gemm<KQ_TYPE_Q4_K, 128, 128, 4>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 128, 128, 4>(p, s);
 }
 

@@ -324,6 +324,31 @@ def _bf16_bits(x32):
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
+@pytest.mark.parametrize("type_,M,N,K", [(Q6_K, 1024, 2048, 8192),    # 32 big tiles, long K: every tile cut in two halves
+                                          (Q4_K, 2048, 5120, 512)])    # 160 tiles: one tile per workgroup
+def test_gemm_bf16_repeatable(gpu, type_, M, N, K):
+    """The automatic work split never sums more than two partial tiles per element, so a call repeated on the
+    same inputs gives the same bits (fp32 atomics on cleared memory commute for two addends)."""
+    import torch
+    from backpack_amd import capi, kquant
+    raw, packed, w = gpu.make_weight(type_, N, K, seed=7)
+    rng = np.random.default_rng(11)
+    bits = _bf16_bits(rng.standard_normal((M, K)).astype(np.float32))
+    xd = torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
+    _say("gemm repeat", type_, M, N, K)
+    first = kquant.matmul(xd, w).cpu().numpy()
+    assert capi.last_kernel() == "gemm_bf16"
+    capi.set_option("gemm_split", 1)    # the same tiles, each walked by one workgroup: no atomics
+    try:
+        whole = kquant.matmul(xd, w).cpu().numpy()
+    finally:
+        capi.set_option("gemm_split", 0)
+    assert np.allclose(first, whole, rtol=0, atol=1e-4 * float(np.abs(whole).max()))
+    for _ in range(3):
+        again = kquant.matmul(xd, w).cpu().numpy()
+        assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+
+
 @pytest.mark.parametrize("type_,M,N,K,tile", GEMM_SHAPES)
 def test_gemm_bf16_vs_oracle(gpu, kqo, type_, M, N, K, tile):
     import torch
