@@ -232,6 +232,22 @@ def test_gemv_stream_shapes(gpu, kqo, type_, N, K, depth, rows_per_wave, M):
                      label=f"stream {type_} {N}x{K} d{depth} r{rows_per_wave}")
 
 
+@pytest.mark.parametrize("type_,M,N,K", [(Q6_K, 5, 4096, 14336), (Q4_K, 16, 6144, 4096)])
+def test_tile_kernel_k_split_repeatable_and_counters_rearmed(gpu, type_, M, N, K):
+    """Matrices of few rows: K is cut over workgroups and the last one to arrive adds the partial tiles in
+    split order, so repeated calls give the same bits; the arrival counters are back at zero for the next."""
+    import torch
+    from backpack_amd import capi, kquant
+    raw, packed, w = gpu.make_weight(type_, N, K, seed=5)
+    x = torch.from_numpy(np.random.default_rng(3).standard_normal((M, K)).astype(np.float32)).cuda()
+    _say("mtile repeat", type_, M, N, K)
+    first = kquant.matmul(x, w).cpu().numpy()
+    assert capi.last_kernel() == "mtile"
+    for _ in range(3):
+        again = kquant.matmul(x, w).cpu().numpy()
+        assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+
+
 def test_matmul_y_offset_no_bias(gpu, kqo):
     import torch
     from backpack_amd import kquant
