@@ -29,6 +29,11 @@ class WeightDesc(C.Structure):
                 ("data", C.c_void_p), ("bytes", C.c_size_t)]
 
 
+class GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("type", C.c_uint32), ("n_dims", C.c_uint32), ("dims", C.c_uint64 * 4),
+                ("offset", C.c_uint64), ("bytes", C.c_uint64), ("data", C.c_void_p)]
+
+
 _SIGS = {
     "bpk_version": (C.c_int, []),
     "bpk_last_error": (C.c_char_p, []),
@@ -43,6 +48,24 @@ _SIGS = {
                                     C.POINTER(C.c_uint32), C.POINTER(C.c_void_p)]),
     "bpk_weight_describe": (C.c_int, [C.c_void_p, C.POINTER(WeightDesc)]),
     "bpk_weight_destroy": (C.c_int, [C.c_void_p]),
+    "bpk_gguf_open": (C.c_int, [C.c_char_p, C.POINTER(C.c_void_p)]),
+    "bpk_gguf_close": (C.c_int, [C.c_void_p]),
+    "bpk_gguf_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint32), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64),
+                                C.POINTER(C.c_uint64)]),
+    "bpk_gguf_tensor_at": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(GgufTensor)]),
+    "bpk_gguf_find_tensor": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(GgufTensor)]),
+    "bpk_gguf_has_key": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "bpk_gguf_key_type": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "bpk_gguf_get_u32": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint32, C.POINTER(C.c_uint32)]),
+    "bpk_gguf_get_f32": (C.c_int, [C.c_void_p, C.c_char_p, C.c_float, C.POINTER(C.c_float)]),
+    "bpk_gguf_get_bool": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.POINTER(C.c_int)]),
+    "bpk_gguf_get_string": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t)]),
+    "bpk_gguf_array_len": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)]),
+    "bpk_gguf_array_string": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_void_p, C.c_size_t,
+                                        C.POINTER(C.c_size_t)]),
+    "bpk_gguf_array_data": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_uint64),
+                                      C.POINTER(C.c_uint32)]),
+    "bpk_gguf_weight_create": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.c_uint32, C.POINTER(C.c_void_p)]),
     "bpk_kq_matmul": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
                                 C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p]),
     "bpk_kq_matmul_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,

@@ -9,6 +9,7 @@
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <thread>
 #include <vector>
 
 #include "kq_format.h"
@@ -37,15 +38,38 @@ int fail(int code, const char* fmt, ...)
     return code;
 }
 
+}  // namespace
+
+// The same for the library's other sources: stores the message bpk_last_error() returns.
+namespace kq {
+int api_fail(int code, const char* fmt, va_list ap)
+{
+    vsnprintf(t_err, sizeof t_err, fmt, ap);
+    return code;
+}
+}  // namespace kq
+
+namespace {
+
 int hip_fail(hipError_t e, const char* what)
 {
     return fail(BPK_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+// Pinned double buffer of the weight upload: one half is filled by host threads while the other is in
+// flight to the device.
+constexpr size_t kStageBytes = size_t(32) << 20;
+struct UploadStage {
+    void* buf[2] = {nullptr, nullptr};
+    hipEvent_t sent[2] = {nullptr, nullptr};
+    hipStream_t stream = nullptr;
+};
+
 struct DeviceState {
     bool ready = false;
     kq::SplitScratch split{};
     uint32_t* moe_tiles = nullptr;   // kMoeWords words
+    UploadStage up{};                // created by the first upload on the device
 };
 
 std::mutex g_mu;
@@ -168,6 +192,11 @@ int bpk_shutdown(void)
         (void)hipFree(st.split.partial);
         (void)hipFree(st.split.counters);
         (void)hipFree(st.moe_tiles);
+        for (int b = 0; b < 2; ++b) {
+            if (st.up.buf[b]) (void)hipHostFree(st.up.buf[b]);
+            if (st.up.sent[b]) (void)hipEventDestroy(st.up.sent[b]);
+        }
+        if (st.up.stream) (void)hipStreamDestroy(st.up.stream);
         st = DeviceState{};
     }
     if (cur >= 0) (void)hipSetDevice(cur);
@@ -204,6 +233,31 @@ struct bpk_weight {
     int device;
 };
 
+// Packed rows [row0, row0+n) of the stacked matrix -> dst (n*stride bytes).  Parts are raw GGUF rows of
+// row_bytes each; a packed row is the raw row plus zero padding to the word boundary.
+static void pack_stacked_rows(const void* const* parts, const uint32_t* n_rows, uint32_t n_parts, uint64_t row0,
+                              uint64_t n, size_t row_bytes, size_t stride, uint8_t* dst)
+{
+    uint64_t first = 0;
+    for (uint32_t i = 0; i < n_parts && n; first += n_rows[i], ++i) {
+        if (row0 >= first + n_rows[i]) continue;
+        const uint64_t r = row0 - first;
+        const uint64_t take = n_rows[i] - r < n ? n_rows[i] - r : n;
+        const uint8_t* src = (const uint8_t*)parts[i] + r * row_bytes;
+        if (stride == row_bytes) {
+            memcpy(dst, src, take * row_bytes);
+        } else {
+            for (uint64_t k = 0; k < take; ++k) {
+                memcpy(dst + k * stride, src + k * row_bytes, row_bytes);
+                memset(dst + k * stride + row_bytes, 0, stride - row_bytes);
+            }
+        }
+        dst += take * stride;
+        row0 += take;
+        n -= take;
+    }
+}
+
 int bpk_weight_create(int type, uint32_t K, uint32_t n_parts, const void* const* parts, const uint32_t* n_rows,
                       bpk_weight** out)
 {
@@ -220,27 +274,64 @@ int bpk_weight_create(int type, uint32_t K, uint32_t n_parts, const void* const*
     if (int rc = current_state(&st)) return rc;
     uint32_t nb, rs;
     bpk_kq_layout(type, K, &nb, &rs);
-    const size_t bytes = (size_t)N * rs * 4u;
-    std::vector<uint32_t> host;
-    try {
-        host.resize((size_t)N * rs);
-    } catch (const std::bad_alloc&) {
-        return fail(BPK_ERR_SHAPE, "host staging of %zu bytes failed", bytes);
-    }
-    size_t row = 0;
-    for (uint32_t i = 0; i < n_parts; ++i) {
-        bpk_kq_pack_host(type, parts[i], n_rows[i], K, host.data() + row * rs);
-        row += n_rows[i];
+    const size_t row_bytes = (size_t)nb * kq::block_bytes(type), stride = (size_t)rs * 4u;
+    if (stride > kStageBytes) return fail(BPK_ERR_SHAPE, "a row of %zu bytes exceeds the upload stage", stride);
+    const size_t bytes = (size_t)N * stride;
+
+    // One upload at a time per process: the stage is shared.
+    static std::mutex up_mu;
+    std::lock_guard<std::mutex> lk(up_mu);
+    UploadStage& up = st->up;
+    hipError_t e = hipSuccess;
+    if (!up.stream) {
+        e = hipStreamCreateWithFlags(&up.stream, hipStreamNonBlocking);
+        for (int b = 0; b < 2 && e == hipSuccess; ++b) {
+            e = hipHostMalloc(&up.buf[b], kStageBytes, hipHostMallocDefault);
+            if (e == hipSuccess) e = hipEventCreateWithFlags(&up.sent[b], hipEventDisableTiming);
+        }
+        if (e != hipSuccess) return hip_fail(e, "creating the upload stage");
     }
     void* dptr = nullptr;
     // 16 trailing bytes let 128-bit loads of the last row's tail stay in bounds
-    hipError_t e = hipMalloc(&dptr, bytes + 16);
+    e = hipMalloc(&dptr, bytes + 16);
     if (e != hipSuccess) return hip_fail(e, "hipMalloc(weights)");
-    e = hipMemcpy(dptr, host.data(), bytes, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMemset((uint8_t*)dptr + bytes, 0, 16);
+
+    const uint64_t rows_per_chunk = kStageBytes / stride;
+    const unsigned hw = std::thread::hardware_concurrency();
+    const unsigned n_threads = hw >= 8 ? 8 : (hw ? hw : 1);
+    uint64_t row = 0;
+    for (uint64_t c = 0; row < N && e == hipSuccess; ++c) {
+        const int b = (int)(c & 1);
+        if (c >= 2) e = hipEventSynchronize(up.sent[b]);
+        if (e != hipSuccess) break;
+        const uint64_t n = N - row < rows_per_chunk ? N - row : rows_per_chunk;
+        uint8_t* dst = (uint8_t*)up.buf[b];
+        // host threads share the chunk's rows; small chunks are not worth a thread each
+        const unsigned t_use = n * stride >= (size_t(4) << 20) ? n_threads : 1;
+        if (t_use == 1) {
+            pack_stacked_rows(parts, n_rows, n_parts, row, n, row_bytes, stride, dst);
+        } else {
+            std::vector<std::thread> pool;
+            const uint64_t per = (n + t_use - 1) / t_use;
+            for (unsigned t = 0; t < t_use; ++t) {
+                const uint64_t r0 = t * per;
+                if (r0 >= n) break;
+                const uint64_t cnt = n - r0 < per ? n - r0 : per;
+                pool.emplace_back(pack_stacked_rows, parts, n_rows, n_parts, row + r0, cnt, row_bytes, stride,
+                                  dst + r0 * stride);
+            }
+            for (auto& th : pool) th.join();
+        }
+        e = hipMemcpyAsync((uint8_t*)dptr + row * stride, dst, n * stride, hipMemcpyHostToDevice, up.stream);
+        if (e == hipSuccess) e = hipEventRecord(up.sent[b], up.stream);
+        row += n;
+    }
+    if (e == hipSuccess) e = hipMemsetAsync((uint8_t*)dptr + bytes, 0, 16, up.stream);
+    const hipError_t e_sync = hipStreamSynchronize(up.stream);   // also on failure: the stage must be idle on return
+    if (e == hipSuccess) e = e_sync;
     if (e != hipSuccess) {
         (void)hipFree(dptr);
-        return hip_fail(e, "hipMemcpy(weights)");
+        return hip_fail(e, "uploading weights");
     }
     bpk_weight* w = new (std::nothrow) bpk_weight;
     if (!w) {

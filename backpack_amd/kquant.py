@@ -64,6 +64,38 @@ def from_raw(type_: int, raw: np.ndarray, N: int, K: int, device="cuda") -> KQua
     return upload(type_, pack_host(type_, raw, N, K), N, K, device)
 
 
+class _LibraryWeight:
+    """Device allocation owned by the library (bpk_weight); freed with the object."""
+
+    def __init__(self, handle, desc):
+        self._h, self._ptr, self.nbytes = handle, desc.data, desc.bytes
+        self.device = torch.device("cuda", torch.cuda.current_device())
+
+    def data_ptr(self) -> int:
+        return self._ptr
+
+    def __del__(self):
+        try:
+            if self._h:
+                capi.lib().bpk_weight_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+def from_gguf(g, names) -> KQuantPacked:
+    """Named Q4_K / Q6_K tensors of an open GGUFFile -> one device weight, rows stacked in order
+    (the loader's tensor -> packKQ -> fuseKQ -> uploadKQWeight, runtime/model_runner.cpp:1275-1338)."""
+    import ctypes as C
+    names = [names] if isinstance(names, str) else list(names)
+    arr = (C.c_char_p * len(names))(*[n.encode() for n in names])
+    h = C.c_void_p()
+    capi.check(capi.lib().bpk_gguf_weight_create(g.handle, arr, len(names), C.byref(h)))
+    d = capi.WeightDesc()
+    capi.check(capi.lib().bpk_weight_describe(h, C.byref(d)))
+    return KQuantPacked(_LibraryWeight(h, d), d.type, d.N, d.K, d.row_stride_words, d.n_blocks)
+
+
 def fuse(parts: list[KQuantPacked]) -> KQuantPacked:
     """Row-wise concatenation of matrices with equal K and type (fuseKQ)."""
     a = parts[0]

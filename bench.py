@@ -54,6 +54,8 @@ def parse():
     ap.add_argument("--moe", action="store_true",
                     help="also time the Qwen3-30B-A3B-shaped routed-expert FFN at T = 1 and T = 256")
     ap.add_argument("--all", action="store_true", help="--prefill --verify --moe")
+    ap.add_argument("--load", action="store_true",
+                    help="also write a GGUF file of Q4_K / Q6_K matrices and time file -> device weights")
     ap.add_argument("--gemm-tile", type=int, default=0,
                     help="force the prefill GEMM tile (0 = the library's own choice)")
     ap.add_argument("--gemm-split", type=int, default=0,
@@ -275,6 +277,8 @@ def main():
         out["verify"] = verify_leg(mats, wb, use_graph)
     if args.moe or args.all:
         out["moe"] = moe_leg()
+    if args.load:
+        out["gguf_load"] = load_leg()
     if not args.no_prefill:
         # the second half of the metric: M=2048 dequant-GEMM TFLOP/s and its fraction of the bf16 MFMA peak
         out["prefill"] = prefill_leg()
@@ -286,6 +290,63 @@ def main():
         torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
+
+
+def load_leg(n_layers=8):
+    """GGUF file -> device weights: a file of n_layers x [gate, up (Q4_K, stacked into one weight), down
+    (Q6_K)] at the layer set's shapes is written to the temporary directory, opened, and every weight is
+    created from it.  Two passes: the second finds the file in the page cache and the upload stage warm."""
+    import tempfile
+    import struct
+    import numpy as np
+    import torch
+    from backpack_amd import capi, kquant, synth
+    from backpack_amd.gguf import GGUFFile
+    H, I = 4096, 14336
+    rng = np.random.default_rng(0)
+
+    def raw(type_, N, K):
+        nb = K // 256
+        bb = 144 if type_ == synth.Q4_K else 210
+        return rng.integers(0, 256, size=N * nb * bb, dtype=np.uint8)
+    tensors = []
+    for l in range(n_layers):
+        tensors += [(f"blk.{l}.ffn_gate.weight", (H, I), synth.Q4_K), (f"blk.{l}.ffn_up.weight", (H, I), synth.Q4_K),
+                    (f"blk.{l}.ffn_down.weight", (I, H), synth.Q6_K)]
+
+    def s(b):
+        return struct.pack("<Q", len(b)) + b
+    with tempfile.TemporaryDirectory() as d:
+        path = d + "/load.gguf"
+        head = struct.pack("<IIQQ", 0x46554747, 3, len(tensors), 0)
+        datas, pos = [], 0
+        for name, dims, type_ in tensors:
+            body = raw(type_, dims[1], dims[0])
+            pos = (pos + 31) // 32 * 32
+            head += s(name.encode()) + struct.pack("<IQQIQ", 2, dims[0], dims[1], type_, pos)
+            datas.append((pos, body))
+            pos += body.size
+        data_offset = (len(head) + 31) // 32 * 32
+        with open(path, "wb") as f:
+            f.write(head)
+            for off, body in datas:
+                f.seek(data_offset + off)
+                f.write(body.tobytes())
+        total = sum(b.size for _, b in datas)
+        del datas
+        res = {"file_bytes": data_offset + pos, "weight_bytes": total}
+        for label in ("first_pass", "second_pass"):
+            t0 = time.perf_counter()
+            ws = []
+            with GGUFFile(path) as g:
+                for l in range(n_layers):
+                    ws.append(kquant.from_gguf(g, [f"blk.{l}.ffn_gate.weight", f"blk.{l}.ffn_up.weight"]))
+                    ws.append(kquant.from_gguf(g, f"blk.{l}.ffn_down.weight"))
+            torch.cuda.synchronize()
+            sec = time.perf_counter() - t0
+            res[label] = {"s": round(sec, 3), "GBps": round(total / sec / 1e9, 2)}
+            del ws
+    return res
 
 
 def config0_leg():

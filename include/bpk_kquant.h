@@ -44,7 +44,10 @@ enum {
     BPK_ERR_ALIGN = -4,     /* pointer or stride alignment not met            */
     BPK_ERR_HIP = -5,       /* a HIP runtime call failed                      */
     BPK_ERR_DEVICE = -6,    /* the current device is not gfx950               */
-    BPK_ERR_WORKSPACE = -7  /* workspace missing or too small                 */
+    BPK_ERR_WORKSPACE = -7, /* workspace missing or too small                 */
+    BPK_ERR_IO = -8,        /* a file could not be opened or mapped           */
+    BPK_ERR_FORMAT = -9,    /* not a GGUF file, or truncated / inconsistent   */
+    BPK_ERR_NOT_FOUND = -10 /* no tensor / metadata element of that name      */
 };
 
 /* Library version, major*10000 + minor*100 + patch. */
@@ -98,6 +101,78 @@ BPK_API int bpk_weight_create(int type, uint32_t K, uint32_t n_parts,
                               bpk_weight **out);
 BPK_API int bpk_weight_describe(const bpk_weight *w, bpk_weight_desc *out);
 BPK_API int bpk_weight_destroy(bpk_weight *w);
+
+/* ---- GGUF container: replaces GGUFFile for this path ----------------------
+ * runtime/gguf_loader.h:49-86 (GGUFFile, its getters) and
+ * runtime/gguf_loader.cpp:90-182 (open: magic "GGUF", version, tensor and
+ * key-value counts, typed key-value pairs, tensor table, data section at the
+ * next aligned offset).  The file is memory-mapped read-only and every length
+ * and offset in it is checked against the file size.  Versions 2 and 3.
+ * `general.alignment` is honoured when present (default 32, the constant of
+ * gguf_loader.cpp:151).  Pointers returned (names, data) stay valid until
+ * bpk_gguf_close. */
+typedef struct bpk_gguf bpk_gguf;
+
+typedef struct bpk_gguf_tensor {
+    const char *name;   /* NUL-terminated                                   */
+    uint32_t type;      /* GGUF tensor type code (runtime/gguf_loader.h:23-36) */
+    uint32_t n_dims;    /* 0..4                                             */
+    uint64_t dims[4];   /* dims[0] = row length (K); unused entries are 1   */
+    uint64_t offset;    /* from the start of the data section               */
+    uint64_t bytes;     /* size of the data; 0 when the type is not known here */
+    const void *data;   /* host address inside the mapping                  */
+} bpk_gguf_tensor;
+
+BPK_API int bpk_gguf_open(const char *path, bpk_gguf **out);
+BPK_API int bpk_gguf_close(bpk_gguf *g);
+/* Any of the out pointers may be NULL. */
+BPK_API int bpk_gguf_info(const bpk_gguf *g, uint32_t *version,
+                          uint64_t *n_tensors, uint64_t *n_kv,
+                          uint64_t *data_offset);
+/* Tensors in file order / by name (GGUFFile::tensors, ::tensor_index). */
+BPK_API int bpk_gguf_tensor_at(const bpk_gguf *g, uint64_t index,
+                               bpk_gguf_tensor *out);
+BPK_API int bpk_gguf_find_tensor(const bpk_gguf *g, const char *name,
+                                 bpk_gguf_tensor *out);
+
+/* Metadata getters with the reference's defaults-and-coercions behaviour
+ * (runtime/gguf_loader.cpp:155-182): a missing key or a value of another kind
+ * yields `def`, never an error.  get_u32 accepts integers of any width and, for
+ * an int32/uint32 array, returns its largest element (gguf_loader.cpp:158-166).
+ * get_f32 accepts f32 and f64.  has_key returns 1 or 0. */
+BPK_API int bpk_gguf_has_key(const bpk_gguf *g, const char *key);
+/* GGUF metadata value type code of the key (0 u8 .. 8 string, 9 array, 10 u64,
+ * 11 i64, 12 f64), or -1 when absent. */
+BPK_API int bpk_gguf_key_type(const bpk_gguf *g, const char *key);
+BPK_API int bpk_gguf_get_u32(const bpk_gguf *g, const char *key, uint32_t def,
+                             uint32_t *out);
+BPK_API int bpk_gguf_get_f32(const bpk_gguf *g, const char *key, float def,
+                             float *out);
+BPK_API int bpk_gguf_get_bool(const bpk_gguf *g, const char *key, int def,
+                              int *out);
+/* Copies at most cap-1 bytes into buf and terminates it; *len (may be NULL)
+ * receives the full length, 0 when the key is absent or not a string. */
+BPK_API int bpk_gguf_get_string(const bpk_gguf *g, const char *key, char *buf,
+                                size_t cap, size_t *len);
+/* Arrays (GGUFFile::getStringArray etc., runtime/gguf_loader.h:73-85): element
+ * count and element type code (0 when absent), one string element, and the
+ * address of the packed elements of a fixed-size-element array. */
+BPK_API int bpk_gguf_array_len(const bpk_gguf *g, const char *key, uint64_t *n,
+                               uint32_t *elem_type);
+BPK_API int bpk_gguf_array_string(const bpk_gguf *g, const char *key,
+                                  uint64_t index, char *buf, size_t cap,
+                                  size_t *len);
+BPK_API int bpk_gguf_array_data(const bpk_gguf *g, const char *key,
+                                const void **data, uint64_t *n,
+                                uint32_t *elem_type);
+
+/* Named Q4_K / Q6_K matrices of the file (GGUF shape {K, N}) -> one device
+ * weight with the rows stacked in the order given: the tensor -> packKQ ->
+ * fuseKQ -> uploadKQWeight sequence of runtime/model_runner.cpp:1275-1338
+ * (q|k|v and gate|up are stacked that way there).  All parts must share type
+ * and K; another tensor type fails with BPK_ERR_TYPE. */
+BPK_API int bpk_gguf_weight_create(const bpk_gguf *g, const char *const *names,
+                                   uint32_t n_names, bpk_weight **out);
 
 /* ---- matmul: replaces the q4k_matmul* / q6k_matmul* dispatches -------------
  * Bindings 0:X 1:W 2:Bias 3:Y 4:P of runtime/kernels/quant_kq/q4k_matmul.wgsl:20-95,

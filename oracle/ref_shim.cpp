@@ -6,7 +6,9 @@
 // its own: every call forwards to pack_q4k / pack_q6k / dequant_kquant
 // (runtime/gguf_loader.h:108-124, :147) so the restatement in kq_oracle.c can
 // be compared with the reference as this compiler builds it, and so the
-// benchmark can time the reference's real CPU path.
+// benchmark can time the reference's real CPU path; the bpref_gguf_* calls
+// forward to GGUFFile (runtime/gguf_loader.h:56-86) so the library's container
+// reader can be compared with the reference's parser on the same files.
 #include "gguf_loader.h"
 
 #include <chrono>
@@ -58,6 +60,92 @@ int bpref_matmul_timed(int type, const float* X, const void* raw, float* deq,
     if (t_dequant) *t_dequant = std::chrono::duration<double>(t1 - t0).count();
     if (t_dot) *t_dot = std::chrono::duration<double>(t2 - t1).count();
     return 0;
+}
+
+// ---- GGUFFile, field by field ------------------------------------------------
+void* bpref_gguf_open(const char* path)
+{
+    GGUFFile* g = new GGUFFile;
+    if (!g->open(path)) { delete g; return nullptr; }
+    return g;
+}
+
+void bpref_gguf_close(void* h) { delete (GGUFFile*)h; }
+
+void bpref_gguf_info(const void* h, uint32_t* version, uint64_t* n_tensors, uint64_t* data_offset)
+{
+    const GGUFFile* g = (const GGUFFile*)h;
+    *version = g->version;
+    *n_tensors = g->n_tensors;
+    *data_offset = g->data_offset;
+}
+
+// name: pointer into the GGUFFile (valid until close); dims: up to 8 entries.
+int bpref_gguf_tensor(const void* h, uint64_t i, const char** name, uint32_t* type, uint32_t* n_dims,
+                      uint64_t* dims, uint64_t* offset)
+{
+    const GGUFFile* g = (const GGUFFile*)h;
+    if (i >= g->tensors.size()) return -1;
+    const GGUFTensorInfo& t = g->tensors[i];
+    *name = t.name.c_str();
+    *type = (uint32_t)t.type;
+    *n_dims = (uint32_t)t.shape.size();
+    for (size_t d = 0; d < t.shape.size() && d < 8; d++) dims[d] = t.shape[d];
+    *offset = t.offset;
+    return 0;
+}
+
+int64_t bpref_gguf_find(const void* h, const char* name)
+{
+    const GGUFFile* g = (const GGUFFile*)h;
+    auto it = g->tensor_index.find(name);
+    return it == g->tensor_index.end() ? -1 : (int64_t)it->second;
+}
+
+int bpref_gguf_has_key(const void* h, const char* key) { return ((const GGUFFile*)h)->hasKey(key) ? 1 : 0; }
+uint32_t bpref_gguf_u32(const void* h, const char* key, uint32_t def) { return ((const GGUFFile*)h)->getU32(key, def); }
+float bpref_gguf_f32(const void* h, const char* key, float def) { return ((const GGUFFile*)h)->getFloat(key, def); }
+int bpref_gguf_bool(const void* h, const char* key, int def) { return ((const GGUFFile*)h)->getBool(key, def != 0) ? 1 : 0; }
+
+// Copies getString(key, def) into buf (cap bytes, terminated); returns its length.
+size_t bpref_gguf_string(const void* h, const char* key, const char* def, char* buf, size_t cap)
+{
+    const std::string s = ((const GGUFFile*)h)->getString(key, def);
+    if (cap) {
+        const size_t n = s.size() < cap - 1 ? s.size() : cap - 1;
+        std::memcpy(buf, s.data(), n);
+        buf[n] = 0;
+    }
+    return s.size();
+}
+
+// Element count of a string array (-1 when the key holds none) and one element.
+int64_t bpref_gguf_string_array_len(const void* h, const char* key)
+{
+    auto* a = ((const GGUFFile*)h)->getStringArray(key);
+    return a ? (int64_t)a->size() : -1;
+}
+
+size_t bpref_gguf_string_array_at(const void* h, const char* key, uint64_t i, char* buf, size_t cap)
+{
+    auto* a = ((const GGUFFile*)h)->getStringArray(key);
+    if (!a || i >= a->size()) return 0;
+    const std::string& s = (*a)[i];
+    if (cap) {
+        const size_t n = s.size() < cap - 1 ? s.size() : cap - 1;
+        std::memcpy(buf, s.data(), n);
+        buf[n] = 0;
+    }
+    return s.size();
+}
+
+// int32 array: count (-1 when none); copies up to cap elements.
+int64_t bpref_gguf_i32_array(const void* h, const char* key, int32_t* out, uint64_t cap)
+{
+    auto* a = ((const GGUFFile*)h)->getI32Array(key);
+    if (!a) return -1;
+    for (uint64_t i = 0; i < a->size() && i < cap; i++) out[i] = (*a)[i];
+    return (int64_t)a->size();
 }
 
 }  // extern "C"
