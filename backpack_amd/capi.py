@@ -29,6 +29,13 @@ class WeightDesc(C.Structure):
                 ("data", C.c_void_p), ("bytes", C.c_size_t)]
 
 
+class Fusion(C.Structure):
+    _fields_ = [("prologue", C.c_int), ("norm_w", C.c_void_p), ("eps", C.c_float), ("residual", C.c_void_p)]
+
+
+PRO_NONE, PRO_RMS_NORM, PRO_SILU_MUL, PRO_GELU_MUL = range(4)
+
+
 class GgufTensor(C.Structure):
     _fields_ = [("name", C.c_char_p), ("type", C.c_uint32), ("n_dims", C.c_uint32), ("dims", C.c_uint64 * 4),
                 ("offset", C.c_uint64), ("bytes", C.c_uint64), ("data", C.c_void_p)]
@@ -68,6 +75,10 @@ _SIGS = {
     "bpk_gguf_weight_create": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.c_uint32, C.POINTER(C.c_void_p)]),
     "bpk_kq_matmul": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
                                 C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p]),
+    "bpk_kq_matmul_fused_workspace_bytes": (C.c_size_t, [C.c_uint32, C.c_uint32, C.c_uint32]),
+    "bpk_kq_matmul_fused": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
+                                      C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32,
+                                      C.POINTER(Fusion), C.c_void_p, C.c_size_t, C.c_void_p]),
     "bpk_kq_matmul_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
                                      C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p]),
     "bpk_kq_dequant_rows": (C.c_int, [C.c_int, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_uint32,

@@ -28,6 +28,7 @@ thread_local int t_family = 0;
 thread_local kq::GemvTuning t_gemv;
 thread_local int t_gemm_tile = 0;
 thread_local int t_gemm_split = 0;
+thread_local int t_fused_separate = 0;
 
 int fail(int code, const char* fmt, ...)
 {
@@ -168,6 +169,10 @@ int bpk_set_option(const char* name, int value)
     if (!strcmp(name, "gemm_tile")) {
         if (value != 0 && value != 128 && value != 256) return fail(BPK_ERR_SHAPE, "gemm_tile must be 0, 128 or 256");
         t_gemm_tile = value;
+        return BPK_OK;
+    }
+    if (!strcmp(name, "fused_separate")) {
+        t_fused_separate = value != 0;
         return BPK_OK;
     }
     if (!strcmp(name, "gemm_split")) {
@@ -411,6 +416,67 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
         e = kq::launch_matmul_generic(a, s);
     }
     return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+size_t bpk_kq_matmul_fused_workspace_bytes(uint32_t M, uint32_t N, uint32_t K)
+{
+    const size_t x = ((size_t)M * K * sizeof(float) + 255u) & ~(size_t)255u;
+    return x + (size_t)M * N * sizeof(float);
+}
+
+int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bias, float* Y, uint32_t M, uint32_t N,
+                        uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, uint32_t y_offset,
+                        const bpk_kq_fusion* f, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!f) return fail(BPK_ERR_NULL, "fusion descriptor must be non-null");
+    if (f->prologue < BPK_PRO_NONE || f->prologue > BPK_PRO_GELU_MUL)
+        return fail(BPK_ERR_SHAPE, "prologue %d unknown", f->prologue);
+    if (f->prologue == BPK_PRO_RMS_NORM && !f->norm_w) return fail(BPK_ERR_NULL, "norm_w must be non-null for the norm prologue");
+    if (f->prologue == BPK_PRO_NONE && !f->residual)
+        return bpk_kq_matmul(type, X, W, bias, Y, M, N, K, n_blocks, row_stride_words, y_offset, stream);
+    if (int rc = check_matmul(type, X, W, Y, M, N, K, n_blocks, row_stride_words)) return rc;
+    if (((uintptr_t)f->norm_w | (uintptr_t)f->residual) & 3u) return fail(BPK_ERR_ALIGN, "norm_w and residual must be 4-byte aligned");
+    if (M == 0) return BPK_OK;
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    kq::MatmulArgs a{};
+    a.type = type; a.X = X; a.W = (const uint8_t*)W; a.bias = bias; a.Y = Y;
+    a.M = M; a.N = N; a.K = K; a.n_blocks = n_blocks;
+    a.row_stride_bytes = row_stride_words * 4u;
+    a.y_offset = y_offset;
+    a.ldy = N;
+    // one launch where the lanes-along-K kernel takes the shape
+    if (!t_fused_separate && (t_family == 0 || t_family == 5)) {
+        a.pro = f->prologue; a.norm_w = f->norm_w; a.eps = f->eps; a.residual = f->residual;
+        if (kq::gemv_stream_supported(a) && N <= 32768u) {
+            t_kernel = "gemv_stream_fused";
+            const hipError_t e = kq::launch_gemv_stream(a, t_gemv, s);
+            return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+        }
+        if (t_family == 5) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");
+    }
+    // otherwise the same function in up to three launches through the caller's workspace
+    const size_t x_bytes = ((size_t)M * K * sizeof(float) + 255u) & ~(size_t)255u;
+    const bool need_x = f->prologue != BPK_PRO_NONE, need_y = f->residual != nullptr;
+    const size_t need = (need_x ? x_bytes : 0) + (need_y ? (size_t)M * N * sizeof(float) : 0);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15u))
+        return fail(BPK_ERR_WORKSPACE, "this shape needs a 16-byte aligned workspace of %zu bytes (given %zu)", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    float* wx = (float*)workspace;
+    float* wy = (float*)((uint8_t*)workspace + (need_x ? x_bytes : 0));
+    if (need_x) {
+        const hipError_t e = kq::launch_prologue_rows(f->prologue, X, f->norm_w, f->eps, M, K, wx, s);
+        if (e != hipSuccess) return hip_fail(e, "prologue_rows");
+    }
+    if (int rc = bpk_kq_matmul(type, need_x ? wx : X, W, bias, need_y ? wy : Y, M, N, K, n_blocks, row_stride_words,
+                               need_y ? 0u : y_offset, stream))
+        return rc;
+    if (need_y) {
+        const hipError_t e = kq::launch_add_residual(wy, f->residual, Y, M, N, N, y_offset, s);
+        if (e != hipSuccess) return hip_fail(e, "add_residual");
+    }
+    return BPK_OK;
 }
 
 int bpk_kq_matmul_bf16(int type, const uint16_t* X, const void* W, const float* bias, float* Y, uint32_t M,

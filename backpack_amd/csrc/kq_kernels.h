@@ -26,6 +26,14 @@ struct MatmulArgs {
     const uint8_t* W2;
     float* Y2;
     const float* X2;
+    // fused forms of the dense decode matvec, honoured by the lanes-along-K launch only (other launches
+    // must be given pro == 0 and residual == nullptr): pro 1 = RMSNorm of the X row with weight norm_w,
+    // 2 / 3 = X rows are gate | up (2K floats) and x = silu / gelu_tanh (gate) * up; residual is added to
+    // every output (indexed like Y, may alias it)
+    int pro = 0;
+    const float* norm_w = nullptr;
+    float eps = 0.0f;
+    const float* residual = nullptr;
 };
 
 // Per-device scratch for split-K partial sums and arrival counters.
@@ -39,6 +47,13 @@ struct SplitScratch {
 hipError_t launch_dequant_rows(int type, const uint8_t* W, uint32_t row_stride_bytes,
                                const int32_t* rows, uint32_t M, uint32_t K, float* out,
                                hipStream_t s);
+
+// Stand-alone RMSNorm (pro 1) / silu-mul (2) / gelu-mul (3) of M rows into out [M,K], and
+// Y[m, y_offset + n] = T[m, n] + R[m, y_offset + n].
+hipError_t launch_prologue_rows(int pro, const float* X, const float* norm_w, float eps, uint32_t M, uint32_t K,
+                                float* out, hipStream_t s);
+hipError_t launch_add_residual(const float* T, const float* R, float* Y, uint32_t M, uint32_t N, uint32_t ldy,
+                               uint32_t y_offset, hipStream_t s);
 
 // Any shape with K % 256 == 0, any 4-byte aligned W.  M tiled by 4 inside.
 hipError_t launch_matmul_generic(const MatmulArgs& a, hipStream_t s);

@@ -27,28 +27,60 @@ namespace kq {
 typedef _Float16 s_half2 __attribute__((ext_vector_type(2)));
 typedef uint32_t s_u32x4 __attribute__((ext_vector_type(4)));
 
-struct StreamParams {
+// Kernel arguments come in three sizes, and a kernel is compiled for each: the wave's first
+// instructions fetch them, and every further 64 bytes of them cost a launch a measurable fraction of a
+// microsecond, so the dense decode matvec gets the smallest set that describes it.
+struct StreamDense {          // 56 bytes
     const float* X;
     const uint8_t* W;
     const float* bias;
     float* Y;
-    uint32_t N, K, n_blocks, row_stride_bytes, y_offset;
-    // expert indirection (nullptr for the dense case): blockIdx.y is a (token, slot) pair that uses
-    // weight rows expert_idx[pair]*N .. +N-1, X row pair / k_slots (or pair, x_per_slot) and Y row pair
+    uint32_t N, K, n_blocks, row_stride_bytes, y_offset, ldy;
+    static constexpr bool kGrouped = false, kFused = false;
+};
+
+// Dense matvec with a prologue on the activations (STREAM_PRO_*; for the act forms the X rows are
+// gate | up, 2K floats) and a term added to every output (indexed like Y; may be Y itself).
+struct StreamFused {
+    const float* X;
+    const uint8_t* W;
+    const float* bias;
+    float* Y;
+    uint32_t N, K, n_blocks, row_stride_bytes, y_offset, ldy;
+    int pro;
+    float eps;
+    const float* norm_w;
+    const float* residual;
+    static constexpr bool kGrouped = false, kFused = true;
+};
+
+// Expert indirection: blockIdx.y is a (token, slot) pair that uses weight rows expert_idx[pair]*N ..
+// +N-1, X row pair / k_slots (or pair, x_per_slot) and Y row pair.  MoE FFN fusions: a twin matrix of
+// the same shape served by blockIdx.z == 1 (gate and up read the same x), and an activation input:
+// x = silu(X) * X2 (down reads gate and up).
+struct StreamGrouped {
+    const float* X;
+    const uint8_t* W;
+    const float* bias;
+    float* Y;
+    uint32_t N, K, n_blocks, row_stride_bytes, y_offset, ldy;
     const uint32_t* expert_idx;
-    uint32_t k_slots, ldy;
+    uint32_t k_slots;
     int x_per_slot;
-    // MoE FFN fusions (grouped launches): a twin matrix of the same shape served by blockIdx.z == 1
-    // (gate and up read the same x), and an activation input: x = silu(X) * X2 (down reads gate and up)
     const uint8_t* W2;
     float* Y2;
     const float* X2;
+    static constexpr bool kGrouped = true, kFused = false;
 };
 
+constexpr int STREAM_PRO_NONE = 0;   // x = X
+constexpr int STREAM_PRO_NORM = 1;   // x = X * rsqrt(mean(X^2) + eps) * norm_w   (quant_kq/q4k_matmul_norm.wgsl:50-91)
+constexpr int STREAM_PRO_SILU = 2;   // x = silu(X) * X2                          (fused/silu_mul_fused.wgsl:39-49)
+constexpr int STREAM_PRO_GELU = 3;   // x = gelu_tanh(X) * X2                     (quant_kq/q4k_down_gelu.wgsl:50-56)
+
 // Redirects the pointers of a grouped launch to the pair this workgroup serves.
-__device__ __forceinline__ void stream_select_pair(StreamParams& p)
+__device__ __forceinline__ void stream_select_pair(StreamGrouped& p)
 {
-    if (!p.expert_idx) return;
     if (blockIdx.z) { p.W = p.W2; p.Y = p.Y2; }
     const uint32_t pair = blockIdx.y;
     p.W += (size_t)p.expert_idx[pair] * p.N * p.row_stride_bytes;
@@ -57,21 +89,79 @@ __device__ __forceinline__ void stream_select_pair(StreamParams& p)
     if (p.X2) p.X2 += xrow;
     p.Y += (size_t)pair * p.ldy;
 }
+__device__ __forceinline__ void stream_select_pair(StreamDense&) {}
+__device__ __forceinline__ void stream_select_pair(StreamFused&) {}
 
-// Four activations: X as it is, or silu(X) * X2 with silu(g) = g / (exp(-g) + 1) (the formula of
-// moe_silu_mul_kernel, so that the fused and the separate form agree to the bit).
-template <bool ACT>
-__device__ __forceinline__ float4 stream_x4(const StreamParams& p, const float4* xp)
+// Which prologue a launch runs, where the second activation input lies relative to the first (in
+// floats), and the distance between the X rows of two tokens.
+__device__ __forceinline__ int stream_pro(const StreamDense&) { return STREAM_PRO_NONE; }
+__device__ __forceinline__ int stream_pro(const StreamFused& p) { return p.pro; }
+__device__ __forceinline__ int stream_pro(const StreamGrouped& p) { return p.X2 ? STREAM_PRO_SILU : STREAM_PRO_NONE; }
+__device__ __forceinline__ ptrdiff_t stream_x2_off(const StreamDense&) { return 0; }
+__device__ __forceinline__ ptrdiff_t stream_x2_off(const StreamFused& p) { return (ptrdiff_t)p.K; }
+__device__ __forceinline__ ptrdiff_t stream_x2_off(const StreamGrouped& p) { return p.X2 - p.X; }
+__device__ __forceinline__ const float* stream_norm_w(const StreamFused& p) { return p.norm_w; }
+__device__ __forceinline__ float stream_eps(const StreamFused& p) { return p.eps; }
+template <typename PT> __device__ __forceinline__ const float* stream_norm_w(const PT&) { return nullptr; }
+template <typename PT> __device__ __forceinline__ float stream_eps(const PT&) { return 0.0f; }
+__device__ __forceinline__ const float* stream_residual(const StreamFused& p) { return p.residual; }
+template <typename PT> __device__ __forceinline__ const float* stream_residual(const PT&) { return nullptr; }
+__device__ __forceinline__ uint32_t stream_ldx(const StreamDense& p) { return p.K; }
+__device__ __forceinline__ uint32_t stream_ldx(const StreamFused& p) { return p.pro >= STREAM_PRO_SILU ? 2u * p.K : p.K; }
+__device__ __forceinline__ uint32_t stream_ldx(const StreamGrouped& p) { return p.K; }
+
+// silu(g) = g / (exp(-g) + 1) and the tanh form of gelu the reference uses.  The grouped (MoE) kernels
+// evaluate silu with expf and a true division, the formula of moe_silu_mul_kernel, so that their fused
+// and separate forms agree to the bit; the dense fused kernels use the hardware exponential and
+// reciprocal (a few units in the last place, far inside the path's 1e-3), because this arithmetic sits
+// in front of the first weight of every launch.
+template <int PRO, bool FAST>
+__device__ __forceinline__ float stream_act(float g, float u)
+{
+    if constexpr (PRO == STREAM_PRO_SILU) {
+        if constexpr (FAST) return g * __builtin_amdgcn_rcpf(__expf(-g) + 1.0f) * u;
+        else return g / (expf(-g) + 1.0f) * u;
+    } else {
+        const float inner = 0.7978845608f * (g + 0.044715f * g * g * g);
+        // tanh(z) = 1 - 2 / (exp(2z) + 1); 0.5 g (1 + tanh z) = g - g / (exp(2z) + 1)
+        const float e = __expf(2.0f * inner);
+        return (g - g * __builtin_amdgcn_rcpf(e + 1.0f)) * u;
+    }
+}
+
+// Four activations: X as it is (also for the norm, which scales afterwards), or act(X) * X2.
+template <int PRO, bool FAST>
+__device__ __forceinline__ float4 stream_x4(const float4* xp, ptrdiff_t x2_off)
 {
     float4 v = *xp;
-    if constexpr (ACT) {
-        const float4 u = *(const float4*)((const float*)xp - p.X + p.X2);
-        v.x = v.x / (expf(-v.x) + 1.0f) * u.x;
-        v.y = v.y / (expf(-v.y) + 1.0f) * u.y;
-        v.z = v.z / (expf(-v.z) + 1.0f) * u.z;
-        v.w = v.w / (expf(-v.w) + 1.0f) * u.w;
+    if constexpr (PRO == STREAM_PRO_SILU || PRO == STREAM_PRO_GELU) {
+        const float4 u = *(const float4*)((const float*)xp + x2_off);
+        v.x = stream_act<PRO, FAST>(v.x, u.x);
+        v.y = stream_act<PRO, FAST>(v.y, u.y);
+        v.z = stream_act<PRO, FAST>(v.z, u.z);
+        v.w = stream_act<PRO, FAST>(v.w, u.w);
     }
     return v;
+}
+
+// One branch around a whole x prologue, so that every form issues its loads back to back.
+// One branch around a whole x prologue, so that every form issues its loads back to back.  A kernel
+// carries only the forms its argument set can ask for.
+template <typename PT, typename F>
+__device__ __forceinline__ void stream_dispatch_pro(const PT& p, F&& f)
+{
+    if constexpr (PT::kFused) {
+        const int pro = stream_pro(p);
+        if (pro == STREAM_PRO_NONE) f(std::integral_constant<int, STREAM_PRO_NONE>{});
+        else if (pro == STREAM_PRO_SILU) f(std::integral_constant<int, STREAM_PRO_SILU>{});
+        else if (pro == STREAM_PRO_NORM) f(std::integral_constant<int, STREAM_PRO_NORM>{});
+        else f(std::integral_constant<int, STREAM_PRO_GELU>{});
+    } else if constexpr (PT::kGrouped) {
+        if (stream_pro(p) == STREAM_PRO_SILU) f(std::integral_constant<int, STREAM_PRO_SILU>{});
+        else f(std::integral_constant<int, STREAM_PRO_NONE>{});
+    } else {
+        f(std::integral_constant<int, STREAM_PRO_NONE>{});
+    }
 }
 
 __device__ __forceinline__ float s_fma_h(_Float16 h, float x, float acc) { return __builtin_fmaf((float)h, x, acc); }
@@ -204,8 +294,8 @@ struct Q4Slot {
 };
 
 // P passes of 8 superblocks cover a row (n_blocks <= 8 * P); D rows in flight; MT tokens.
-template <int P, int NW, int D, int MT>
-__global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
+template <int P, int NW, int D, int MT, typename PT>
+__global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
 {
     stream_select_pair(p);
     const uint32_t lane = threadIdx.x & 63u;
@@ -222,36 +312,69 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
 
     float xlo[P][MT][16], xhi[P][MT][16], xs_lo[P][MT], xs_hi[P][MT];
     uint32_t hoff[P];
-    // (one branch around the whole prologue, so that either form issues its loads back to back)
-    auto load_x = [&](auto act) {
-        constexpr bool ACT = decltype(act)::value;
+    const uint32_t ldx = stream_ldx(p);
+    const ptrdiff_t x2_off = stream_x2_off(p);
+    auto load_x = [&](auto pro) {
+        constexpr int PRO = decltype(pro)::value;
 #pragma unroll
-    for (int pass = 0; pass < P; ++pass) {
-        uint32_t b = pass * 8u + bl;
-        const bool valid = b < p.n_blocks;
-        b = valid ? b : p.n_blocks - 1u;
-        hoff[pass] = b * KQ_Q4K_BYTES;
+        for (int pass = 0; pass < P; ++pass) {
+            uint32_t b = pass * 8u + bl;
+            const bool valid = b < p.n_blocks;
+            b = valid ? b : p.n_blocks - 1u;
+            hoff[pass] = b * KQ_Q4K_BYTES;
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            const float4* xp = (const float4*)(p.X + (size_t)t * p.K + (size_t)b * KQ_QK + 64u * g + 16u * h);
+            for (int t = 0; t < MT; ++t) {
+                const float4* xp = (const float4*)(p.X + (size_t)t * ldx + (size_t)b * KQ_QK + 64u * g + 16u * h);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float4 lo = stream_x4<ACT>(p, xp + i), hi = stream_x4<ACT>(p, xp + 8 + i);
-                if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
-                xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
-                xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
+                for (int i = 0; i < 4; ++i) {
+                    float4 lo = stream_x4<PRO, PT::kFused>(xp + i, x2_off), hi = stream_x4<PRO, PT::kFused>(xp + 8 + i, x2_off);
+                    if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
+                    xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
+                    xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
+                }
+                if constexpr (PRO != STREAM_PRO_NORM) {
+                    float sl = 0.0f, sh_ = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
+                    xs_lo[pass][t] = sl;
+                    xs_hi[pass][t] = sh_;
+                }
             }
-            float sl = 0.0f, sh_ = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
-            xs_lo[pass][t] = sl;
-            xs_hi[pass][t] = sh_;
         }
-    }
-
+        if constexpr (PRO == STREAM_PRO_NORM && PT::kFused) {
+            // the wave holds the whole row: its sum of squares is one reduction away
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                float ss = 0.0f;
+#pragma unroll
+                for (int pass = 0; pass < P; ++pass)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        ss = __builtin_fmaf(xlo[pass][t][i], xlo[pass][t][i], __builtin_fmaf(xhi[pass][t][i], xhi[pass][t][i], ss));
+                const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)p.K + stream_eps(p));
+#pragma unroll
+                for (int pass = 0; pass < P; ++pass) {
+                    const float* wp = stream_norm_w(p) + hoff[pass] / KQ_Q4K_BYTES * KQ_QK + 64u * g + 16u * h;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        xlo[pass][t][i] = xlo[pass][t][i] * rstd * wp[i];
+                        xhi[pass][t][i] = xhi[pass][t][i] * rstd * wp[32 + i];
+                    }
+                }
+            }
+#pragma unroll
+            for (int pass = 0; pass < P; ++pass)
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    float sl = 0.0f, sh_ = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
+                    xs_lo[pass][t] = sl;
+                    xs_hi[pass][t] = sh_;
+                }
+        }
     };
-    if (p.X2) load_x(std::true_type{});
-    else load_x(std::false_type{});
+    stream_dispatch_pro(p, load_x);
 
     // Ring of D rows in flight.  Slot d is refilled as soon as its row has been
     // consumed; the wait before a slot's arithmetic leaves the (D-1) younger
@@ -260,6 +383,8 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
     // no branch and the number of loads in flight is the same at every wait.
     constexpr int SLOT_LOADS = 2 * P;
     Q4Slot<P> ring[D] = {};
+    // (The ring is filled after the prologue even where that is long: registers with a load in flight
+    // must stay where they are, and across the prologue's arithmetic the compiler moves them.)
 #pragma unroll
     for (int d = 0; d < D; ++d)
         ring[d].fill(p.W + (size_t)(gw + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, hoff, j);
@@ -294,7 +419,12 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(StreamParams p)
             const uint32_t r = gw + (c0 + lane) * stride;
             const float bias = p.bias ? p.bias[r] : 0.0f;
 #pragma unroll
-            for (int t = 0; t < MT; ++t) p.Y[(size_t)t * p.ldy + p.y_offset + r] = res[t] + bias;
+            for (int t = 0; t < MT; ++t) {
+                const size_t at = (size_t)t * p.ldy + p.y_offset + r;
+                float y = res[t] + bias;
+                if constexpr (PT::kFused) y += stream_residual(p) ? stream_residual(p)[at] : 0.0f;
+                p.Y[at] = y;
+            }
         }
     }
     asm volatile("s_waitcnt vmcnt(0)");   // the ring's last refills land before the wave ends
@@ -408,8 +538,8 @@ __device__ __forceinline__ void q6k_piece_dot(const Q6Piece& v, const float (&x)
 
 // Workgroup = KW waves, one K slice of 8*P superblocks each; the workgroup walks
 // rows blockIdx.x, + gridDim.x, ...; D rows in flight per wave.
-template <int P, int KW, int D, int MT>
-__global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
+template <int P, int KW, int D, int MT, typename PT>
+__global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(PT p)
 {
     stream_select_pair(p);
     __shared__ float part[KW > 1 ? KW : 1][MT][64];
@@ -422,34 +552,87 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
 
     float x[P][MT][4][8], m32xs[P][MT][4];
     uint32_t boff[P];
-    auto load_x = [&](auto act) {
-        constexpr bool ACT = decltype(act)::value;
+    const uint32_t ldx = stream_ldx(p);
+    const ptrdiff_t x2_off = stream_x2_off(p);
+    auto load_x = [&](auto pro) {
+        constexpr int PRO = decltype(pro)::value;
 #pragma unroll
-    for (int pass = 0; pass < P; ++pass) {
-        uint32_t b = (wave * P + pass) * 8u + bl;
-        const bool valid = b < p.n_blocks;
-        b = valid ? b : p.n_blocks - 1u;
-        boff[pass] = b * KQ_Q6K_BYTES;
+        for (int pass = 0; pass < P; ++pass) {
+            uint32_t b = (wave * P + pass) * 8u + bl;
+            const bool valid = b < p.n_blocks;
+            b = valid ? b : p.n_blocks - 1u;
+            boff[pass] = b * KQ_Q6K_BYTES;
 #pragma unroll
-        for (int tk = 0; tk < MT; ++tk) {
-            const float4* xp = (const float4*)(p.X + (size_t)tk * p.K + (size_t)b * KQ_QK + 128u * n + 8u * lg);
+            for (int tk = 0; tk < MT; ++tk) {
+                const float4* xp = (const float4*)(p.X + (size_t)tk * ldx + (size_t)b * KQ_QK + 128u * n + 8u * lg);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                float4 lo = stream_x4<ACT>(p, xp + 8 * k), hi = stream_x4<ACT>(p, xp + 8 * k + 1);
-                if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
-                x[pass][tk][k][0] = lo.x; x[pass][tk][k][1] = lo.y; x[pass][tk][k][2] = lo.z; x[pass][tk][k][3] = lo.w;
-                x[pass][tk][k][4] = hi.x; x[pass][tk][k][5] = hi.y; x[pass][tk][k][6] = hi.z; x[pass][tk][k][7] = hi.w;
-                float sum = 0.0f;
+                for (int k = 0; k < 4; ++k) {
+                    float4 lo = stream_x4<PRO, PT::kFused>(xp + 8 * k, x2_off), hi = stream_x4<PRO, PT::kFused>(xp + 8 * k + 1, x2_off);
+                    if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
+                    x[pass][tk][k][0] = lo.x; x[pass][tk][k][1] = lo.y; x[pass][tk][k][2] = lo.z; x[pass][tk][k][3] = lo.w;
+                    x[pass][tk][k][4] = hi.x; x[pass][tk][k][5] = hi.y; x[pass][tk][k][6] = hi.z; x[pass][tk][k][7] = hi.w;
+                    if constexpr (PRO != STREAM_PRO_NORM) {
+                        float sum = 0.0f;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) sum += x[pass][tk][k][i];
-                m32xs[pass][tk][k] = -32.0f * sum;
+                        for (int i = 0; i < 8; ++i) sum += x[pass][tk][k][i];
+                        m32xs[pass][tk][k] = -32.0f * sum;
+                    }
+                }
             }
         }
-    }
-
+        if constexpr (PRO == STREAM_PRO_NORM && PT::kFused) {
+            // each wave holds a K slice: the slices' sums of squares meet in LDS
+#pragma unroll
+            for (int tk = 0; tk < MT; ++tk) {
+                float ss = 0.0f;
+#pragma unroll
+                for (int pass = 0; pass < P; ++pass)
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) ss = __builtin_fmaf(x[pass][tk][k][i], x[pass][tk][k][i], ss);
+                ss = wave_sum(ss);
+                if (KW > 1) {
+                    if (lane == 0) part[wave][tk][0] = ss;
+                    __syncthreads();
+                    ss = part[0][tk][0];
+#pragma unroll
+                    for (int w = 1; w < KW; ++w) ss += part[w][tk][0];
+                }
+                const float rstd = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
+#pragma unroll
+                for (int pass = 0; pass < P; ++pass) {
+                    const float* wp = stream_norm_w(p) + boff[pass] / KQ_Q6K_BYTES * KQ_QK + 128u * n + 8u * lg;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) x[pass][tk][k][i] = x[pass][tk][k][i] * rstd * wp[32 * k + i];
+                }
+            }
+            if (KW > 1) __syncthreads();   // part is reused by the row loop
+#pragma unroll
+            for (int pass = 0; pass < P; ++pass)
+#pragma unroll
+                for (int tk = 0; tk < MT; ++tk)
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        float sum = 0.0f;
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) sum += x[pass][tk][k][i];
+                        m32xs[pass][tk][k] = -32.0f * sum;
+                    }
+        }
     };
-    if (p.X2) load_x(std::true_type{});
-    else load_x(std::false_type{});
+    stream_dispatch_pro(p, load_x);
+    // The activations' sums are complete before the first weight request goes out: here, arithmetic on
+    // them that sank below the ring's fill waited for the weights as well and cost half a microsecond
+    // per launch (volatile statements keep their order, and this one makes the sums its operands).  The
+    // Q4_K kernel measured faster without such a pin.
+#pragma unroll
+    for (int pass = 0; pass < P; ++pass)
+#pragma unroll
+        for (int tk = 0; tk < MT; ++tk)
+            asm volatile("" : "+v"(m32xs[pass][tk][0]), "+v"(m32xs[pass][tk][1]), "+v"(m32xs[pass][tk][2]), "+v"(m32xs[pass][tk][3]));
 
     if (n_rows == 0) return;   // whole workgroup
     constexpr int SLOT_LOADS = 5 * P;
@@ -500,7 +683,10 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(StreamParams p)
 #pragma unroll
                     for (int w = 1; w < KW; ++w) y += part[w][tk][lane];
                 }
-                p.Y[(size_t)tk * p.ldy + p.y_offset + r] = y + bias;
+                const size_t at = (size_t)tk * p.ldy + p.y_offset + r;
+                y += bias;
+                if constexpr (PT::kFused) y += stream_residual(p) ? stream_residual(p)[at] : 0.0f;
+                p.Y[at] = y;
             }
         }
         if (KW > 1) __syncthreads();
@@ -535,33 +721,38 @@ bool gemv_stream_supported(const MatmulArgs& a)
     }
     if (a.type == KQ_TYPE_Q6_K) {
         if (a.n_blocks > 112) return false;
+        // the two-token kernel for the longest rows has no registers to spare for the fused forms
+        if (a.n_blocks > 56 && a.M == 2 && !a.expert_idx && (a.pro != 0 || a.residual)) return false;
         if (((uintptr_t)a.W & 1u) || (a.row_stride_bytes & 1u)) return false;
         return true;
     }
     return false;
 }
 
-hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStream_t s)
+// Launches of one instantiation.  Not every combination exists: grouped launches are one token per
+// pair, the fused forms run two rows in flight per wave whatever the depth option says, and the
+// two-token Q6_K kernel for the longest rows has no registers to spare for the fused forms
+// (gemv_stream_supported declines those calls).
+template <int P, int KW, int D, int MT, typename PT>
+static void launch_q6k_one(dim3 grid, hipStream_t s, const PT& p)
 {
-    StreamParams p;
-    p.X = (const float*)a.X;
-    p.W = a.W;
-    p.bias = a.bias;
-    p.Y = a.Y;
-    p.N = a.N; p.K = a.K;
-    p.n_blocks = a.n_blocks;
-    p.row_stride_bytes = a.row_stride_bytes;
-    p.y_offset = a.y_offset;
-    p.expert_idx = a.expert_idx;
-    p.k_slots = a.k_slots;
-    p.ldy = a.ldy;
-    p.x_per_slot = a.x_per_slot;
-    p.W2 = a.expert_idx ? a.W2 : nullptr;
-    p.Y2 = a.Y2;
-    p.X2 = a.expert_idx ? a.X2 : nullptr;
-    const uint32_t twins = p.W2 ? 2u : 1u;            // grid.z
-    const uint32_t pairs = a.expert_idx ? a.M : 1u;   // grid.y
-    const bool two = !a.expert_idx && a.M == 2;       // two tokens share every weight load
+    constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && (D != 2 || (P == 2 && KW == 7 && MT == 2)));
+    if constexpr (!absent) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, D, MT, PT>), grid, dim3(64 * KW), 0, s, p);
+}
+
+template <int P, int NW, int D, int MT, typename PT>
+static void launch_q4k_one(dim3 grid, hipStream_t s, const PT& p)
+{
+    constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && D != 2);
+    if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT>), grid, dim3(64 * NW), 0, s, p);
+}
+
+template <typename PT>
+static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, hipStream_t s, const PT& p,
+                                     uint32_t pairs, uint32_t twins)
+{
+    const bool two = !PT::kGrouped && a.M == 2;       // two tokens share every weight load
+    const dim3 grid_yz(1, pairs, twins);
     // Measured on MI355X: these kernels run best with about 40 KB of weight loads
     // in flight per CU: 4 to 8 waves, two to four rows in flight each.  More waves
     // or deeper rings are slower.
@@ -572,12 +763,13 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
         const int pp = nb <= 8u ? 1 : nb <= 16u ? 2 : nb <= 56u ? 1 : 2;
         uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 8u / (uint32_t)kw, t.splits);
         wgs = (wgs + pairs * twins - 1u) / (pairs * twins);   // the pairs of a grouped launch share the machine
-        const int depth = t.depth > 0 ? t.depth : 2;
+        const int depth = PT::kFused ? 2 : t.depth > 0 ? t.depth : 2;
+        const dim3 grid(wgs, pairs, twins);
 #define KQ_STREAM6_MT(P, KW, MT) \
     do { \
-        if (depth <= 1) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 1, MT>), dim3(wgs, pairs, twins), dim3(64 * KW), 0, s, p); \
-        else if (depth <= 2) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 2, MT>), dim3(wgs, pairs, twins), dim3(64 * KW), 0, s, p); \
-        else hipLaunchKernelGGL((q6k_stream_kernel<P, KW, 4, MT>), dim3(wgs, pairs, twins), dim3(64 * KW), 0, s, p); \
+        if (depth <= 1) launch_q6k_one<P, KW, 1, MT>(grid, s, p); \
+        else if (depth <= 2) launch_q6k_one<P, KW, 2, MT>(grid, s, p); \
+        else launch_q6k_one<P, KW, 4, MT>(grid, s, p); \
     } while (0)
 #define KQ_STREAM6(P, KW) \
     do { \
@@ -598,11 +790,12 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     uint32_t wgs = t.splits > 0 ? ((a.N + (uint32_t)t.splits - 1u) / (uint32_t)t.splits + NW - 1u) / NW
                                 : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
     wgs = (wgs + pairs * twins - 1u) / (pairs * twins);
-    const int depth = t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
+    const int depth = PT::kFused ? 2 : t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
+    const dim3 grid(wgs, pairs, twins);
 #define KQ_STREAM_LAUNCH(P, D) \
     do { \
-        if (two) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, 2>), dim3(wgs, pairs, twins), dim3(64 * NW), 0, s, p); \
-        else hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, 1>), dim3(wgs, pairs, twins), dim3(64 * NW), 0, s, p); \
+        if (two) launch_q4k_one<P, NW, D, 2>(grid, s, p); \
+        else launch_q4k_one<P, NW, D, 1>(grid, s, p); \
     } while (0)
     if (a.n_blocks <= 8u) {
         if (depth <= 1) KQ_STREAM_LAUNCH(1, 1);
@@ -615,6 +808,47 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
     }
 #undef KQ_STREAM_LAUNCH
     return hipGetLastError();
+}
+
+template <typename PT>
+static void stream_fill_common(PT& p, const MatmulArgs& a)
+{
+    p.X = (const float*)a.X;
+    p.W = a.W;
+    p.bias = a.bias;
+    p.Y = a.Y;
+    p.N = a.N; p.K = a.K;
+    p.n_blocks = a.n_blocks;
+    p.row_stride_bytes = a.row_stride_bytes;
+    p.y_offset = a.y_offset;
+    p.ldy = a.ldy;
+}
+
+hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStream_t s)
+{
+    if (a.expert_idx) {
+        StreamGrouped p;
+        stream_fill_common(p, a);
+        p.expert_idx = a.expert_idx;
+        p.k_slots = a.k_slots;
+        p.x_per_slot = a.x_per_slot;
+        p.W2 = a.W2;
+        p.Y2 = a.Y2;
+        p.X2 = a.X2;
+        return launch_stream_with(a, t, s, p, a.M, p.W2 ? 2u : 1u);   // grid.y = pairs, grid.z = twins
+    }
+    if (a.pro != STREAM_PRO_NONE || a.residual) {
+        StreamFused p;
+        stream_fill_common(p, a);
+        p.pro = a.pro;
+        p.eps = a.eps;
+        p.norm_w = a.norm_w;
+        p.residual = a.residual;
+        return launch_stream_with(a, t, s, p, 1u, 1u);
+    }
+    StreamDense p;
+    stream_fill_common(p, a);
+    return launch_stream_with(a, t, s, p, 1u, 1u);
 }
 
 }  // namespace kq

@@ -54,6 +54,8 @@ def parse():
     ap.add_argument("--moe", action="store_true",
                     help="also time the Qwen3-30B-A3B-shaped routed-expert FFN at T = 1 and T = 256")
     ap.add_argument("--all", action="store_true", help="--prefill --verify --moe")
+    ap.add_argument("--fused", action="store_true",
+                    help="also time the layer set with RMSNorm folded into qkv and act*mul + residual into down")
     ap.add_argument("--load", action="store_true",
                     help="also write a GGUF file of Q4_K / Q6_K matrices and time file -> device weights")
     ap.add_argument("--gemm-tile", type=int, default=0,
@@ -277,6 +279,8 @@ def main():
         out["verify"] = verify_leg(mats, wb, use_graph)
     if args.moe or args.all:
         out["moe"] = moe_leg()
+    if args.fused or args.all:
+        out["fused"] = fused_leg(mats, use_graph)
     if args.load:
         out["gguf_load"] = load_leg()
     if not args.no_prefill:
@@ -290,6 +294,65 @@ def main():
         torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
+
+
+def fused_leg(mats, use_graph):
+    """The decode layer set with what surrounds two of its matvecs folded in: qkv reads x through RMSNorm,
+    down reads silu(gate)*up from the gate|up output and adds the residual in place.  Timed three ways on
+    the same weights: plain matvecs only (what the headline measures), fused (one launch each), and the
+    same function as separate launches (norm, act*mul, add beside the matvecs)."""
+    import torch
+    from backpack_amd import capi, kquant
+    hidden = next(w.K for n, w, _, _ in mats if n == "qkv")
+    inter = next(w.K for n, w, _, _ in mats if n == "down")
+    norm_w = torch.ones(hidden, device="cuda")
+    gate_up = next(y for n, _, _, y in mats if n == "gate_up")
+    resid = torch.zeros(1, hidden, device="cuda")
+    ws = torch.empty(capi.lib().bpk_kq_matmul_fused_workspace_bytes(1, max(w.N for _, w, _, _ in mats), inter),
+                     dtype=torch.uint8, device="cuda")
+
+    def fused_pass():
+        for name, w, x, y in mats:
+            if name == "qkv":
+                kquant.matmul_fused(x, w, capi.PRO_RMS_NORM, norm_w=norm_w, eps=1e-5, out=y, workspace=ws)
+            elif name == "down":
+                kquant.matmul_fused(gate_up, w, capi.PRO_SILU_MUL, residual=resid, out=resid, workspace=ws)
+            else:
+                kquant.matmul(x, w, out=y)
+
+    def timed(one_pass, steps=20, warmup=3):
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            one_pass()
+            stream.synchronize()
+            step = one_pass
+            if use_graph:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=stream):
+                    one_pass()
+                step = graph.replay
+            for _ in range(warmup):
+                step()
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(steps):
+                step()
+            e1.record(stream)
+            stream.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    res = {"plain_ms": round(timed(lambda: [kquant.matmul(x, w, out=y) for _, w, x, y in mats]), 4)}
+    res["fused_ms"] = round(timed(fused_pass), 4)
+    res["kernel"] = capi.last_kernel()
+    capi.set_option("fused_separate", 1)
+    try:
+        res["separate_ms"] = round(timed(fused_pass), 4)
+    finally:
+        capi.set_option("fused_separate", 0)
+    n = sum(1 for name, *_ in mats if name in ("qkv", "down"))
+    res["launches_saved"] = int(n * 1.5)     # norm per qkv; act*mul and add per down
+    return res
 
 
 def load_leg(n_layers=8):

@@ -196,6 +196,49 @@ BPK_API int bpk_kq_matmul(int type, const float *X, const void *W,
                           uint32_t row_stride_words, uint32_t y_offset,
                           void *stream);
 
+/* ---- fused decode forms: replace the dispatches either side of the matvec ----
+ * What the reference wrote as q4k_matmul_norm / q6k_matmul_norm
+ * (runtime/kernels/quant_kq/q4k_matmul_norm.wgsl:50-91: RMSNorm of the X row
+ * inside the matvec, bindings 5:NormW 6:{K,0,0,eps}) and q4k_down_gelu /
+ * q6k_down_gelu (quant_kq/q4k_down_gelu.wgsl:11-56: binding 0 is the fused
+ * gate|up buffer), and the dispatches it still issues separately: rms_norm
+ * (kernels/norm/rms_norm.wgsl:15-20), silu_mul_fused / gelu_mul_fused
+ * (kernels/fused/silu_mul_fused.wgsl:39-49, gelu_mul_fused.wgsl:22-32) before
+ * down, add_inplace after it (runtime/model_runner.cpp:3748-3793).
+ *
+ *   x[m,k] = X[m,k]                                              BPK_PRO_NONE
+ *          = X[m,k] * rsqrt(mean_k(X[m,:]^2) + eps) * norm_w[k]  BPK_PRO_RMS_NORM
+ *          = silu(X[m,k]) * X[m,K+k],  X rows are 2K floats      BPK_PRO_SILU_MUL
+ *          = gelu_tanh(X[m,k]) * X[m,K+k]                        BPK_PRO_GELU_MUL
+ *   Y[m*N + y_offset + n] = bias[n] + residual[m*N + y_offset + n]
+ *                           + sum_k x[m,k] * dequant(W)[n,k]
+ *
+ * silu(g) = g / (1 + exp(-g)); gelu_tanh(g) = 0.5 g (1 + tanh(0.7978845608 (g +
+ * 0.044715 g^3))).  residual may be NULL (= zeros) and may be Y itself (the
+ * in-place add).  M <= 2 with rows the decode kernel holds in registers
+ * (Q4_K: K <= 4096; Q6_K: K <= 28672 for one token, K <= 14336 for two;
+ * N <= 32768) is one launch and needs no workspace.  Other shapes run the same function as prologue, matmul and add
+ * launches through `workspace` (device memory, 16-byte aligned, at least
+ * bpk_kq_matmul_fused_workspace_bytes(M, N, K) bytes) and fail with
+ * BPK_ERR_WORKSPACE without it. */
+enum { BPK_PRO_NONE = 0, BPK_PRO_RMS_NORM = 1, BPK_PRO_SILU_MUL = 2, BPK_PRO_GELU_MUL = 3 };
+
+typedef struct bpk_kq_fusion {
+    int prologue;          /* BPK_PRO_*                               */
+    const float *norm_w;   /* f32 [K] (device), BPK_PRO_RMS_NORM only */
+    float eps;             /* BPK_PRO_RMS_NORM only                   */
+    const float *residual; /* f32 (device), indexed like Y, or NULL   */
+} bpk_kq_fusion;
+
+BPK_API size_t bpk_kq_matmul_fused_workspace_bytes(uint32_t M, uint32_t N,
+                                                   uint32_t K);
+BPK_API int bpk_kq_matmul_fused(int type, const float *X, const void *W,
+                                const float *bias, float *Y, uint32_t M,
+                                uint32_t N, uint32_t K, uint32_t n_blocks,
+                                uint32_t row_stride_words, uint32_t y_offset,
+                                const bpk_kq_fusion *fusion, void *workspace,
+                                size_t workspace_bytes, void *stream);
+
 /* Prefill form: X is bf16 [M,K] (raw 16-bit patterns), Y f32 [M,N].  Weight
  * tiles are dequantised to bf16 in LDS and contracted on the matrix cores
  * with fp32 accumulation.  The reference has no such kernel: its k-quant
@@ -272,7 +315,9 @@ BPK_API int bpk_force_kernel(int family);
  * GEMM (128 or 256); "gemm_split": how the 256-tile GEMM hands out work
  * (1 = one tile per workgroup, 2 = the walk over tiles and k steps cut into
  * equal shares per compute unit, tiles cut between workgroups are summed with
- * fp32 atomics).  0 = automatic. */
+ * fp32 atomics); "fused_separate": 1 makes bpk_kq_matmul_fused run its prologue,
+ * matmul and add as separate launches for every shape (needs the workspace).
+ * 0 = automatic. */
 BPK_API int bpk_set_option(const char *name, int value);
 
 #ifdef __cplusplus

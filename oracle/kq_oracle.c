@@ -228,6 +228,35 @@ int kqo_matmul(int type, const float *X, const uint32_t *packed, const float *bi
     return 0;
 }
 
+int kqo_prologue(int pro, const float *X, const float *norm_w, float eps,
+                 uint32_t M, uint32_t K, float *out)
+{
+    if (pro < 1 || pro > 3) return -1;
+    for (uint32_t m = 0; m < M; ++m) {
+        float *o = out + (size_t)m * K;
+        if (pro == 1) {
+            const float *x = X + (size_t)m * K;
+            float ss = 0.0f;
+            for (uint32_t k = 0; k < K; ++k) ss += x[k] * x[k];
+            const float rstd = 1.0f / sqrtf(ss / (float)K + eps);
+            for (uint32_t k = 0; k < K; ++k) o[k] = x[k] * rstd * norm_w[k];
+        } else {
+            const float *g = X + (size_t)m * 2u * K, *u = g + K;
+            for (uint32_t k = 0; k < K; ++k) {
+                float a;
+                if (pro == 2) {
+                    a = g[k] / (expf(0.0f - g[k]) + 1.0f);
+                } else {
+                    const float inner = 0.7978845608f * (g[k] + 0.044715f * g[k] * g[k] * g[k]);
+                    a = 0.5f * g[k] * (1.0f + tanhf(inner));
+                }
+                o[k] = a * u[k];
+            }
+        }
+    }
+    return 0;
+}
+
 int kqo_matmul_f64(int type, const float *X, const uint32_t *packed,
                    const float *bias, double *Y, uint32_t M, uint32_t N,
                    uint32_t K, uint32_t row_stride_words)

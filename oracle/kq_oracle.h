@@ -106,6 +106,19 @@ int kqo_matmul(int type, const float *X, const uint32_t *packed, const float *bi
                float *Y, uint32_t M, uint32_t N, uint32_t K,
                uint32_t row_stride_words, uint32_t y_offset, uint32_t ldy);
 
+/* What the fused decode forms apply to X before the contraction
+ * (pro 1: runtime/kernels/norm/rms_norm.wgsl:15-20 and
+ * quant_kq/q4k_matmul_norm.wgsl:50-91, x * rstd * w with
+ * rstd = 1/sqrt(sum(x^2)/K + eps), the squares summed in k order;
+ * pro 2: kernels/fused/silu_mul_fused.wgsl:39-49, g/(exp(-g)+1) * u;
+ * pro 3: kernels/fused/gelu_mul_fused.wgsl:22-32, the tanh form).  For pro 2/3
+ * the rows of X are gate | up, 2K floats.  out: M x K.  The reference holds no
+ * test of these kernels: the restatement is pinned on closed forms in fp64
+ * (tests/test_oracle_pins.py), the composition with the matmul is unpinned
+ * beyond that. */
+int kqo_prologue(int pro, const float *X, const float *norm_w, float eps,
+                 uint32_t M, uint32_t K, float *out);
+
 /* Same contraction in fp64 with no bias rounding: the ground truth that both
  * fp32 summation orders are compared with. */
 int kqo_matmul_f64(int type, const float *X, const uint32_t *packed,

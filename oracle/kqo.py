@@ -54,6 +54,7 @@ def _load() -> C.CDLL:
                                      C.c_uint32, _f32p]
     lib.kqo_matmul.argtypes = [C.c_int, _f32p, _u32p, _f32p, _f32p, C.c_uint32,
                                C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32]
+    lib.kqo_prologue.argtypes = [C.c_int, _f32p, _f32p, C.c_float, C.c_uint32, C.c_uint32, _f32p]
     lib.kqo_matmul_f64.argtypes = [C.c_int, _f32p, _u32p, _f32p, _f64p, C.c_uint32,
                                    C.c_uint32, C.c_uint32, C.c_uint32]
     lib.kqo_matmul_bf16.argtypes = [C.c_int, _u16p, _u32p, _f32p, _f32p, C.c_uint32,
@@ -177,6 +178,17 @@ def matmul(type_: int, X, packed, N: int, K: int, bias=None, y_offset: int = 0,
                           row_stride_words(type_, K), y_offset, ldy)
     assert rc == 0
     return Y
+
+
+def prologue(pro: int, X, K: int, norm_w=None, eps: float = 0.0) -> np.ndarray:
+    """RMSNorm (1) / silu(gate)*up (2) / gelu_tanh(gate)*up (3) of the rows of X; gate | up rows are 2K wide."""
+    X = _c(X, np.float32)
+    M = X.size // (K if pro == 1 else 2 * K)
+    out = np.empty((M, K), dtype=np.float32)
+    w = _c(norm_w, np.float32) if norm_w is not None else np.zeros(1, np.float32)
+    rc = lib().kqo_prologue(pro, _p(X, _f32p), _p(w, _f32p), eps, M, K, _p(out, _f32p))
+    assert rc == 0
+    return out
 
 
 def matmul_f64(type_: int, X, packed, N: int, K: int, bias=None) -> np.ndarray:

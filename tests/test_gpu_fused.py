@@ -1,0 +1,134 @@
+"""Fused decode forms (bpk_kq_matmul_fused) against the oracle: the prologue the reference's
+q4k_matmul_norm / q4k_down_gelu kernels apply, composed with the oracle matmul and the residual add.
+One-launch shapes and the workspace path must compute the same function."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+Q4_K, Q6_K = 12, 14
+NONE, NORM, SILU, GELU = range(4)
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from backpack_amd import capi
+    capi.check(capi.lib().bpk_init(0))
+    import gpu_util
+    return gpu_util
+
+
+def _case(gpu, kqo, type_, M, N, K, pro, with_res, with_bias, seed):
+    rng = np.random.default_rng(seed)
+    raw, packed, w = gpu.make_weight(type_, N, K, seed=seed)
+    X = (rng.standard_normal((M, K if pro in (NONE, NORM) else 2 * K)) * 1.5).astype(np.float32)
+    norm_w = (1 + 0.1 * rng.standard_normal(K)).astype(np.float32) if pro == NORM else None
+    res = rng.standard_normal((M, N)).astype(np.float32) if with_res else None
+    bias = rng.standard_normal(N).astype(np.float32) if with_bias else None
+    xp = X if pro == NONE else kqo.prologue(pro, X, K, norm_w=norm_w, eps=1e-5)
+    return w, packed, X, norm_w, res, bias, xp
+
+
+def _check(gpu, kqo, type_, got, xp, packed, N, K, res, bias, label):
+    # the residual enters after the contraction: compare got - residual with the oracle matmul of x'.
+    # slack 1e-5: exp / tanh / rsqrt come from a different libm than the oracle's, which moves x' by
+    # an ulp or two before the contraction.
+    got = np.asarray(got, dtype=np.float64).reshape(-1, N)
+    if res is not None:
+        got = got - res.astype(np.float64)
+    gpu.check_matmul(kqo, type_, got.astype(np.float32), xp, packed, N, K, bias=bias, label=label, slack=1e-5)
+
+
+ONE_LAUNCH = [
+    # type, M, N, K, prologue, residual, bias
+    (Q4_K, 1, 384, 4096, NORM, False, False),     # norm -> qkv
+    (Q4_K, 2, 200, 2048, NORM, True, True),
+    (Q4_K, 1, 130, 1024, SILU, True, False),
+    (Q4_K, 2, 96, 4096, GELU, True, False),
+    (Q4_K, 1, 64, 512, NONE, True, True),         # residual only
+    (Q6_K, 1, 256, 14336, SILU, True, False),     # act -> down -> residual, the decode FFN tail
+    (Q6_K, 2, 100, 14336, SILU, True, False),
+    (Q6_K, 1, 77, 4096, NORM, False, True),
+    (Q6_K, 2, 64, 7168, NORM, True, False),       # norm across K slices of several waves
+    (Q6_K, 1, 50, 28672, GELU, False, False),
+    (Q6_K, 2, 40, 2048, GELU, True, True),
+    (Q6_K, 1, 33, 768, NORM, True, False),
+]
+
+
+@pytest.mark.parametrize("type_,M,N,K,pro,with_res,with_bias", ONE_LAUNCH)
+def test_fused_one_launch(gpu, kqo, type_, M, N, K, pro, with_res, with_bias):
+    from backpack_amd import capi, kquant
+    print("fused", type_, M, N, K, pro, with_res, with_bias, flush=True)
+    w, packed, X, norm_w, res, bias, xp = _case(gpu, kqo, type_, M, N, K, pro, with_res, with_bias, seed=N + K)
+    y = kquant.matmul_fused(gpu.dev(X), w, pro, norm_w=gpu.dev(norm_w) if norm_w is not None else None, eps=1e-5,
+                            residual=gpu.dev(res) if res is not None else None,
+                            bias=gpu.dev(bias) if bias is not None else None, allow_workspace=False)
+    assert capi.last_kernel() == "gemv_stream_fused"
+    _check(gpu, kqo, type_, y.cpu().numpy(), xp, packed, N, K, res, bias, f"fused {type_} {M}x{N}x{K} pro={pro}")
+
+
+def test_fused_residual_in_place_and_same_as_separate_launches(gpu, kqo):
+    """x += down(silu(gate) * up): the residual is the output buffer; and the one-launch result equals the
+    three-launch result of the workspace path on the same inputs to fp32 summation-order accuracy."""
+    import torch
+    from backpack_amd import capi, kquant
+    N, K = 512, 14336
+    w, packed, X, _, res, _, xp = _case(gpu, kqo, Q6_K, 1, N, K, SILU, True, False, seed=5)
+    y = gpu.dev(res.copy())
+    kquant.matmul_fused(gpu.dev(X), w, SILU, residual=y, out=y, allow_workspace=False)
+    _check(gpu, kqo, Q6_K, y.cpu().numpy(), xp, packed, N, K, res, None, "in-place residual")
+    capi.set_option("fused_separate", 1)      # prologue, matmul and add launches
+    try:
+        y2 = gpu.dev(res.copy())
+        kquant.matmul_fused(gpu.dev(X), w, SILU, residual=y2, out=y2)
+        assert capi.last_kernel() == "gemv_stream"
+    finally:
+        capi.set_option("fused_separate", 0)
+    _check(gpu, kqo, Q6_K, y2.cpu().numpy(), xp, packed, N, K, res, None, "in-place residual, workspace path")
+    scale = float(np.sqrt(np.mean((y.cpu().numpy() - res) ** 2)))
+    assert float((y - y2).abs().max()) <= 2e-5 * scale
+
+
+WORKSPACE = [
+    (Q4_K, 1, 100, 14336, SILU, True),     # Q4_K rows longer than the decode kernel's registers
+    (Q4_K, 5, 96, 2048, NORM, True),       # more than two tokens
+    (Q6_K, 16, 64, 1024, GELU, False),
+    (Q6_K, 2, 48, 28672, NORM, True),      # the two-token long-row kernel carries no norm
+    (Q4_K, 3, 40, 512, NONE, True),
+]
+
+
+@pytest.mark.parametrize("type_,M,N,K,pro,with_res", WORKSPACE)
+def test_fused_workspace_path(gpu, kqo, type_, M, N, K, pro, with_res):
+    from backpack_amd import capi, kquant
+    print("fused ws", type_, M, N, K, pro, with_res, flush=True)
+    w, packed, X, norm_w, res, bias, xp = _case(gpu, kqo, type_, M, N, K, pro, with_res, False, seed=M + K)
+    args = dict(norm_w=gpu.dev(norm_w) if norm_w is not None else None, eps=1e-5,
+                residual=gpu.dev(res) if res is not None else None)
+    with pytest.raises(capi.BpkError) as e:
+        kquant.matmul_fused(gpu.dev(X), w, pro, allow_workspace=False, **args)
+    assert e.value.code == -7
+    y = kquant.matmul_fused(gpu.dev(X), w, pro, **args)
+    assert capi.last_kernel() != "gemv_stream_fused"
+    _check(gpu, kqo, type_, y.cpu().numpy(), xp, packed, N, K, res, None, f"fused ws {type_} {M}x{N}x{K}")
+
+
+def test_fused_argument_checks(gpu):
+    import ctypes as C
+    from backpack_amd import capi, kquant
+    raw, packed, w = gpu.make_weight(Q4_K, 8, 256, seed=1)
+    x = gpu.dev(np.zeros((1, 256), np.float32))
+    y = gpu.dev(np.zeros((1, 8), np.float32))
+    L = capi.lib()
+
+    def call(f):
+        return L.bpk_kq_matmul_fused(Q4_K, x.data_ptr(), w.data.data_ptr(), None, y.data_ptr(), 1, 8, 256, 1, 36, 0,
+                                     f, None, 0, None)
+    assert call(None) == -3
+    assert call(C.byref(capi.Fusion(7, None, 0.0, None))) == -2
+    assert call(C.byref(capi.Fusion(capi.PRO_RMS_NORM, None, 1e-5, None))) == -3
+    assert call(C.byref(capi.Fusion(capi.PRO_NONE, None, 0.0, None))) == 0     # plain matmul
+    assert L.bpk_kq_matmul_fused_workspace_bytes(3, 10, 256) == 3 * 256 * 4 + 3 * 10 * 4

@@ -290,3 +290,35 @@ def test_moe_ffn_composition(kqo):
     y = kqo.moe_matmul(Q6_K, act.reshape(T * k, I), down, eidx, H, I, x_per_slot=True)
     want = (ew[..., None].astype(np.float64) * y).sum(axis=1)
     assert np.allclose(out, want, rtol=2e-4, atol=2e-4 * np.abs(want).max())
+
+
+# ---- prologues of the fused decode forms -----------------------------------------
+def test_prologues_against_closed_forms_in_float64(kqo):
+    """RMSNorm, silu*up and gelu_tanh*up against their definitions evaluated in float64 by numpy:
+    a dropped eps, a mean over the wrong length, gate and up swapped, a wrong constant or sign in
+    the gelu would each move the result by far more than the float32 rounding allowed here."""
+    rng = np.random.default_rng(11)
+    M, K = 3, 768
+    x = (rng.standard_normal((M, K)) * 3).astype(np.float32)
+    w = (1 + 0.2 * rng.standard_normal(K)).astype(np.float32)
+    for eps in (1e-6, 0.5):
+        got = kqo.prologue(1, x, K, norm_w=w, eps=eps)
+        x64 = x.astype(np.float64)
+        want = x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + eps) * w
+        assert np.abs(got - want).max() <= 4e-7 * np.abs(want).max()
+    # rows are independent and the norm is scale-free up to eps
+    assert np.array_equal(kqo.prologue(1, x[1:2], K, norm_w=w, eps=1e-6), kqo.prologue(1, x, K, norm_w=w, eps=1e-6)[1:2])
+    a = kqo.prologue(1, x, K, norm_w=w, eps=0.0)
+    b = kqo.prologue(1, 4.0 * x, K, norm_w=w, eps=0.0)
+    assert np.abs(a - b).max() <= 4e-7 * np.abs(a).max()
+    gu = (rng.standard_normal((M, 2 * K)) * 4).astype(np.float32)
+    g, u = gu[:, :K].astype(np.float64), gu[:, K:].astype(np.float64)
+    silu = kqo.prologue(2, gu, K)
+    assert np.abs(silu - g / (1 + np.exp(-g)) * u).max() <= 1e-6 * np.abs(u).max() * 4
+    gelu = kqo.prologue(3, gu, K)
+    want = 0.5 * g * (1 + np.tanh(np.sqrt(2 / np.pi) * (g + 0.044715 * g ** 3))) * u
+    assert np.abs(gelu - want).max() <= 2e-6 * np.abs(u).max() * 4
+    # special values: silu(0) = gelu(0) = 0; large positive gate passes up through, large negative kills it
+    edge = np.array([[0.0, 30.0, -30.0, 1.0, 2.0, 3.0]], dtype=np.float32)
+    assert kqo.prologue(2, edge, 3).tolist() == [[0.0, 60.0, -0.0]] or np.allclose(kqo.prologue(2, edge, 3), [[0, 60, 0]], atol=1e-10)
+    assert np.allclose(kqo.prologue(3, edge, 3), [[0, 60, 0]], atol=1e-10)
