@@ -70,6 +70,7 @@ struct DeviceState {
     bool ready = false;
     kq::SplitScratch split{};
     uint32_t* moe_tiles = nullptr;   // kMoeWords words
+    float* route_logits = nullptr;   // ROUTE_SPREAD_TOKENS x 1024 router logits of a small-T route call
     UploadStage up{};                // created by the first upload on the device
 };
 
@@ -95,6 +96,7 @@ int ensure_device(int device, DeviceState** out)
         if (e == hipSuccess) e = hipMalloc((void**)&st.split.counters, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMemset(st.split.counters, 0, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMalloc((void**)&st.moe_tiles, kMoeWords * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipMalloc((void**)&st.route_logits, kq::ROUTE_SPREAD_TOKENS * 1024u * sizeof(float));
         if (cur != device && cur >= 0) (void)hipSetDevice(cur);
         if (e != hipSuccess) return hip_fail(e, "allocating split-K scratch");
         st.split.capacity_floats = kPartialFloats;
@@ -197,6 +199,7 @@ int bpk_shutdown(void)
         (void)hipFree(st.split.partial);
         (void)hipFree(st.split.counters);
         (void)hipFree(st.moe_tiles);
+        (void)hipFree(st.route_logits);
         for (int b = 0; b < 2; ++b) {
             if (st.up.buf[b]) (void)hipHostFree(st.up.buf[b]);
             if (st.up.sent[b]) (void)hipEventDestroy(st.up.sent[b]);
@@ -567,6 +570,44 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
         t_kernel = "generic_indirect";
         e = kq::launch_matmul_generic(a, s);
     }
+    return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+static int check_route(uint32_t T, uint32_t n_experts, uint32_t k, const void* idx, const void* wt)
+{
+    if (!idx || !wt) return fail(BPK_ERR_NULL, "idx and wt must be non-null");
+    if (n_experts == 0 || n_experts > 1024u) return fail(BPK_ERR_SHAPE, "n_experts=%u out of range (1..1024)", n_experts);
+    if (k == 0 || k > 16u || k > n_experts) return fail(BPK_ERR_SHAPE, "k=%u out of range (1..min(16, n_experts))", k);
+    if ((uint64_t)T * n_experts > 0xFFFFFFFFull) return fail(BPK_ERR_SHAPE, "T * n_experts too large");
+    return BPK_OK;
+}
+
+int bpk_moe_topk_softmax(const float* logits, uint32_t T, uint32_t n_experts, uint32_t k, int normalize,
+                         uint32_t* idx, float* wt, void* stream)
+{
+    if (!logits) return fail(BPK_ERR_NULL, "logits must be non-null");
+    if (int rc = check_route(T, n_experts, k, idx, wt)) return rc;
+    if (T == 0) return BPK_OK;
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
+    t_kernel = "moe_topk_softmax";
+    const hipError_t e = kq::launch_topk_softmax(logits, T, n_experts, k, normalize, idx, wt, (hipStream_t)stream);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+int bpk_moe_route(const float* X, const float* router_w, uint32_t T, uint32_t hidden, uint32_t n_experts, uint32_t k,
+                  int normalize, float* logits, uint32_t* idx, float* wt, void* stream)
+{
+    if (!X || !router_w) return fail(BPK_ERR_NULL, "X and router_w must be non-null");
+    if (int rc = check_route(T, n_experts, k, idx, wt)) return rc;
+    if (hidden == 0 || hidden % 4u) return fail(BPK_ERR_SHAPE, "hidden=%u is not a positive multiple of 4", hidden);
+    if (((uintptr_t)X | (uintptr_t)router_w) & 15u) return fail(BPK_ERR_ALIGN, "X and router_w must be 16-byte aligned");
+    if (T == 0) return BPK_OK;
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
+    t_kernel = "moe_route";
+    const hipError_t e = kq::launch_route(X, router_w, T, hidden, n_experts, k, normalize, logits, st->route_logits,
+                                          idx, wt, (hipStream_t)stream);
     return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
 }
 

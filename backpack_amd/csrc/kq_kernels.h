@@ -55,6 +55,15 @@ hipError_t launch_prologue_rows(int pro, const float* X, const float* norm_w, fl
 hipError_t launch_add_residual(const float* T, const float* R, float* Y, uint32_t M, uint32_t N, uint32_t ldy,
                                uint32_t y_offset, hipStream_t s);
 
+// MoE router stage: per token the k largest of n_experts logits (iterated argmax, lowest index on ties)
+// and the softmax over them; and the same behind an fp32 router matvec.  n_experts <= 1024, k <= 16.
+hipError_t launch_topk_softmax(const float* logits, uint32_t T, uint32_t n_experts, uint32_t k, int normalize,
+                               uint32_t* idx, float* wt, hipStream_t s);
+constexpr uint32_t ROUTE_SPREAD_TOKENS = 64;   // fewer tokens: experts spread over workgroups, two launches
+hipError_t launch_route(const float* X, const float* router_w, uint32_t T, uint32_t hidden, uint32_t n_experts,
+                        uint32_t k, int normalize, float* logits_out, float* logits_scratch, uint32_t* idx, float* wt,
+                        hipStream_t s);
+
 // Any shape with K % 256 == 0, any 4-byte aligned W.  M tiled by 4 inside.
 hipError_t launch_matmul_generic(const MatmulArgs& a, hipStream_t s);
 

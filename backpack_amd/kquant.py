@@ -180,6 +180,29 @@ def moe_matmul(x: torch.Tensor, w: KQuantPacked, expert_idx: torch.Tensor, n_exp
     return out
 
 
+def moe_topk_softmax(logits: torch.Tensor, k: int, normalize: bool = True):
+    """Router selection per token: (idx int32 [T,k], wt f32 [T,k]) from logits f32 [T, n_experts]."""
+    assert logits.is_cuda and logits.is_contiguous() and logits.dtype == torch.float32
+    T, E = logits.shape
+    idx = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    wt = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+    capi.check(capi.lib().bpk_moe_topk_softmax(_ptr(logits), T, E, k, int(normalize), _ptr(idx), _ptr(wt), _stream()))
+    return idx, wt
+
+
+def moe_route(x: torch.Tensor, router_w: torch.Tensor, k: int, normalize: bool = True, want_logits: bool = False):
+    """Router matvec (fp32 [n_experts, hidden]) and selection in one launch."""
+    assert x.is_contiguous() and router_w.is_contiguous() and x.dtype == router_w.dtype == torch.float32
+    T, H = x.shape
+    E = router_w.shape[0]
+    idx = torch.empty((T, k), dtype=torch.int32, device=x.device)
+    wt = torch.empty((T, k), dtype=torch.float32, device=x.device)
+    logits = torch.empty((T, E), dtype=torch.float32, device=x.device) if want_logits else None
+    capi.check(capi.lib().bpk_moe_route(_ptr(x), _ptr(router_w), T, H, E, k, int(normalize), _ptr(logits), _ptr(idx),
+                                        _ptr(wt), _stream()))
+    return (idx, wt, logits) if want_logits else (idx, wt)
+
+
 def moe_ffn(x: torch.Tensor, gate: KQuantPacked, up: KQuantPacked, down: KQuantPacked,
             expert_idx: torch.Tensor, expert_wt: torch.Tensor, n_experts: int) -> torch.Tensor:
     """Routed-expert FFN: sum_s wt[t,s] * down_e(silu(gate_e x) * up_e x)."""

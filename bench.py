@@ -497,7 +497,18 @@ def moe_leg():
         sec = e0.elapsed_time(e1) * 1e-3 / (reps * len(layers))
         nbytes = touched * per_expert
         flops = 2.0 * T * k * 3 * H * I
-        res[f"T{T}"] = {"us_per_layer": round(sec * 1e6, 2), "experts_touched": touched, "weight_bytes": nbytes,
+        # the router stage in front of it: fp32 router matvec + top-k softmax
+        wr = torch.randn(E, H, device="cuda") / H ** 0.5
+        kquant.moe_route(x, wr, k)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps * len(layers)):
+            kquant.moe_route(x, wr, k)
+        e1.record()
+        torch.cuda.synchronize()
+        route_us = e0.elapsed_time(e1) * 1e3 / (reps * len(layers))
+        res[f"T{T}"] = {"us_per_layer": round(sec * 1e6, 2), "route_us": round(route_us, 2),
+                        "experts_touched": touched, "weight_bytes": nbytes,
                         "GBps": round(nbytes / sec / 1e9, 1), "TFLOPs": round(flops / sec / 1e12, 2),
                         "kernel": capi.last_kernel()}
     return res

@@ -278,6 +278,29 @@ BPK_API int bpk_kq_moe_matmul(int type, const float *X, const void *W,
                               uint32_t row_stride_words, int x_per_slot,
                               void *stream);
 
+/* ---- MoE router stage: replaces moe_topk_softmax (and the router matmul) ----
+ * runtime/kernels/moe/topk_softmax.wgsl:23-67, dispatched after the router
+ * matmul in runtime/model_runner.cpp:3532-3548; its outputs are the expert_idx /
+ * expert_wt inputs of the calls above and below.  Per token: k passes of argmax
+ * over the experts not yet taken (`v > best` with best starting at -3.4e38 and
+ * index 0, so the lowest index wins a tie), then wt = exp(v - max) over the
+ * selected, times 1/sum when `normalize` is set and the sum is positive.
+ * logits: f32 [T, n_experts]; idx: u32 [T, k]; wt: f32 [T, k] (all device).
+ * n_experts <= 1024 (the reference's mask array), k <= 16 (its MAX_K). */
+BPK_API int bpk_moe_topk_softmax(const float *logits, uint32_t T,
+                                 uint32_t n_experts, uint32_t k, int normalize,
+                                 uint32_t *idx, float *wt, void *stream);
+
+/* The same behind the router matvec, one launch: logits[t, e] = sum_h X[t, h] *
+ * router_w[e, h] in fp32 (GGUF keeps `ffn_gate_inp.weight` as F32 [hidden,
+ * n_experts]; the reference requantises it to Q8 for its Q8 matmul,
+ * model_runner.cpp:3532-3540).  `logits` may be NULL when the caller does not
+ * need them.  hidden % 4 == 0; X and router_w 16-byte aligned. */
+BPK_API int bpk_moe_route(const float *X, const float *router_w, uint32_t T,
+                          uint32_t hidden, uint32_t n_experts, uint32_t k,
+                          int normalize, float *logits, uint32_t *idx, float *wt,
+                          void *stream);
+
 /* Whole routed-expert FFN for T tokens, replacing the per-slot dispatch list of
  * runtime/model_runner.cpp:3584-3651 (gate, up, silu*mul, down, weighted
  * accumulate) and the batched form in runtime/ops/moe.cpp:486-592:
