@@ -70,6 +70,7 @@ struct DeviceState {
     bool ready = false;
     kq::SplitScratch split{};
     uint32_t* moe_tiles = nullptr;   // kMoeWords words
+    uint32_t* argmax_scratch = nullptr;   // partial values | partial indices | tickets of bpk_argmax_rows
     float* route_logits = nullptr;   // ROUTE_SPREAD_TOKENS x 1024 router logits of a small-T route call
     UploadStage up{};                // created by the first upload on the device
 };
@@ -96,6 +97,9 @@ int ensure_device(int device, DeviceState** out)
         if (e == hipSuccess) e = hipMalloc((void**)&st.split.counters, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMemset(st.split.counters, 0, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMalloc((void**)&st.moe_tiles, kMoeWords * sizeof(uint32_t));
+        constexpr size_t kArgmaxWords = (size_t)kq::ARGMAX_MAX_ROWS * (2u * kq::ARGMAX_PARTS + 1u);
+        if (e == hipSuccess) e = hipMalloc((void**)&st.argmax_scratch, kArgmaxWords * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipMemset(st.argmax_scratch, 0, kArgmaxWords * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMalloc((void**)&st.route_logits, kq::ROUTE_SPREAD_TOKENS * 1024u * sizeof(float));
         if (cur != device && cur >= 0) (void)hipSetDevice(cur);
         if (e != hipSuccess) return hip_fail(e, "allocating split-K scratch");
@@ -200,6 +204,7 @@ int bpk_shutdown(void)
         (void)hipFree(st.split.counters);
         (void)hipFree(st.moe_tiles);
         (void)hipFree(st.route_logits);
+        (void)hipFree(st.argmax_scratch);
         for (int b = 0; b < 2; ++b) {
             if (st.up.buf[b]) (void)hipHostFree(st.up.buf[b]);
             if (st.up.sent[b]) (void)hipEventDestroy(st.up.sent[b]);
@@ -571,6 +576,30 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
         e = kq::launch_matmul_generic(a, s);
     }
     return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+int bpk_argmax_rows(const float* logits, uint32_t M, uint32_t N, uint32_t ld, int32_t* out_idx, float* out_val,
+                    void* stream)
+{
+    if (!logits || !out_idx) return fail(BPK_ERR_NULL, "logits and out_idx must be non-null");
+    if (N == 0 || ld < N) return fail(BPK_ERR_SHAPE, "N=%u must be positive and ld=%u at least N", N, ld);
+    if (M == 0) return BPK_OK;
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
+    float* pv = (float*)st->argmax_scratch;
+    uint32_t* pi = st->argmax_scratch + (size_t)kq::ARGMAX_MAX_ROWS * kq::ARGMAX_PARTS;
+    uint32_t* tickets = pi + (size_t)kq::ARGMAX_MAX_ROWS * kq::ARGMAX_PARTS;
+    const hipError_t e = kq::launch_argmax_rows(logits, M, N, ld, out_idx, out_val, pv, pi, tickets, (hipStream_t)stream);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, "argmax_rows");
+}
+
+int bpk_kq_matmul_argmax(int type, const float* X, const void* W, const float* bias, float* logits, uint32_t M,
+                         uint32_t N, uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, int32_t* out_idx,
+                         float* out_val, void* stream)
+{
+    if (!out_idx) return fail(BPK_ERR_NULL, "out_idx must be non-null");
+    if (int rc = bpk_kq_matmul(type, X, W, bias, logits, M, N, K, n_blocks, row_stride_words, 0, stream)) return rc;
+    return bpk_argmax_rows(logits, M, N, N, out_idx, out_val, stream);
 }
 
 static int check_route(uint32_t T, uint32_t n_experts, uint32_t k, const void* idx, const void* wt)

@@ -64,6 +64,13 @@ hipError_t launch_route(const float* X, const float* router_w, uint32_t T, uint3
                         uint32_t k, int normalize, float* logits_out, float* logits_scratch, uint32_t* idx, float* wt,
                         hipStream_t s);
 
+// Index (and value) of the largest element of each of M rows of N floats, rows ld apart; one launch per
+// ARGMAX_MAX_ROWS rows.  Scratch: ARGMAX_MAX_ROWS * ARGMAX_PARTS partial values and indices, and
+// ARGMAX_MAX_ROWS tickets that are zero between launches.
+constexpr uint32_t ARGMAX_PARTS = 64, ARGMAX_MAX_ROWS = 256;
+hipError_t launch_argmax_rows(const float* logits, uint32_t M, uint32_t N, uint32_t ld, int32_t* out_idx,
+                              float* out_val, float* part_val, uint32_t* part_idx, uint32_t* tickets, hipStream_t s);
+
 // Any shape with K % 256 == 0, any 4-byte aligned W.  M tiled by 4 inside.
 hipError_t launch_matmul_generic(const MatmulArgs& a, hipStream_t s);
 

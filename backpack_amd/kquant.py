@@ -153,6 +153,28 @@ def matmul_fused(x: torch.Tensor, w: KQuantPacked, prologue: int = capi.PRO_NONE
     return out
 
 
+def argmax_rows(logits: torch.Tensor):
+    """(index int32 [M], value f32 [M]) of the largest element of each row; lowest index on ties."""
+    assert logits.is_cuda and logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1
+    M, N = logits.shape
+    idx = torch.empty(M, dtype=torch.int32, device=logits.device)
+    val = torch.empty(M, dtype=torch.float32, device=logits.device)
+    capi.check(capi.lib().bpk_argmax_rows(_ptr(logits), M, N, logits.stride(0), _ptr(idx), _ptr(val), _stream()))
+    return idx, val
+
+
+def matmul_argmax(x: torch.Tensor, w: KQuantPacked, bias: torch.Tensor | None = None):
+    """lm_head and greedy pick in one call: (logits [M,N], index int32 [M], value f32 [M])."""
+    assert x.is_cuda and x.is_contiguous() and x.dtype == torch.float32 and x.shape[-1] == w.K
+    M = x.numel() // w.K
+    logits = torch.empty((M, w.N), dtype=torch.float32, device=x.device)
+    idx = torch.empty(M, dtype=torch.int32, device=x.device)
+    val = torch.empty(M, dtype=torch.float32, device=x.device)
+    capi.check(capi.lib().bpk_kq_matmul_argmax(w.type, _ptr(x), _ptr(w.data), _ptr(bias), _ptr(logits), M, w.N, w.K,
+                                               w.n_blocks, w.row_stride_words, _ptr(idx), _ptr(val), _stream()))
+    return logits, idx, val
+
+
 def dequant_rows(w: KQuantPacked, rows: torch.Tensor | None = None, M: int | None = None) -> torch.Tensor:
     """fp32 rows of the matrix (the q6k_gather contract); rows: int32 device tensor."""
     if rows is not None:

@@ -350,6 +350,16 @@ def fused_leg(mats, use_graph):
         res["separate_ms"] = round(timed(fused_pass), 4)
     finally:
         capi.set_option("fused_separate", 0)
+    # the greedy pick behind lm_head: one launch over the 128256 logits, timed in a graph of 50
+    logits = next(y for n_, _, _, y in mats if n_ == "lm_head")
+    idx = torch.empty(1, dtype=torch.int32, device="cuda")
+    val = torch.empty(1, dtype=torch.float32, device="cuda")
+
+    def picks():
+        for _ in range(50):
+            capi.check(capi.lib().bpk_argmax_rows(logits.data_ptr(), 1, logits.shape[1], logits.shape[1], idx.data_ptr(),
+                                                  val.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    res["argmax_us"] = round(timed(picks) * 1e3 / 50, 2)
     n = sum(1 for name, *_ in mats if name in ("qkv", "down"))
     res["launches_saved"] = int(n * 1.5)     # norm per qkv; act*mul and add per down
     return res

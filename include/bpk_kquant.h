@@ -239,6 +239,27 @@ BPK_API int bpk_kq_matmul_fused(int type, const float *X, const void *W,
                                 const bpk_kq_fusion *fusion, void *workspace,
                                 size_t workspace_bytes, void *stream);
 
+/* ---- greedy sampling tail: replaces argmax + argmax_reduce -----------------
+ * The two dispatches after the lm_head matvec (kernels argmax.wgsl /
+ * argmax_reduce.wgsl, wired in runtime/model_runner.cpp:2441-2453), as one
+ * launch: out_idx[m] = index of the largest of logits[m*ld .. +N-1], the
+ * lowest index among equal maxima (the reference leaves ties to its lane
+ * order), 0 when nothing exceeds -1e30 (the reference's starting value).
+ * out_val (may be NULL) receives the maximum.  Launches on one device share a
+ * scratch area and must not overlap. */
+BPK_API int bpk_argmax_rows(const float *logits, uint32_t M, uint32_t N,
+                            uint32_t ld, int32_t *out_idx, float *out_val,
+                            void *stream);
+
+/* lm_head and its argmax in one call (runtime/model_runner.cpp:4124-4135 then
+ * :2441-2453): bpk_kq_matmul with y_offset 0 into `logits` (f32 [M,N], kept for
+ * the caller) followed by bpk_argmax_rows on it. */
+BPK_API int bpk_kq_matmul_argmax(int type, const float *X, const void *W,
+                                 const float *bias, float *logits, uint32_t M,
+                                 uint32_t N, uint32_t K, uint32_t n_blocks,
+                                 uint32_t row_stride_words, int32_t *out_idx,
+                                 float *out_val, void *stream);
+
 /* Prefill form: X is bf16 [M,K] (raw 16-bit patterns), Y f32 [M,N].  Weight
  * tiles are dequantised to bf16 in LDS and contracted on the matrix cores
  * with fp32 accumulation.  The reference has no such kernel: its k-quant

@@ -241,6 +241,18 @@ def moe_topk_softmax(logits, k: int, normalize: bool = True):
     return idx, wt
 
 
+def argmax_rows(logits) -> np.ndarray:
+    """Greedy pick per row as the reference's argmax + argmax_reduce kernels compute it on a sequential
+    scan (`v > best` from best = -1e30, index 0; argmax.wgsl, wired in runtime/model_runner.cpp:2441-2453):
+    the first index holding the maximum, 0 when nothing exceeds -1e30.  Pinned by a python loop on small
+    rows in tests/test_oracle_pins.py."""
+    lg = np.asarray(logits, dtype=np.float32)
+    masked = np.where(lg > np.float32(-1e30), lg, -np.inf)      # NaN compares false: never picked
+    idx = np.argmax(masked, axis=1)
+    none = ~np.any(lg > np.float32(-1e30), axis=1)
+    return np.where(none, 0, idx).astype(np.int32)
+
+
 def moe_offsets(idx, rows_per_expert: int) -> np.ndarray:
     idx = _c(idx, np.uint32)
     out = np.empty_like(idx)

@@ -322,3 +322,23 @@ def test_prologues_against_closed_forms_in_float64(kqo):
     edge = np.array([[0.0, 30.0, -30.0, 1.0, 2.0, 3.0]], dtype=np.float32)
     assert kqo.prologue(2, edge, 3).tolist() == [[0.0, 60.0, -0.0]] or np.allclose(kqo.prologue(2, edge, 3), [[0, 60, 0]], atol=1e-10)
     assert np.allclose(kqo.prologue(3, edge, 3), [[0, 60, 0]], atol=1e-10)
+
+
+def test_argmax_rows_is_the_sequential_scan(kqo):
+    """The numpy form against the reference's scan written out as a loop, including ties, rows with
+    nothing above the starting value, NaN and infinities."""
+    rng = np.random.default_rng(2)
+    rows = [rng.standard_normal(37).astype(np.float32) for _ in range(20)]
+    rows += [np.zeros(37, np.float32), np.full(37, -2e30, np.float32), np.full(37, -np.inf, np.float32)]
+    r = rng.standard_normal(37).astype(np.float32); r[[5, 20]] = r.max() + 1; rows.append(r)     # a tie
+    r = rng.standard_normal(37).astype(np.float32); r[3] = np.nan; r[30] = np.inf; rows.append(r)
+    r = np.full(37, np.nan, np.float32); rows.append(r)
+    lg = np.stack(rows)
+    want = []
+    for row in lg:
+        best, bi = np.float32(-1e30), 0
+        for i, v in enumerate(row):
+            if v > best:
+                best, bi = v, i
+        want.append(bi)
+    assert kqo.argmax_rows(lg).tolist() == want
