@@ -12,6 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libbpk_kquant.so")
 
 Q4_K = 12
+Q5_K = 13
 Q6_K = 14
 
 FAMILY_AUTO, FAMILY_GENERIC, FAMILY_GEMV_ROWS, FAMILY_MFMA_SMALL, FAMILY_MFMA_GEMM = range(5)

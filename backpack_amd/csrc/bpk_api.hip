@@ -119,12 +119,15 @@ int current_state(DeviceState** out)
     return ensure_device(dev, out);
 }
 
-bool known_type(int type) { return type == BPK_TYPE_Q4_K || type == BPK_TYPE_Q6_K; }
+bool known_type(int type) { return type == BPK_TYPE_Q4_K || type == BPK_TYPE_Q5_K || type == BPK_TYPE_Q6_K; }
+// Q5_K is served by the packers, the row dequantiser and the fp32 matmul (generic kernel); the bf16 GEMM
+// and the MoE entry points take the two types their kernels are written for.
+bool fast_type(int type) { return type == BPK_TYPE_Q4_K || type == BPK_TYPE_Q6_K; }
 
 int check_matmul(int type, const void* X, const void* W, const void* Y, uint32_t M, uint32_t N, uint32_t K,
                  uint32_t n_blocks, uint32_t row_stride_words)
 {
-    if (!known_type(type)) return fail(BPK_ERR_TYPE, "unsupported GGUF type %d (Q4_K=12, Q6_K=14)", type);
+    if (!known_type(type)) return fail(BPK_ERR_TYPE, "unsupported GGUF type %d (Q4_K=12, Q5_K=13, Q6_K=14)", type);
     if (!X || !W || !Y) return fail(BPK_ERR_NULL, "X, W and Y must be non-null");
     if (K == 0 || K % KQ_QK) return fail(BPK_ERR_SHAPE, "K=%u is not a positive multiple of 256", K);
     if (N == 0) return fail(BPK_ERR_SHAPE, "N must be positive");
@@ -490,6 +493,7 @@ int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bi
 int bpk_kq_matmul_bf16(int type, const uint16_t* X, const void* W, const float* bias, float* Y, uint32_t M,
                        uint32_t N, uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, void* stream)
 {
+    if (type == BPK_TYPE_Q5_K) return fail(BPK_ERR_TYPE, "the bf16 GEMM takes Q4_K and Q6_K");
     if (int rc = check_matmul(type, X, W, Y, M, N, K, n_blocks, row_stride_words)) return rc;
     if (M == 0) return BPK_OK;
     if (int rc = current_state(nullptr)) return rc;
@@ -525,6 +529,7 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
                       uint32_t k, uint32_t n_experts, uint32_t N, uint32_t K, uint32_t n_blocks,
                       uint32_t row_stride_words, int x_per_slot, void* stream)
 {
+    if (type == BPK_TYPE_Q5_K) return fail(BPK_ERR_TYPE, "the MoE entry points take Q4_K and Q6_K");
     if (int rc = check_matmul(type, X, W, Y, T, N, K, n_blocks, row_stride_words)) return rc;
     if (!expert_idx) return fail(BPK_ERR_NULL, "expert_idx must be non-null");
     if (k == 0 || n_experts == 0) return fail(BPK_ERR_SHAPE, "k and n_experts must be positive");
@@ -652,7 +657,7 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
                    uint32_t n_experts, uint32_t hidden, uint32_t inter, void* scratch, size_t scratch_bytes,
                    void* stream)
 {
-    if (!known_type(type_gu) || !known_type(type_dn)) return fail(BPK_ERR_TYPE, "unsupported GGUF type");
+    if (!fast_type(type_gu) || !fast_type(type_dn)) return fail(BPK_ERR_TYPE, "the MoE entry points take Q4_K and Q6_K");
     if (!X || !gate || !up || !down || !expert_idx || !expert_wt || !out)
         return fail(BPK_ERR_NULL, "X, gate, up, down, expert_idx, expert_wt and out must be non-null");
     if (k == 0 || n_experts == 0) return fail(BPK_ERR_SHAPE, "k and n_experts must be positive");

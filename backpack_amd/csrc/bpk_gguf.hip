@@ -440,7 +440,7 @@ int bpk_gguf_array_string(const bpk_gguf* g, const char* key, uint64_t index, ch
     return BPK_OK;
 }
 
-// Named Q4_K / Q6_K matrices (GGUF shape {K, N}) -> one device weight, rows stacked in the order given
+// Named Q4_K / Q5_K / Q6_K matrices (GGUF shape {K, N}) -> one device weight, rows stacked in the order given
 // (q|k|v, gate|up).  All parts must share the type and K.
 int bpk_gguf_weight_create(const bpk_gguf* g, const char* const* names, uint32_t n_names, bpk_weight** out)
 {
@@ -454,8 +454,8 @@ int bpk_gguf_weight_create(const bpk_gguf* g, const char* const* names, uint32_t
         auto it = g->index.find(names[i]);
         if (it == g->index.end()) return fail(BPK_ERR_NOT_FOUND, "no tensor named %s", names[i]);
         const Tensor& t = g->tensors[it->second];
-        if (t.type != BPK_TYPE_Q4_K && t.type != BPK_TYPE_Q6_K)
-            return fail(BPK_ERR_TYPE, "%s has GGUF type %u; this path takes Q4_K (12) and Q6_K (14)", names[i], t.type);
+        if (t.type != BPK_TYPE_Q4_K && t.type != BPK_TYPE_Q5_K && t.type != BPK_TYPE_Q6_K)
+            return fail(BPK_ERR_TYPE, "%s has GGUF type %u; this path takes Q4_K (12), Q5_K (13) and Q6_K (14)", names[i], t.type);
         if (t.n_dims < 1 || t.n_dims > 2 || t.dims[0] > 0xFFFFFFFFull || t.dims[1] > 0xFFFFFFFFull || t.dims[1] == 0)
             return fail(BPK_ERR_SHAPE, "%s is not a matrix", names[i]);
         if (i == 0) { type = t.type; K = (uint32_t)t.dims[0]; }

@@ -1,4 +1,4 @@
-// kq_dequant.hip — dequantise selected rows of a packed Q4_K / Q6_K matrix to
+// kq_dequant.hip — dequantise selected rows of a packed Q4_K / Q5_K / Q6_K matrix to
 // fp32, bit-identical to the CPU formula.  One thread per output element; the
 // 256 threads of a workgroup cover one superblock of one output row, so the
 // block's bytes are read once from HBM and served from cache to the rest.
@@ -17,10 +17,10 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(const uint8_t* __rest
     const uint32_t b = blockIdx.x;
     const int32_t rid = rows ? rows[m] : (int32_t)m;
     const uint32_t row = rid > 0 ? (uint32_t)rid : 0u;
-    constexpr uint32_t BB = TYPE == KQ_TYPE_Q4_K ? KQ_Q4K_BYTES : KQ_Q6K_BYTES;
+    constexpr uint32_t BB = TYPE == KQ_TYPE_Q4_K ? KQ_Q4K_BYTES : TYPE == KQ_TYPE_Q5_K ? KQ_Q5K_BYTES : KQ_Q6K_BYTES;
     const uint8_t* blk = W + (size_t)row * row_stride_bytes + (size_t)b * BB;
     const uint32_t e = threadIdx.x;
-    const float v = TYPE == KQ_TYPE_Q4_K ? q4k_element(blk, e) : q6k_element(blk, e);
+    const float v = kq_element<TYPE>(blk, e);
     out[(size_t)m * K + (size_t)b * KQ_QK + e] = v;
 }
 
@@ -39,6 +39,9 @@ hipError_t launch_dequant_rows(int type, const uint8_t* W, uint32_t row_stride_b
         float* o = out + (size_t)m0 * K;
         if (type == KQ_TYPE_Q4_K)
             hipLaunchKernelGGL(dequant_rows_kernel<KQ_TYPE_Q4_K>, grid, dim3(256), 0, s, w,
+                               row_stride_bytes, r, K, o);
+        else if (type == KQ_TYPE_Q5_K)
+            hipLaunchKernelGGL(dequant_rows_kernel<KQ_TYPE_Q5_K>, grid, dim3(256), 0, s, w,
                                row_stride_bytes, r, K, o);
         else
             hipLaunchKernelGGL(dequant_rows_kernel<KQ_TYPE_Q6_K>, grid, dim3(256), 0, s, w,

@@ -14,16 +14,18 @@
 #include <stdint.h>
 
 #define KQ_TYPE_Q4_K 12
+#define KQ_TYPE_Q5_K 13
 #define KQ_TYPE_Q6_K 14
 #define KQ_QK 256
 #define KQ_Q4K_BYTES 144
+#define KQ_Q5K_BYTES 176
 #define KQ_Q6K_BYTES 210
 
 namespace kq {
 
 __host__ __device__ inline uint32_t block_bytes(int type)
 {
-    return type == KQ_TYPE_Q4_K ? KQ_Q4K_BYTES : type == KQ_TYPE_Q6_K ? KQ_Q6K_BYTES : 0u;
+    return type == KQ_TYPE_Q4_K ? KQ_Q4K_BYTES : type == KQ_TYPE_Q5_K ? KQ_Q5K_BYTES : type == KQ_TYPE_Q6_K ? KQ_Q6K_BYTES : 0u;
 }
 
 // Exact IEEE half -> float including subnormals, infinities and NaN payloads:
@@ -84,6 +86,34 @@ __device__ __forceinline__ float q4k_element(const uint8_t* blk, uint32_t e)
     return __fsub_rn(a, b);
 }
 
+// One Q5_K element (176-byte block: d, dmin, the Q4_K scale bytes, 32 bytes of fifth bits at 16, the
+// nibbles at 48): (d*sc)*(nibble | bit<<4) - dmin*mn, rounded as the CPU formula rounds it.
+__device__ __forceinline__ float q5k_element(const uint8_t* blk, uint32_t e)
+{
+    const float d = half_bits_to_float(u16_at(blk, 0));
+    const float dmin = half_bits_to_float(u16_at(blk, 2));
+    const uint32_t sb = e >> 5, i = e & 31u;
+    uint32_t u0 = 0, u1 = 0, u2 = 0;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        u0 |= byte_at(blk, 4 + t) << (8 * t);
+        u1 |= byte_at(blk, 8 + t) << (8 * t);
+        u2 |= byte_at(blk, 12 + t) << (8 * t);
+    }
+    uint32_t sc, mn;
+    q4k_scale_min(u0, u1, u2, (int)sb, sc, mn);
+    const uint32_t qb = byte_at(blk, 48 + (sb >> 1) * 32 + i);
+    const uint32_t lo = (sb & 1u) ? (qb >> 4) : (qb & 15u);
+    const uint32_t q = lo | (((byte_at(blk, 16 + i) >> sb) & 1u) << 4);
+    const float a = __fmul_rn(__fmul_rn(d, (float)sc), (float)q);
+    const float b = __fmul_rn(dmin, (float)mn);
+    return __fsub_rn(a, b);
+}
+
+// Element e of a block of any of the three types.
+template <int TYPE>
+__device__ __forceinline__ float kq_element(const uint8_t* blk, uint32_t e);
+
 __device__ __forceinline__ float q6k_element(const uint8_t* blk, uint32_t e)
 {
     const float d = half_bits_to_float(u16_at(blk, 208));
@@ -95,5 +125,9 @@ __device__ __forceinline__ float q6k_element(const uint8_t* blk, uint32_t e)
     const int sc = (int)(int8_t)byte_at(blk, 192 + 8 * h + 2 * t + (l >> 4));
     return __fmul_rn(__fmul_rn(d, (float)sc), (float)q);
 }
+
+template <> __device__ __forceinline__ float kq_element<KQ_TYPE_Q4_K>(const uint8_t* blk, uint32_t e) { return q4k_element(blk, e); }
+template <> __device__ __forceinline__ float kq_element<KQ_TYPE_Q5_K>(const uint8_t* blk, uint32_t e) { return q5k_element(blk, e); }
+template <> __device__ __forceinline__ float kq_element<KQ_TYPE_Q6_K>(const uint8_t* blk, uint32_t e) { return q6k_element(blk, e); }
 
 }  // namespace kq

@@ -21,7 +21,7 @@ __device__ __forceinline__ float wave_sum(float v)
 template <int TYPE, int MT, bool INDIRECT>
 __global__ __launch_bounds__(256) void matmul_generic_kernel(MatmulArgs a)
 {
-    constexpr uint32_t BB = TYPE == KQ_TYPE_Q4_K ? KQ_Q4K_BYTES : KQ_Q6K_BYTES;
+    constexpr uint32_t BB = TYPE == KQ_TYPE_Q4_K ? KQ_Q4K_BYTES : TYPE == KQ_TYPE_Q5_K ? KQ_Q5K_BYTES : KQ_Q6K_BYTES;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t n = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (n >= a.N) return;  // whole wave leaves together
@@ -53,8 +53,7 @@ __global__ __launch_bounds__(256) void matmul_generic_kernel(MatmulArgs a)
         float w[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            w[j] = TYPE == KQ_TYPE_Q4_K ? q4k_element(blk, lane * 4u + j)
-                                        : q6k_element(blk, lane * 4u + j);
+            w[j] = kq_element<TYPE>(blk, lane * 4u + j);
         const size_t k0 = (size_t)b * KQ_QK + lane * 4u;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
@@ -92,6 +91,8 @@ hipError_t launch_matmul_generic(const MatmulArgs& a, hipStream_t s)
             dim3 grid(gx, pc);
             if (a.type == KQ_TYPE_Q4_K)
                 hipLaunchKernelGGL((matmul_generic_kernel<KQ_TYPE_Q4_K, 1, true>), grid, dim3(256), 0, s, c);
+            else if (a.type == KQ_TYPE_Q5_K)
+                hipLaunchKernelGGL((matmul_generic_kernel<KQ_TYPE_Q5_K, 1, true>), grid, dim3(256), 0, s, c);
             else
                 hipLaunchKernelGGL((matmul_generic_kernel<KQ_TYPE_Q6_K, 1, true>), grid, dim3(256), 0, s, c);
         }
@@ -107,6 +108,8 @@ hipError_t launch_matmul_generic(const MatmulArgs& a, hipStream_t s)
         dim3 grid(gx, (mc + MT - 1) / MT);
         if (a.type == KQ_TYPE_Q4_K)
             hipLaunchKernelGGL((matmul_generic_kernel<KQ_TYPE_Q4_K, MT, false>), grid, dim3(256), 0, s, c);
+        else if (a.type == KQ_TYPE_Q5_K)
+            hipLaunchKernelGGL((matmul_generic_kernel<KQ_TYPE_Q5_K, MT, false>), grid, dim3(256), 0, s, c);
         else
             hipLaunchKernelGGL((matmul_generic_kernel<KQ_TYPE_Q6_K, MT, false>), grid, dim3(256), 0, s, c);
     }

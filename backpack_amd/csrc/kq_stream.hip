@@ -221,10 +221,14 @@ __device__ __forceinline__ void ring_load2(uint32_t& v, const uint8_t* ptr)
 //   hdr: the block's first 16 bytes; q: 16 quant bytes (piece j of the block)
 //   xlo/xhi: activations of the piece's 16 elements in the even / odd sub-block
 //   sel_hi: lane constant, j/2 >= 2;  sh: lane constant, 16 * ((j/2) & 1)
-template <int MT>
+// Q5: qh holds the 16 bytes of fifth bits of the piece's elements (bit 2g of a byte for the even sub-block,
+// bit 2g+1 for the odd one, sbit = 2g); the bit joins its nibble in the fp16 mantissa (bit 4 beside a low
+// nibble, bit 8 beside a high one: a five-bit value is still a subnormal).
+template <int MT, bool Q5 = false>
 __device__ __forceinline__ void q4k_piece_dot(const s_u32x4 hdr, const s_u32x4 q, const float (&xlo)[MT][16],
                                               const float (&xhi)[MT][16], const float (&xs_lo)[MT],
-                                              const float (&xs_hi)[MT], bool sel_hi, uint32_t sh, float (&acc)[MT])
+                                              const float (&xs_hi)[MT], bool sel_hi, uint32_t sh, float (&acc)[MT],
+                                              const s_u32x4 qh = s_u32x4{0, 0, 0, 0}, uint32_t sbit = 0)
 {
     float alo[MT], ahi[MT];
 #pragma unroll
@@ -233,10 +237,21 @@ __device__ __forceinline__ void q4k_piece_dot(const s_u32x4 hdr, const s_u32x4 q
     for (int m = 0; m < 4; ++m) {
         const uint32_t w = q[m];
         const uint32_t w8 = w >> 8;
-        const s_half2 a = __builtin_bit_cast(s_half2, w & 0x000F000Fu);     // low nibbles of bytes 0, 2
-        const s_half2 b = __builtin_bit_cast(s_half2, w & 0x00F000F0u);     // high nibbles of bytes 0, 2 (x16)
-        const s_half2 c = __builtin_bit_cast(s_half2, w8 & 0x000F000Fu);    // low nibbles of bytes 1, 3
-        const s_half2 d = __builtin_bit_cast(s_half2, w8 & 0x00F000F0u);    // high nibbles of bytes 1, 3 (x16)
+        uint32_t ua = w & 0x000F000Fu;     // low nibbles of bytes 0, 2
+        uint32_t ub = w & 0x00F000F0u;     // high nibbles of bytes 0, 2 (x16)
+        uint32_t uc = w8 & 0x000F000Fu;    // low nibbles of bytes 1, 3
+        uint32_t ud = w8 & 0x00F000F0u;    // high nibbles of bytes 1, 3 (x16)
+        if constexpr (Q5) {
+            const uint32_t hb = qh[m] >> sbit;   // bit 0 of each byte: even sub-block; bit 1: odd sub-block
+            ua |= (hb << 4) & 0x00100010u;
+            uc |= (hb >> 4) & 0x00100010u;
+            ub |= (hb << 7) & 0x01000100u;
+            ud |= (hb >> 1) & 0x01000100u;
+        }
+        const s_half2 a = __builtin_bit_cast(s_half2, ua);
+        const s_half2 b = __builtin_bit_cast(s_half2, ub);
+        const s_half2 c = __builtin_bit_cast(s_half2, uc);
+        const s_half2 d = __builtin_bit_cast(s_half2, ud);
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
             alo[t] = s_fma_h(a.x, xlo[t][4 * m + 0], alo[t]);
@@ -270,23 +285,31 @@ __device__ __forceinline__ void q4k_piece_dot(const s_u32x4 hdr, const s_u32x4 q
     }
 }
 
-// One row in flight for the Q4_K kernel: P headers and P quant pieces per lane.
-template <int P>
+// One row in flight for the Q4_K / Q5_K kernel: P headers and P quant pieces per lane, for Q5_K also P
+// pieces of fifth bits (blocks of 176 bytes: header, 32 bytes of fifth bits, quants).
+template <int P, bool Q5>
 struct Q4Slot {
-    s_u32x4 hdr[P], q[P];
+    s_u32x4 hdr[P], q[P], qh[Q5 ? P : 1];
     __device__ __forceinline__ void fill(const uint8_t* row, const uint32_t (&hoff)[P], uint32_t j)
     {
 #pragma unroll
         for (int pass = 0; pass < P; ++pass) {
             ring_load16(hdr[pass], row + hoff[pass]);
-            ring_load16(q[pass], row + hoff[pass] + 16u + 16u * j);
+            ring_load16(q[pass], row + hoff[pass] + (Q5 ? 48u : 16u) + 16u * j);
+            if constexpr (Q5) ring_load16(qh[pass], row + hoff[pass] + 16u + 16u * (j & 1u));
         }
     }
     // Every register of the slot passes through the wait.
     template <int N>
     __device__ __forceinline__ void wait()
     {
-        if constexpr (P == 1)
+        if constexpr (Q5 && P == 1)
+            asm volatile("s_waitcnt vmcnt(%3)" : "+v"(hdr[0]), "+v"(q[0]), "+v"(qh[0]) : "n"(N));
+        else if constexpr (Q5)
+            asm volatile("s_waitcnt vmcnt(%6)"
+                         : "+v"(hdr[0]), "+v"(q[0]), "+v"(qh[0]), "+v"(hdr[1]), "+v"(q[1]), "+v"(qh[1])
+                         : "n"(N));
+        else if constexpr (P == 1)
             asm volatile("s_waitcnt vmcnt(%2)" : "+v"(hdr[0]), "+v"(q[0]) : "n"(N));
         else
             asm volatile("s_waitcnt vmcnt(%4)" : "+v"(hdr[0]), "+v"(q[0]), "+v"(hdr[1]), "+v"(q[1]) : "n"(N));
@@ -294,7 +317,7 @@ struct Q4Slot {
 };
 
 // P passes of 8 superblocks cover a row (n_blocks <= 8 * P); D rows in flight; MT tokens.
-template <int P, int NW, int D, int MT, typename PT>
+template <int P, int NW, int D, int MT, typename PT, bool Q5 = false>
 __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
 {
     stream_select_pair(p);
@@ -309,6 +332,7 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
     const uint32_t bl = lane >> 3, j = lane & 7u, g = j >> 1, h = j & 1u;
     const bool sel_hi = g >= 2u;
     const uint32_t sh = 16u * (g & 1u);
+    constexpr uint32_t BLOCK = Q5 ? KQ_Q5K_BYTES : KQ_Q4K_BYTES;
 
     float xlo[P][MT][16], xhi[P][MT][16], xs_lo[P][MT], xs_hi[P][MT];
     uint32_t hoff[P];
@@ -321,7 +345,7 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
             uint32_t b = pass * 8u + bl;
             const bool valid = b < p.n_blocks;
             b = valid ? b : p.n_blocks - 1u;
-            hoff[pass] = b * KQ_Q4K_BYTES;
+            hoff[pass] = b * BLOCK;
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 const float4* xp = (const float4*)(p.X + (size_t)t * ldx + (size_t)b * KQ_QK + 64u * g + 16u * h);
@@ -354,7 +378,7 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
                 const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)p.K + stream_eps(p));
 #pragma unroll
                 for (int pass = 0; pass < P; ++pass) {
-                    const float* wp = stream_norm_w(p) + hoff[pass] / KQ_Q4K_BYTES * KQ_QK + 64u * g + 16u * h;
+                    const float* wp = stream_norm_w(p) + hoff[pass] / BLOCK * KQ_QK + 64u * g + 16u * h;
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         xlo[pass][t][i] = xlo[pass][t][i] * rstd * wp[i];
@@ -381,8 +405,8 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
     // slots' loads outstanding.  Past the end of the wave's rows the last row is
     // fetched and summed again (cache hits, result dropped), so the row loop has
     // no branch and the number of loads in flight is the same at every wait.
-    constexpr int SLOT_LOADS = 2 * P;
-    Q4Slot<P> ring[D] = {};
+    constexpr int SLOT_LOADS = (Q5 ? 3 : 2) * P;
+    Q4Slot<P, Q5> ring[D] = {};
     // (The ring is filled after the prologue even where that is long: registers with a load in flight
     // must stay where they are, and across the prologue's arithmetic the compiler moves them.)
 #pragma unroll
@@ -405,8 +429,8 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
                 for (int t = 0; t < MT; ++t) acc[t] = 0.0f;
 #pragma unroll
                 for (int pass = 0; pass < P; ++pass)
-                    q4k_piece_dot<MT>(ring[d].hdr[pass], ring[d].q[pass], xlo[pass], xhi[pass], xs_lo[pass],
-                                      xs_hi[pass], sel_hi, sh, acc);
+                    q4k_piece_dot<MT, Q5>(ring[d].hdr[pass], ring[d].q[pass], xlo[pass], xhi[pass], xs_lo[pass],
+                                          xs_hi[pass], sel_hi, sh, acc, ring[d].qh[Q5 ? pass : 0], 2u * g);
                 ring[d].fill(p.W + (size_t)(gw + min(c0 + i + D, n_rows - 1u) * stride) * p.row_stride_bytes, hoff, j);
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
@@ -714,7 +738,8 @@ bool gemv_stream_supported(const MatmulArgs& a)
     if (a.expert_idx && (a.M < 1 || a.M > 65535u || a.bias)) return false;
     if (((uintptr_t)a.X & 15u)) return false;
     if (a.n_blocks < 1) return false;
-    if (a.type == KQ_TYPE_Q4_K) {
+    if (a.type == KQ_TYPE_Q4_K || a.type == KQ_TYPE_Q5_K) {
+        if (a.type == KQ_TYPE_Q5_K && a.expert_idx) return false;
         if (a.n_blocks > 16) return false;
         if (((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u)) return false;
         return true;
@@ -740,11 +765,13 @@ static void launch_q6k_one(dim3 grid, hipStream_t s, const PT& p)
     if constexpr (!absent) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, D, MT, PT>), grid, dim3(64 * KW), 0, s, p);
 }
 
-template <int P, int NW, int D, int MT, typename PT>
+// (Q5_K: no grouped launches, the MoE entry points do not take the type; at most two rows in flight, the
+// third load per pass leaves no registers for four.)
+template <int P, int NW, int D, int MT, typename PT, bool Q5>
 static void launch_q4k_one(dim3 grid, hipStream_t s, const PT& p)
 {
-    constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && D != 2);
-    if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT>), grid, dim3(64 * NW), 0, s, p);
+    constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && D != 2) || (Q5 && (PT::kGrouped || D > 2));
+    if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT, Q5>), grid, dim3(64 * NW), 0, s, p);
 }
 
 template <typename PT>
@@ -790,12 +817,16 @@ static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, h
     uint32_t wgs = t.splits > 0 ? ((a.N + (uint32_t)t.splits - 1u) / (uint32_t)t.splits + NW - 1u) / NW
                                 : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
     wgs = (wgs + pairs * twins - 1u) / (pairs * twins);
-    const int depth = PT::kFused ? 2 : t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
+    const bool q5 = a.type == KQ_TYPE_Q5_K;
+    int depth = PT::kFused ? 2 : t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
+    if (q5 && depth > 2) depth = 2;
     const dim3 grid(wgs, pairs, twins);
 #define KQ_STREAM_LAUNCH(P, D) \
     do { \
-        if (two) launch_q4k_one<P, NW, D, 2>(grid, s, p); \
-        else launch_q4k_one<P, NW, D, 1>(grid, s, p); \
+        if (q5 && two) launch_q4k_one<P, NW, D, 2, PT, true>(grid, s, p); \
+        else if (q5) launch_q4k_one<P, NW, D, 1, PT, true>(grid, s, p); \
+        else if (two) launch_q4k_one<P, NW, D, 2, PT, false>(grid, s, p); \
+        else launch_q4k_one<P, NW, D, 1, PT, false>(grid, s, p); \
     } while (0)
     if (a.n_blocks <= 8u) {
         if (depth <= 1) KQ_STREAM_LAUNCH(1, 1);

@@ -14,7 +14,7 @@ import numpy as np
 import torch
 
 from . import capi
-from .capi import Q4_K, Q6_K  # noqa: F401
+from .capi import Q4_K, Q5_K, Q6_K  # noqa: F401
 
 
 def _stream() -> int:
@@ -44,7 +44,7 @@ def pack_host(type_: int, raw: np.ndarray, N: int, K: int) -> np.ndarray:
     """pack_q4k / pack_q6k on the host through the library's packer."""
     raw = np.ascontiguousarray(raw, dtype=np.uint8)
     nb, rs = capi.layout(type_, K)
-    assert raw.size == N * nb * (144 if type_ == Q4_K else 210), "raw size does not match N x K"
+    assert raw.size == N * nb * {12: 144, 13: 176, 14: 210}[type_], "raw size does not match N x K"
     out = np.empty(N * rs, dtype=np.uint32)
     capi.check(capi.lib().bpk_kq_pack_host(type_, raw.ctypes.data, N, K, out.ctypes.data))
     return out

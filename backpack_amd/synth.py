@@ -19,7 +19,8 @@ import numpy as np
 Q4_K = 12
 Q6_K = 14
 QK_K = 256
-BLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
+Q5_K = 13
+BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210}
 SIGMA = 0.01
 
 
@@ -77,6 +78,28 @@ def q4k_decode_f64(d, dmin, sc, mn, q) -> np.ndarray:
     return w.reshape(N, nb * 256)
 
 
+def q5k_fields(rng: np.random.Generator, N: int, nb: int):
+    d, dmin, sc, mn, _ = q4k_fields(rng, N, nb)
+    q = rng.integers(0, 32, size=(N, nb, 256), dtype=np.uint8)
+    return d, dmin, sc, mn, q
+
+
+def q5k_encode(d, dmin, sc, mn, q) -> np.ndarray:
+    """Decoded fields -> raw 176-byte superblocks: the Q4_K header, 32 bytes of fifth bits (bit sb of
+    byte i belongs to element i of sub-block sb), then the Q4_K nibble bytes."""
+    N, nb = d.shape
+    low = q4k_encode(d, dmin, sc, mn, q & 15)
+    blk = np.zeros((N, nb, 176), dtype=np.uint8)
+    blk[..., 0:16] = low[..., 0:16]
+    hi = (q >> 4).reshape(N, nb, 8, 32)
+    qh = np.zeros((N, nb, 32), dtype=np.uint8)
+    for sb in range(8):
+        qh |= hi[:, :, sb, :] << sb
+    blk[..., 16:48] = qh
+    blk[..., 48:176] = low[..., 16:144]
+    return blk
+
+
 def q6k_fields(rng: np.random.Generator, N: int, nb: int):
     d = np.abs(rng.normal(0.0, SIGMA, size=(N, nb))).astype(np.float16)
     sc = rng.integers(-64, 64, size=(N, nb, 16), dtype=np.int8)
@@ -118,6 +141,8 @@ def make_raw(type_: int, N: int, K: int, seed: int = 0) -> np.ndarray:
     nb = n_blocks(K)
     if type_ == Q4_K:
         blk = q4k_encode(*q4k_fields(rng, N, nb))
+    elif type_ == Q5_K:
+        blk = q5k_encode(*q5k_fields(rng, N, nb))
     elif type_ == Q6_K:
         blk = q6k_encode(*q6k_fields(rng, N, nb))
     else:

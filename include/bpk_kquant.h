@@ -34,11 +34,14 @@ extern "C" {
 
 /* GGUF tensor type codes (runtime/gguf_loader.h:29-30). */
 #define BPK_TYPE_Q4_K 12
+#define BPK_TYPE_Q5_K 13 /* packers, weights, dequantised rows and the fp32 matmul
+                            (bpk_kq_matmul, bpk_kq_matmul_fused, _argmax); the bf16
+                            GEMM and the MoE calls return BPK_ERR_TYPE for it */
 #define BPK_TYPE_Q6_K 14
 
 enum {
     BPK_OK = 0,
-    BPK_ERR_TYPE = -1,      /* not Q4_K / Q6_K                               */
+    BPK_ERR_TYPE = -1,      /* not a type this entry point serves            */
     BPK_ERR_SHAPE = -2,     /* K not a multiple of 256, zero sizes, overflow  */
     BPK_ERR_NULL = -3,      /* required pointer is NULL                       */
     BPK_ERR_ALIGN = -4,     /* pointer or stride alignment not met            */
@@ -69,7 +72,8 @@ BPK_API int bpk_shutdown(void);
 /* ---- layout: replaces the descriptor half of pack_q4k / pack_q6k ----------
  * runtime/gguf_loader.cpp:359-379, :403-424; struct KQuantPacked
  * (runtime/gguf_loader.h:108-113).  n_blocks = ceil(K/256);
- * row_stride_words = 36*n_blocks (Q4_K) or ceil(210*n_blocks/4) (Q6_K). */
+ * row_stride_words = 36*n_blocks (Q4_K), 44*n_blocks (Q5_K, pack_q5k,
+ * gguf_loader.cpp:381-401) or ceil(210*n_blocks/4) (Q6_K). */
 BPK_API int bpk_kq_layout(int type, uint32_t K, uint32_t *n_blocks,
                           uint32_t *row_stride_words);
 

@@ -71,6 +71,7 @@ void kqo_q4k_scale_min(const uint8_t s[12], int sb, uint32_t *sc, uint32_t *mn)
 uint32_t kqo_block_bytes(int type)
 {
     if (type == KQO_TYPE_Q4_K) return KQO_Q4K_BLOCK_BYTES;
+    if (type == KQO_TYPE_Q5_K) return KQO_Q5K_BLOCK_BYTES;   /* pack_q5k, runtime/gguf_loader.cpp:381-401 */
     if (type == KQO_TYPE_Q6_K) return KQO_Q6K_BLOCK_BYTES;
     return 0;
 }
@@ -131,6 +132,35 @@ static void q4k_block(const uint8_t *blk, float *out)
     }
 }
 
+/* runtime/gguf_loader.cpp:497-536.  d, dmin fp16 @0, 2; 12 scale bytes @4 (the Q4_K packing); 32
+ * bytes of fifth bits @16 (bit sb of byte i belongs to element i of sub-block sb); 128 nibble bytes
+ * @48.  out = (d*sc)*(nibble | bit<<4) - (dmin*mn), each product rounded to fp32 in that order. */
+static void q5k_block(const uint8_t *blk, float *out)
+{
+    uint16_t hd, hm;
+    memcpy(&hd, blk, 2);
+    memcpy(&hm, blk + 2, 2);
+    const float d = kqo_fp16_to_f32(hd);
+    const float dmin = kqo_fp16_to_f32(hm);
+    const uint8_t *scales = blk + 4;
+    const uint8_t *qh = blk + 16;
+    const uint8_t *qs = blk + 48;
+
+    for (int sb = 0; sb < 8; ++sb) {
+        uint32_t sc_u, mn_u;
+        kqo_q4k_scale_min(scales, sb, &sc_u, &mn_u);
+        const float sc = d * (float)sc_u;
+        const float mn = dmin * (float)mn_u;
+        const uint8_t *q = qs + (sb >> 1) * 32;
+        const int shift = (sb & 1) * 4;
+        for (int i = 0; i < 32; ++i) {
+            const uint32_t nib = ((uint32_t)q[i] >> shift) & 15u;
+            const uint32_t hi = ((uint32_t)qh[i] >> sb) & 1u;
+            out[sb * 32 + i] = sc * (float)(nib | (hi << 4)) - mn;
+        }
+    }
+}
+
 /* runtime/gguf_loader.cpp:537-571.  out = d * (float)scale * (float)(q-32),
  * evaluated left to right. */
 static void q6k_block(const uint8_t *blk, float *out)
@@ -164,6 +194,9 @@ static void dequant_row_bytes(int type, const uint8_t *row, uint32_t nb, float *
     if (type == KQO_TYPE_Q4_K) {
         for (uint32_t b = 0; b < nb; ++b)
             q4k_block(row + (size_t)b * KQO_Q4K_BLOCK_BYTES, out + (size_t)b * KQO_QK_K);
+    } else if (type == KQO_TYPE_Q5_K) {
+        for (uint32_t b = 0; b < nb; ++b)
+            q5k_block(row + (size_t)b * KQO_Q5K_BLOCK_BYTES, out + (size_t)b * KQO_QK_K);
     } else {
         for (uint32_t b = 0; b < nb; ++b)
             q6k_block(row + (size_t)b * KQO_Q6K_BLOCK_BYTES, out + (size_t)b * KQO_QK_K);

@@ -58,10 +58,12 @@ extern "C" {
 
 /* GGUF tensor type codes, runtime/gguf_loader.h:29-30 */
 #define KQO_TYPE_Q4_K 12
+#define KQO_TYPE_Q5_K 13
 #define KQO_TYPE_Q6_K 14
 
 #define KQO_QK_K 256
 #define KQO_Q4K_BLOCK_BYTES 144
+#define KQO_Q5K_BLOCK_BYTES 176
 #define KQO_Q6K_BLOCK_BYTES 210
 
 /* ---- scalar pieces ------------------------------------------------------ */

@@ -23,6 +23,7 @@ int bpref_pack(int type, const void* raw, uint32_t N, uint32_t K, uint32_t* out,
 {
     KQuantPacked p;
     if (type == (int)GGUF_TYPE_Q4_K) p = pack_q4k(raw, N, K);
+    else if (type == (int)GGUF_TYPE_Q5_K) p = pack_q5k(raw, N, K);
     else if (type == (int)GGUF_TYPE_Q6_K) p = pack_q6k(raw, N, K);
     else return -1;
     if (n_blocks) *n_blocks = p.nBlocks;
@@ -33,7 +34,7 @@ int bpref_pack(int type, const void* raw, uint32_t N, uint32_t K, uint32_t* out,
 
 int bpref_dequant(int type, const void* raw, float* out, uint32_t N, uint32_t K)
 {
-    if (type != (int)GGUF_TYPE_Q4_K && type != (int)GGUF_TYPE_Q6_K) return -1;
+    if (type != (int)GGUF_TYPE_Q4_K && type != (int)GGUF_TYPE_Q5_K && type != (int)GGUF_TYPE_Q6_K) return -1;
     dequant_kquant(raw, out, N, K, (GGUFType)type);
     return 0;
 }

@@ -1,4 +1,4 @@
-"""Writes tests/golden/recipes.npz: the reference's nine Q4_K/Q6_K known-answer
+"""Writes tests/golden/recipes.npz: the reference's eleven Q4_K/Q5_K/Q6_K known-answer
 cases with inputs regenerated from their closed forms and expected outputs
 computed by the COMPILED REFERENCE (oracle/_ref/libbp_ref.so -> dequant_kquant)
 followed by the test-suite's sequential fp32 dot, written here as a plain

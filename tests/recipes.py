@@ -1,11 +1,11 @@
-"""The reference's nine Q4_K / Q6_K known-answer recipes, regenerated from their
-closed forms (runtime/tests/kernel_test.cpp:1678-1748).  Inputs only: expected
+"""The reference's eleven Q4_K / Q5_K / Q6_K known-answer recipes, regenerated from
+their closed forms (runtime/tests/kernel_test.cpp:1669-1748).  Inputs only: expected
 values come from the oracle or from the golden fixture, never from here."""
 from __future__ import annotations
 
 import numpy as np
 
-Q4_K, Q6_K = 12, 14
+Q4_K, Q5_K, Q6_K = 12, 13, 14
 
 
 def _h(kqo, f):
@@ -32,6 +32,17 @@ def _q4k(kqo, N, NB, dfun, dmfun, bfun):
             raw[n, b, 0:2] = np.frombuffer(np.uint16(_h(kqo, dfun(n, b))).tobytes(), np.uint8)
             raw[n, b, 2:4] = np.frombuffer(np.uint16(_h(kqo, dmfun(n, b))).tobytes(), np.uint8)
             i = np.arange(4, 144)
+            raw[n, b, 4:] = (bfun(n, b, i) & 255).astype(np.uint8)
+    return raw.reshape(N, -1)
+
+
+def _q5k(kqo, N, NB, dfun, dmfun, bfun):
+    raw = np.zeros((N, NB, 176), dtype=np.uint8)
+    for n in range(N):
+        for b in range(NB):
+            raw[n, b, 0:2] = np.frombuffer(np.uint16(_h(kqo, dfun(n, b))).tobytes(), np.uint8)
+            raw[n, b, 2:4] = np.frombuffer(np.uint16(_h(kqo, dmfun(n, b))).tobytes(), np.uint8)
+            i = np.arange(4, 176)
             raw[n, b, 4:] = (bfun(n, b, i) & 255).astype(np.uint8)
     return raw.reshape(N, -1)
 
@@ -101,6 +112,16 @@ def build(kqo):
     # q4k_matmul_batched8_reference :1744
     R["q4k_matmul_batched8"] = dict(type=Q4_K, M=9, N=9, K=512, seed=5151, bias_on=True,
                                     raw=_q4k(kqo, 9, 2, d2, dm2, q4b), ref="kernel_test.cpp:1744")
+
+    # q5k_matmul_reference :1669
+    R["q5k_matmul"] = dict(
+        type=Q5_K, M=1, N=8, K=256, seed=4242, bias_on=False,
+        raw=_q5k(kqo, 8, 1, d1, lambda n, b: _f(0.01, _mul(0.0005, n)),
+                 lambda n, b, i: n * 37 + i * 13 + 7), ref="kernel_test.cpp:1669")
+    # q5k_matmul_batched4_reference :1732
+    R["q5k_matmul_batched4"] = dict(
+        type=Q5_K, M=5, N=9, K=512, seed=4949, bias_on=True,
+        raw=_q5k(kqo, 9, 2, d2, dm2, lambda n, b, i: n * 29 + b * 11 + i * 19), ref="kernel_test.cpp:1732")
 
     for name, r in R.items():
         if "seed" in r:

@@ -37,11 +37,12 @@ def test_layout_matches_oracle(kqo, type_, K):
 
 def test_layout_rejects_unknown_type():
     with pytest.raises(capi.BpkError) as e:
-        capi.layout(13, 256)   # Q5_K is outside this library
+        capi.layout(11, 256)   # Q3_K is outside this library
     assert e.value.code == -1
+    assert capi.layout(13, 512) == (2, 88)   # Q5_K: 44 words per block
 
 
-@pytest.mark.parametrize("type_,N,K", [(Q4_K, 5, 512), (Q6_K, 7, 768), (Q6_K, 3, 256)])
+@pytest.mark.parametrize("type_,N,K", [(Q4_K, 5, 512), (Q6_K, 7, 768), (Q6_K, 3, 256), (13, 4, 768)])
 def test_pack_host_matches_oracle(kqo, type_, N, K):
     from backpack_amd import kquant  # imports torch; no GPU needed for the packer
     raw = synth.make_raw(type_, N, K, seed=3)

@@ -55,6 +55,8 @@ ONE_LAUNCH = [
     (Q6_K, 1, 50, 28672, GELU, False, False),
     (Q6_K, 2, 40, 2048, GELU, True, True),
     (Q6_K, 1, 33, 768, NORM, True, False),
+    (13, 1, 200, 4096, NORM, True, False),        # Q5_K
+    (13, 2, 64, 1024, SILU, True, True),
 ]
 
 

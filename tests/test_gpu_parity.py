@@ -10,7 +10,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
-Q4_K, Q6_K = 12, 14
+Q4_K, Q5_K, Q6_K = 12, 13, 14
 
 
 @pytest.fixture(scope="module")
@@ -28,7 +28,7 @@ def _say(*a):
 
 
 # ---- dequantised weights: bit-exact ---------------------------------------------
-@pytest.mark.parametrize("type_", [Q4_K, Q6_K])
+@pytest.mark.parametrize("type_", [Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("N,K", [(1, 256), (33, 768), (64, 4096), (5, 14336)])
 def test_dequant_bit_exact(gpu, kqo, type_, N, K):
     from backpack_amd import kquant
@@ -63,9 +63,10 @@ def test_dequant_full_size_row_checksum(gpu, kqo):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-# ---- the reference's nine known-answer cases --------------------------------------
+# ---- the reference's eleven known-answer cases --------------------------------------
 RECIPES = ["q4k_matmul", "q4k_matmul_128", "q6k_matmul", "q6k_gather", "q6k_matmul_wide",
-           "q6k_gather_batched", "q4k_matmul_batched4", "q6k_matmul_batched4", "q4k_matmul_batched8"]
+           "q6k_gather_batched", "q4k_matmul_batched4", "q6k_matmul_batched4", "q4k_matmul_batched8",
+           "q5k_matmul", "q5k_matmul_batched4"]
 
 
 @pytest.mark.parametrize("name", RECIPES)
@@ -88,6 +89,44 @@ def test_reference_recipe(gpu, kqo, name, family):
         capi.force_kernel(0)
     bad, worst = kqo.assert_close(got, g[f"{name}/expected"], atol, rtol)
     assert bad == 0, f"{name}: {bad} elements outside atol={atol} rtol={rtol}, worst excess {worst}"
+
+
+# ---- Q5_K: packers, rows and the fp32 matmul (generic kernel) ------------------------
+@pytest.mark.parametrize("M,N,K,kernel", [(1, 300, 4096, "gemv_stream"), (2, 64, 768, "gemv_stream"),
+                                          (1, 4096, 4096, "gemv_stream"), (2, 6144, 4096, "gemv_stream"),
+                                          (1, 77, 256, "gemv_stream"), (1, 500, 3072, "gemv_stream"),
+                                          (5, 130, 2048, "generic"), (17, 40, 512, "generic"),
+                                          (1, 1000, 14336, "generic")])
+def test_q5k_matmul_vs_oracle(gpu, kqo, M, N, K, kernel):
+    from backpack_amd import capi, kquant
+    _say("q5k matmul", M, N, K)
+    raw, packed, w = gpu.make_weight(Q5_K, N, K, seed=M + N)
+    X = np.random.default_rng(K).standard_normal((M, K)).astype(np.float32)
+    bias = np.random.default_rng(1).standard_normal(N).astype(np.float32)
+    y = kquant.matmul(gpu.dev(X), w, bias=gpu.dev(bias)).cpu().numpy()
+    assert capi.last_kernel() == kernel
+    gpu.check_matmul(kqo, Q5_K, y, X, packed, N, K, bias=bias, label=f"q5k {M}x{N}x{K}")
+    if kernel != "generic":      # and the generic kernel on the same inputs
+        capi.force_kernel(1)
+        try:
+            y1 = kquant.matmul(gpu.dev(X), w, bias=gpu.dev(bias)).cpu().numpy()
+        finally:
+            capi.force_kernel(0)
+        gpu.check_matmul(kqo, Q5_K, y1, X, packed, N, K, bias=bias, label=f"q5k generic {M}x{N}x{K}")
+
+
+def test_q5k_is_refused_where_no_kernel_serves_it(gpu):
+    from backpack_amd import capi, kquant
+    raw, packed, w = gpu.make_weight(Q5_K, 64, 512, seed=1)
+    import torch
+    xb = torch.zeros(256, 512, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(capi.BpkError) as e:
+        kquant.matmul(xb, w)
+    assert e.value.code == -1
+    idx = torch.zeros(2, 2, dtype=torch.int32, device="cuda")
+    with pytest.raises(capi.BpkError) as e:
+        kquant.moe_matmul(torch.zeros(2, 512, device="cuda"), w, idx, 4)
+    assert e.value.code == -1
 
 
 # ---- matmul against the oracle ------------------------------------------------------

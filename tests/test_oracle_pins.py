@@ -9,7 +9,7 @@ import pytest
 from backpack_amd import synth
 
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
-Q4_K, Q6_K = 12, 14
+Q4_K, Q5_K, Q6_K = 12, 13, 14
 
 
 # ---- fp16 -> fp32 ----------------------------------------------------------
@@ -79,6 +79,39 @@ def test_q4k_dequant_is_single_rounding_of_exact_value(kqo):
     assert np.array_equal(got, exact.astype(np.float32))
 
 
+def test_q5k_dequant_is_single_rounding_of_exact_value(kqo):
+    """d*sc*q has at most 11 + 6 + 5 = 22 significant bits, so as for Q4_K the only rounding is the
+    subtraction of dmin*mn."""
+    rng = np.random.default_rng(13)
+    f = synth.q5k_fields(rng, 48, 4)
+    raw = synth.q5k_encode(*f).reshape(48, -1)
+    got = kqo.dequant(Q5_K, raw, 48, 1024)
+    exact = synth.q4k_decode_f64(*f)            # same formula, q now five bits
+    assert np.array_equal(got, exact.astype(np.float32))
+
+
+def test_q5k_element_order_and_fifth_bit_bruteforce(kqo):
+    """One element set to 17 (nibble 1, fifth bit 1), then to 16 (fifth bit alone): it must land in
+    out[e] with that value, and nowhere else."""
+    for e in range(256):
+        for v in (17, 16, 15):
+            d = np.array([[1.0]], dtype=np.float16)
+            z = np.array([[0.0]], dtype=np.float16)
+            sc = np.ones((1, 1, 8), dtype=np.uint8)
+            mn = np.zeros((1, 1, 8), dtype=np.uint8)
+            q = np.zeros((1, 1, 256), dtype=np.uint8)
+            q[0, 0, e] = v
+            blk = synth.q5k_encode(d, z, sc, mn, q)
+            # the layout itself, independent of the encoder: fifth bits at 16 + i, bit sb; nibbles at 48 + 32*(sb/2) + i
+            sb, i = e // 32, e % 32
+            assert blk[0, 0, 16 + i] == ((v >> 4) << sb)
+            assert blk[0, 0, 48 + 32 * (sb // 2) + i] == ((v & 15) << (4 * (sb & 1)))
+            out = kqo.dequant(Q5_K, blk.reshape(1, -1), 1, 256)[0]
+            want = np.zeros(256, dtype=np.float32)
+            want[e] = float(v)
+            assert np.array_equal(out, want)
+
+
 def test_q6k_dequant_is_exact(kqo):
     rng = np.random.default_rng(4)
     f = synth.q6k_fields(rng, 48, 4)
@@ -143,7 +176,7 @@ def test_golden_random_blocks(kqo):
 
 def test_differential_vs_compiled_reference(kqref):
     kqo = kqref
-    for type_, (N, K) in ((Q4_K, (33, 1280)), (Q6_K, (33, 1280))):
+    for type_, (N, K) in ((Q4_K, (33, 1280)), (Q5_K, (33, 1280)), (Q6_K, (33, 1280))):
         raw = synth.make_raw(type_, N, K, seed=11)
         assert np.array_equal(kqo.dequant(type_, raw, N, K).view(np.uint32),
                               kqo.ref_dequant(type_, raw, N, K).view(np.uint32))
@@ -156,6 +189,7 @@ def test_differential_vs_compiled_reference(kqref):
 @pytest.mark.parametrize("K,q4,q6", [(4096, 576, 840), (14336, 2016, 2940), (768, 108, 158),
                                      (2048, 288, 420), (256, 36, 53)])
 def test_row_stride_rule(kqo, K, q4, q6):
+    assert kqo.row_stride_words(Q5_K, K) == 44 * (K // 256) == synth.row_stride_words(Q5_K, K)
     assert kqo.row_stride_words(Q4_K, K) == q4 == synth.row_stride_words(Q4_K, K)
     assert kqo.row_stride_words(Q6_K, K) == q6 == synth.row_stride_words(Q6_K, K)
 
@@ -223,12 +257,12 @@ def test_matmul_bf16_widens_exactly(kqo):
     assert np.array_equal(kqo.matmul_bf16(Q6_K, bits, pk, N, K), kqo.matmul(Q6_K, xw, pk, N, K))
 
 
-# ---- the reference's nine recipes -------------------------------------------
+# ---- the reference's eleven recipes -------------------------------------------
 def test_reference_recipes_against_golden(kqo):
     import recipes
     g = np.load(os.path.join(GOLD, "recipes.npz"))
     R = recipes.build(kqo)
-    assert len(R) == 9
+    assert len(R) == 11
     for name, r in R.items():
         type_, M, N, K, nb, rs = (int(v) for v in g[f"{name}/desc"])
         assert np.array_equal(r["raw"], g[f"{name}/raw"]), name      # closed-form bytes
