@@ -32,10 +32,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 METRIC = "Q4_K M=1 matvec HBM GB/s (% of peak); M=2048 dequant-GEMM TFLOPS (% MFMA)"
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE (profiles/decode_gemv_hbm_traffic_pmc.txt): FETCH_SIZE 32383.4
+# WRITE_SIZE (profiles/decode_gemv_hbm_traffic_pmc.txt): FETCH_SIZE 32386.8
 # x 2.000 KiB + WRITE_SIZE 224.0 x 1.000 KiB, the factors being what the same
 # counters read for a 256 MiB copy kernel.
-MEASURED_TRAFFIC_BYTES = 66550579
+MEASURED_TRAFFIC_BYTES = 66557583
 
 
 def parse():
@@ -238,7 +238,7 @@ def main():
     dom_bytes = synth.weight_bytes(dom_w.type, dom_w.N, dom_w.K) + (dom_w.K + dom_w.N) * 4
     dom_gbs = dom_bytes / (dsec / launches) / 1e9
     roofline = {
-        "kernel": f"kq::q4k_stream_kernel<2, 4, 4> ({capi.last_kernel()}; gate|up 28672x4096 Q4_K, M=1)",
+        "kernel": f"kq::q4k_stream_kernel<2, 4, 4, 1, kq::StreamDense, false> ({capi.last_kernel()}; gate|up 28672x4096 Q4_K, M=1)",
         "bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
         "bytes_per_launch": dom_bytes, "us_per_launch": round(dsec / launches * 1e6, 3),
