@@ -316,18 +316,22 @@ struct Q4Slot {
     }
 };
 
-// P passes of 8 superblocks cover a row (n_blocks <= 8 * P); D rows in flight; MT tokens.
-template <int P, int NW, int D, int MT, typename PT, bool Q5 = false>
-__global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
+// P passes of 8 superblocks cover a row (n_blocks <= 8 * P) or, with KW > 1, a wave's K slice of it
+// (n_blocks <= 8 * P * KW); D rows in flight; MT tokens.  KW == 1: a workgroup is NW independent waves,
+// each with rows of its own.  KW > 1: the KW waves of a workgroup walk the same rows, one K slice each,
+// and their sums meet in LDS once per 64 rows (the form of the Q6_K kernel below).
+template <int P, int NW, int D, int MT, typename PT, bool Q5 = false, int KW = 1>
+__global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT p)
 {
     stream_select_pair(p);
+    __shared__ float part[KW > 1 ? KW : 1][MT][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t gw = blockIdx.x * NW + wave;
+    const uint32_t gw = KW > 1 ? blockIdx.x : blockIdx.x * NW + wave;
     // rows gw, gw + stride, ...: at any moment the waves of the grid read
     // consecutive rows, one contiguous stream across the memory channels
-    const uint32_t stride = gridDim.x * NW;
-    if (gw >= p.N) return;
+    const uint32_t stride = KW > 1 ? gridDim.x : gridDim.x * NW;
+    if (gw >= p.N) return;   // KW > 1: the whole workgroup
     const uint32_t n_rows = (p.N - gw + stride - 1u) / stride;
     const uint32_t bl = lane >> 3, j = lane & 7u, g = j >> 1, h = j & 1u;
     const bool sel_hi = g >= 2u;
@@ -342,7 +346,7 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
         constexpr int PRO = decltype(pro)::value;
 #pragma unroll
         for (int pass = 0; pass < P; ++pass) {
-            uint32_t b = pass * 8u + bl;
+            uint32_t b = ((KW > 1 ? wave * P : 0u) + pass) * 8u + bl;
             const bool valid = b < p.n_blocks;
             b = valid ? b : p.n_blocks - 1u;
             hoff[pass] = b * BLOCK;
@@ -375,7 +379,15 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
 #pragma unroll
                     for (int i = 0; i < 16; ++i)
                         ss = __builtin_fmaf(xlo[pass][t][i], xlo[pass][t][i], __builtin_fmaf(xhi[pass][t][i], xhi[pass][t][i], ss));
-                const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)p.K + stream_eps(p));
+                ss = wave_sum(ss);
+                if (KW > 1) {   // the slices' sums of squares meet in LDS
+                    if (lane == 0) part[wave][t][0] = ss;
+                    __syncthreads();
+                    ss = part[0][t][0];
+#pragma unroll
+                    for (int w = 1; w < KW; ++w) ss += part[w][t][0];
+                }
+                const float rstd = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
 #pragma unroll
                 for (int pass = 0; pass < P; ++pass) {
                     const float* wp = stream_norm_w(p) + hoff[pass] / BLOCK * KQ_QK + 64u * g + 16u * h;
@@ -386,6 +398,7 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
                     }
                 }
             }
+            if (KW > 1) __syncthreads();   // part is reused by the row loop
 #pragma unroll
             for (int pass = 0; pass < P; ++pass)
 #pragma unroll
@@ -439,17 +452,29 @@ __global__ __launch_bounds__(64 * NW) void q4k_stream_kernel(PT p)
                 }
             }
         }
-        if (lane < cnt) {
+        if (KW > 1) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) part[wave][t][lane] = res[t];
+            __syncthreads();
+        }
+        if ((KW == 1 || wave == 0) && lane < cnt) {
             const uint32_t r = gw + (c0 + lane) * stride;
             const float bias = p.bias ? p.bias[r] : 0.0f;
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 const size_t at = (size_t)t * p.ldy + p.y_offset + r;
-                float y = res[t] + bias;
+                float y = res[t];
+                if (KW > 1) {
+                    y = part[0][t][lane];
+#pragma unroll
+                    for (int w = 1; w < KW; ++w) y += part[w][t][lane];
+                }
+                y += bias;
                 if constexpr (PT::kFused) y += stream_residual(p) ? stream_residual(p)[at] : 0.0f;
                 p.Y[at] = y;
             }
         }
+        if (KW > 1) __syncthreads();
     }
     asm volatile("s_waitcnt vmcnt(0)");   // the ring's last refills land before the wave ends
 }
@@ -740,7 +765,11 @@ bool gemv_stream_supported(const MatmulArgs& a)
     if (a.n_blocks < 1) return false;
     if (a.type == KQ_TYPE_Q4_K || a.type == KQ_TYPE_Q5_K) {
         if (a.type == KQ_TYPE_Q5_K && a.expert_idx) return false;
-        if (a.n_blocks > 16) return false;
+        // longer rows are cut into K slices: dense and fused calls only, and the two-token kernel for
+        // the longest rows has no registers for Q5_K's third load or the fused forms
+        if (a.n_blocks > 16 && a.expert_idx) return false;
+        if (a.n_blocks > 112) return false;
+        if (a.n_blocks > 56 && a.M == 2 && (a.type == KQ_TYPE_Q5_K || a.pro != 0 || a.residual)) return false;
         if (((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u)) return false;
         return true;
     }
@@ -772,6 +801,14 @@ static void launch_q4k_one(dim3 grid, hipStream_t s, const PT& p)
 {
     constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && D != 2) || (Q5 && (PT::kGrouped || D > 2));
     if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT, Q5>), grid, dim3(64 * NW), 0, s, p);
+}
+
+// Rows longer than 16 superblocks: K slices over KW waves, two rows in flight, dense and fused calls.
+template <int P, int KW, int MT, typename PT, bool Q5>
+static void launch_q4k_sliced(dim3 grid, hipStream_t s, const PT& p)
+{
+    constexpr bool absent = PT::kGrouped || (P == 2 && KW == 7 && MT == 2 && (PT::kFused || Q5));
+    if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, 1, 2, MT, PT, Q5, KW>), grid, dim3(64 * KW), 0, s, p);
 }
 
 template <typename PT>
@@ -812,12 +849,32 @@ static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, h
 #undef KQ_STREAM6_MT
         return hipGetLastError();
     }
+    const bool q5 = a.type == KQ_TYPE_Q5_K;
+    if (a.n_blocks > 16u) {
+        // the Q6_K kernel's K slices: 4 waves of 8 superblocks up to 32, else 7 waves of 8 or 16
+        const uint32_t nb = a.n_blocks;
+        const int kw = nb <= 32u ? 4 : 7;
+        const int pp = nb <= 56u ? 1 : 2;
+        uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 2u, t.splits);
+        const dim3 grid(wgs, 1, 1);
+#define KQ_STREAM4S(P, KW) \
+    do { \
+        if (q5 && two) launch_q4k_sliced<P, KW, 2, PT, true>(grid, s, p); \
+        else if (q5) launch_q4k_sliced<P, KW, 1, PT, true>(grid, s, p); \
+        else if (two) launch_q4k_sliced<P, KW, 2, PT, false>(grid, s, p); \
+        else launch_q4k_sliced<P, KW, 1, PT, false>(grid, s, p); \
+    } while (0)
+        if (kw == 4) KQ_STREAM4S(1, 4);
+        else if (pp == 1) KQ_STREAM4S(1, 7);
+        else KQ_STREAM4S(2, 7);
+#undef KQ_STREAM4S
+        return hipGetLastError();
+    }
     constexpr int NW = 4;
     // a Q4_K workgroup is NW independent waves, each with its own rows
     uint32_t wgs = t.splits > 0 ? ((a.N + (uint32_t)t.splits - 1u) / (uint32_t)t.splits + NW - 1u) / NW
                                 : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
     wgs = (wgs + pairs * twins - 1u) / (pairs * twins);
-    const bool q5 = a.type == KQ_TYPE_Q5_K;
     int depth = PT::kFused ? 2 : t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
     if (q5 && depth > 2) depth = 2;
     const dim3 grid(wgs, pairs, twins);

@@ -220,8 +220,8 @@ BPK_API int bpk_kq_matmul(int type, const float *X, const void *W,
  * silu(g) = g / (1 + exp(-g)); gelu_tanh(g) = 0.5 g (1 + tanh(0.7978845608 (g +
  * 0.044715 g^3))).  residual may be NULL (= zeros) and may be Y itself (the
  * in-place add).  M <= 2 with rows the decode kernel holds in registers
- * (Q4_K: K <= 4096; Q6_K: K <= 28672 for one token, K <= 14336 for two;
- * N <= 32768) is one launch and needs no workspace.  Other shapes run the same function as prologue, matmul and add
+ * (K <= 28672 for one token, K <= 14336 for two; N <= 32768) is one launch
+ * and needs no workspace.  Other shapes run the same function as prologue, matmul and add
  * launches through `workspace` (device memory, 16-byte aligned, at least
  * bpk_kq_matmul_fused_workspace_bytes(M, N, K) bytes) and fail with
  * BPK_ERR_WORKSPACE without it. */

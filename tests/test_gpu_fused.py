@@ -55,7 +55,12 @@ ONE_LAUNCH = [
     (Q6_K, 1, 50, 28672, GELU, False, False),
     (Q6_K, 2, 40, 2048, GELU, True, True),
     (Q6_K, 1, 33, 768, NORM, True, False),
+    (Q4_K, 1, 100, 14336, SILU, True, False),     # Q4_K long rows: K slices over 7 waves
+    (Q4_K, 2, 90, 14336, NORM, True, True),       # ... the norm's sum of squares across the slices
+    (Q4_K, 1, 70, 8192, GELU, False, False),      # ... 4 slices
+    (Q4_K, 1, 40, 28672, NORM, False, False),     # ... 7 slices of 16 superblocks
     (13, 1, 200, 4096, NORM, True, False),        # Q5_K
+    (13, 1, 120, 14336, SILU, True, False),
     (13, 2, 64, 1024, SILU, True, True),
 ]
 
@@ -95,7 +100,7 @@ def test_fused_residual_in_place_and_same_as_separate_launches(gpu, kqo):
 
 
 WORKSPACE = [
-    (Q4_K, 1, 100, 14336, SILU, True),     # Q4_K rows longer than the decode kernel's registers
+    (Q4_K, 1, 60, 32768, SILU, True),      # rows longer than the decode kernel's K slices hold
     (Q4_K, 5, 96, 2048, NORM, True),       # more than two tokens
     (Q6_K, 16, 64, 1024, GELU, False),
     (Q6_K, 2, 48, 28672, NORM, True),      # the two-token long-row kernel carries no norm

@@ -96,7 +96,9 @@ def test_reference_recipe(gpu, kqo, name, family):
                                           (1, 4096, 4096, "gemv_stream"), (2, 6144, 4096, "gemv_stream"),
                                           (1, 77, 256, "gemv_stream"), (1, 500, 3072, "gemv_stream"),
                                           (5, 130, 2048, "generic"), (17, 40, 512, "generic"),
-                                          (1, 1000, 14336, "generic")])
+                                          (1, 1000, 14336, "gemv_stream"), (2, 300, 8192, "gemv_stream"),
+                                          (1, 200, 28672, "gemv_stream"), (2, 200, 28672, "generic"),
+                                          (1, 50, 32768, "generic")])
 def test_q5k_matmul_vs_oracle(gpu, kqo, M, N, K, kernel):
     from backpack_amd import capi, kquant
     _say("q5k matmul", M, N, K)
@@ -143,7 +145,13 @@ SHAPES = [
     (Q4_K, 1, 100, 256),        # ragged N, single block
     (Q4_K, 1, 333, 3072),       # 12 blocks: the second pass of the lanes-along-K kernel is partial
     (Q4_K, 1, 6144, 4096),      # fused q|k|v
-    (Q4_K, 1, 64, 14336),       # long rows
+    (Q4_K, 1, 64, 14336),       # long rows: K slices over 7 waves
+    (Q4_K, 2, 500, 14336),
+    (Q4_K, 1, 300, 8192),       # ... over 4 waves
+    (Q4_K, 2, 100, 6400),       # ... 25 superblocks: the last slice is partial
+    (Q4_K, 1, 90, 28672),       # ... 7 slices of two passes
+    (Q4_K, 2, 90, 28672),
+    (Q4_K, 1, 40, 32768),       # beyond the slices: row-per-lane kernel
     (Q4_K, 2, 200, 1024),
     (Q4_K, 3, 130, 2048),
     (Q4_K, 4, 65, 512),
