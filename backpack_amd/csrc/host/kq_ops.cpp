@@ -22,6 +22,7 @@ static KQuantPacked pack(GGUFType type, const void* raw, uint32_t N, uint32_t K)
 }
 
 KQuantPacked pack_q4k(const void* raw, uint32_t N, uint32_t K) { return pack(GGUF_TYPE_Q4_K, raw, N, K); }
+KQuantPacked pack_q5k(const void* raw, uint32_t N, uint32_t K) { return pack(GGUF_TYPE_Q5_K, raw, N, K); }
 KQuantPacked pack_q6k(const void* raw, uint32_t N, uint32_t K) { return pack(GGUF_TYPE_Q6_K, raw, N, K); }
 
 KQuantPacked fuseKQ(const std::vector<const KQuantPacked*>& parts)
@@ -92,5 +93,105 @@ int gatherKQ(GGUFType type, const GPUBuffer& W, uint32_t rowStrideWords, const G
     if (rc != BPK_OK) fprintf(stderr, "[gatherKQ] %s\n", bpk_last_error());
     return rc;
 }
+
+int KQFusedDispatch::run(void* stream) const
+{
+    const KQDispatch& d = base;
+    bpk_kq_fusion f{prologue, (const float*)NormW.ptr(), eps, (const float*)Residual.ptr()};
+    const int rc = bpk_kq_matmul_fused((int)d.type, (const float*)d.X.ptr(), d.W.ptr(), (const float*)d.Bias.ptr(),
+                                       (float*)d.Y.ptr(), d.M, d.P.v[1], d.P.v[0], d.P.v[2], d.P.v[3], d.P.v[4], &f,
+                                       Workspace.ptr(), Workspace.handle ? Workspace.size - Workspace.offset : 0, stream);
+    if (rc != BPK_OK) fprintf(stderr, "%s: %s\n", d.name.c_str(), bpk_last_error());
+    return rc;
+}
+
+GGUFFile::~GGUFFile() { bpk_gguf_close(g_); }
+
+bool GGUFFile::open(const std::string& path)
+{
+    bpk_gguf_close(g_);
+    g_ = nullptr;
+    tensors.clear();
+    if (bpk_gguf_open(path.c_str(), &g_) != BPK_OK) {
+        fprintf(stderr, "GGUFFile::open: %s\n", bpk_last_error());
+        return false;
+    }
+    bpk_gguf_info(g_, &version, &n_tensors, nullptr, &data_offset);
+    tensors.resize((size_t)n_tensors);
+    for (uint64_t i = 0; i < n_tensors; ++i) {
+        bpk_gguf_tensor t;
+        bpk_gguf_tensor_at(g_, i, &t);
+        GGUFTensorInfo& o = tensors[(size_t)i];
+        o.name = t.name;
+        o.shape.assign(t.dims, t.dims + t.n_dims);
+        o.type = t.type;
+        o.offset = t.offset;
+        o.data = t.data;
+        o.bytes = t.bytes;
+    }
+    return true;
+}
+
+const GGUFTensorInfo* GGUFFile::find(const std::string& name) const
+{
+    for (const auto& t : tensors)
+        if (t.name == name) return &t;
+    return nullptr;
+}
+
+std::string GGUFFile::getString(const std::string& key, const std::string& def) const
+{
+    if (!g_ || bpk_gguf_key_type(g_, key.c_str()) != 8) return def;
+    size_t n = 0;
+    bpk_gguf_get_string(g_, key.c_str(), nullptr, 0, &n);
+    std::string s(n, '\0');
+    std::vector<char> buf(n + 1);
+    bpk_gguf_get_string(g_, key.c_str(), buf.data(), n + 1, nullptr);
+    s.assign(buf.data(), n);
+    return s;
+}
+
+uint32_t GGUFFile::getU32(const std::string& key, uint32_t def) const
+{
+    uint32_t v = def;
+    if (g_) bpk_gguf_get_u32(g_, key.c_str(), def, &v);
+    return v;
+}
+
+float GGUFFile::getFloat(const std::string& key, float def) const
+{
+    float v = def;
+    if (g_) bpk_gguf_get_f32(g_, key.c_str(), def, &v);
+    return v;
+}
+
+bool GGUFFile::getBool(const std::string& key, bool def) const
+{
+    int v = def;
+    if (g_) bpk_gguf_get_bool(g_, key.c_str(), def, &v);
+    return v != 0;
+}
+
+bool GGUFFile::hasKey(const std::string& key) const { return g_ && bpk_gguf_has_key(g_, key.c_str()); }
+
+bool GGUFFile::loadKQWeight(const std::vector<std::string>& names, GPUBuffer& W, KQuantPacked& desc,
+                            bpk_weight** owner) const
+{
+    std::vector<const char*> c;
+    for (const auto& n : names) c.push_back(n.c_str());
+    if (!g_ || bpk_gguf_weight_create(g_, c.data(), (uint32_t)c.size(), owner) != BPK_OK) {
+        fprintf(stderr, "GGUFFile::loadKQWeight: %s\n", g_ ? bpk_last_error() : "file not open");
+        return false;
+    }
+    bpk_weight_desc d;
+    bpk_weight_describe(*owner, &d);
+    W = GPUBuffer{d.data, d.bytes, 0};
+    desc = KQuantPacked{};
+    desc.N = d.N; desc.K = d.K; desc.rowStrideWords = d.row_stride_words; desc.nBlocks = d.n_blocks;
+    desc.type = (GGUFType)d.type;
+    return true;
+}
+
+void releaseWeight(bpk_weight* owner) { bpk_weight_destroy(owner); }
 
 }  // namespace bp

@@ -1,7 +1,8 @@
 // kq_ops.h — C++ host layer over the C ABI, shaped like the reference's k-quant
 // operator interface so that a ModelRunner-style caller can switch to it:
 //
-//   KQuantPacked, pack_q4k, pack_q6k     runtime/gguf_loader.h:108-124
+//   KQuantPacked, pack_q4k/q5k/q6k       runtime/gguf_loader.h:108-124
+//   GGUFFile and its getters             runtime/gguf_loader.h:49-86
 //   GPUBuffer {handle, size, offset}     runtime/gpu_context.h:47-51 (non-owning view)
 //   uploadKQWeight, fuseKQ               runtime/model_runner.cpp:958-963, :1002-1012
 //   makeKQParams  P = {K,N,nBlocks,rowStrideWords,yOffset}   runtime/model_runner.cpp:2404-2413
@@ -22,7 +23,7 @@
 
 namespace bp {
 
-enum GGUFType : uint32_t { GGUF_TYPE_Q4_K = BPK_TYPE_Q4_K, GGUF_TYPE_Q6_K = BPK_TYPE_Q6_K };
+enum GGUFType : uint32_t { GGUF_TYPE_Q4_K = BPK_TYPE_Q4_K, GGUF_TYPE_Q5_K = BPK_TYPE_Q5_K, GGUF_TYPE_Q6_K = BPK_TYPE_Q6_K };
 
 struct KQuantPacked {
     std::vector<uint32_t> data;   // raw block data as u32 words, rows padded to 4 bytes
@@ -33,6 +34,7 @@ struct KQuantPacked {
 };
 
 KQuantPacked pack_q4k(const void* raw_data, uint32_t N, uint32_t K);
+KQuantPacked pack_q5k(const void* raw_data, uint32_t N, uint32_t K);
 KQuantPacked pack_q6k(const void* raw_data, uint32_t N, uint32_t K);
 
 // Row-wise concatenation of packed matrices with equal K and type (q|k|v, gate|up).
@@ -66,6 +68,55 @@ struct KQDispatch {
     std::string name;
     int run(void* stream = nullptr) const;
 };
+
+// The dispatch group around a decode matvec as one dispatch: RMSNorm of X (NormW bound, eps set), or
+// act(gate) * up with X bound to the fused gate|up buffer, and Residual added to Y (may be Y's buffer).
+// Counterpart of the reference's q4k_matmul_norm / q4k_down_gelu binding sets
+// (runtime/kernels/quant_kq/q4k_matmul_norm.wgsl:12-22, q4k_down_gelu.wgsl:11-15).
+struct KQFusedDispatch {
+    KQDispatch base;
+    int prologue = BPK_PRO_NONE;
+    GPUBuffer NormW, Residual, Workspace;   // Workspace only for shapes that need separate launches
+    float eps = 0.0f;
+    int run(void* stream = nullptr) const;
+};
+
+// Read-only view of a GGUF file with the reference's member names.  Tensor data pointers stay valid
+// until the object is destroyed.
+struct GGUFTensorInfo {
+    std::string name;
+    std::vector<uint64_t> shape;
+    uint32_t type = 0;
+    uint64_t offset = 0;
+    const void* data = nullptr;   // host address of the tensor's bytes
+    uint64_t bytes = 0;
+};
+
+struct GGUFFile {
+    uint32_t version = 0;
+    uint64_t n_tensors = 0;
+    uint64_t data_offset = 0;
+    std::vector<GGUFTensorInfo> tensors;
+
+    GGUFFile() = default;
+    GGUFFile(const GGUFFile&) = delete;
+    GGUFFile& operator=(const GGUFFile&) = delete;
+    ~GGUFFile();
+    bool open(const std::string& path);
+    const GGUFTensorInfo* find(const std::string& name) const;
+    std::string getString(const std::string& key, const std::string& def = "") const;
+    uint32_t getU32(const std::string& key, uint32_t def = 0) const;
+    float getFloat(const std::string& key, float def = 0.0f) const;
+    bool getBool(const std::string& key, bool def = false) const;
+    bool hasKey(const std::string& key) const;
+    // Named k-quant tensors stacked into one device weight (q|k|v, gate|up); W.handle is the library's
+    // allocation and is released with releaseWeight.
+    bool loadKQWeight(const std::vector<std::string>& names, GPUBuffer& W, KQuantPacked& desc, bpk_weight** owner) const;
+
+private:
+    bpk_gguf* g_ = nullptr;
+};
+void releaseWeight(bpk_weight* owner);
 
 // Dequantised rows (the q6k_gather / q6k_gather_batched dispatch).
 int gatherKQ(GGUFType type, const GPUBuffer& W, uint32_t rowStrideWords, const GPUBuffer& tokens, uint32_t M,

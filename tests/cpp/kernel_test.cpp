@@ -1,4 +1,4 @@
-// The reference's nine Q4_K / Q6_K kernel tests (runtime/tests/kernel_test.cpp:1678-1748)
+// The reference's eleven Q4_K / Q5_K / Q6_K kernel tests (runtime/tests/kernel_test.cpp:1669-1748)
 // re-stated against the C++ host layer: same names, same closed-form inputs, same
 // tolerances.  Expected values come from the CPU oracle (test infrastructure),
 // which plays the part of dequant_kquant + the sequential fp32 dot.
@@ -42,7 +42,8 @@ static CheckResult assertClose(const float* a, const float* e, int n, float atol
 static CheckResult runMatmul(GGUFType type, const std::vector<uint8_t>& raw, int M, int N, int K,
                              const std::vector<float>& x, const std::vector<float>& bias, bool biasFirst)
 {
-    KQuantPacked pk = type == GGUF_TYPE_Q4_K ? pack_q4k(raw.data(), N, K) : pack_q6k(raw.data(), N, K);
+    KQuantPacked pk = type == GGUF_TYPE_Q4_K ? pack_q4k(raw.data(), N, K)
+                    : type == GGUF_TYPE_Q5_K ? pack_q5k(raw.data(), N, K) : pack_q6k(raw.data(), N, K);
     std::vector<float> expected(M * N);
     kqo_matmul((int)type, x.data(), pk.data.data(), biasFirst ? bias.data() : nullptr, expected.data(), M, N, K,
                pk.rowStrideWords, 0, 0);
@@ -70,6 +71,18 @@ static std::vector<uint8_t> q4kRaw(int N, int NB, std::function<float(int, int)>
     }
     return raw;
 }
+static std::vector<uint8_t> q5kRaw(int N, int NB, std::function<float(int, int)> d, std::function<float(int, int)> dm,
+                                   std::function<int(int, int, int)> byte)
+{
+    std::vector<uint8_t> raw((size_t)N * NB * 176);
+    for (int n = 0; n < N; n++) for (int b = 0; b < NB; b++) {
+        uint8_t* p = raw.data() + ((size_t)n * NB + b) * 176;
+        uint16_t hd = f32ToF16(d(n, b)), hm = f32ToF16(dm(n, b));
+        memcpy(p, &hd, 2); memcpy(p + 2, &hm, 2);
+        for (int i = 4; i < 176; i++) p[i] = (uint8_t)byte(n, b, i);
+    }
+    return raw;
+}
 static std::vector<uint8_t> q6kRaw(int N, int NB, std::function<float(int, int)> d, std::function<int(int, int, int)> byte)
 {
     std::vector<uint8_t> raw((size_t)N * NB * 210);
@@ -82,6 +95,18 @@ static std::vector<uint8_t> q6kRaw(int N, int NB, std::function<float(int, int)>
 }
 static std::vector<float> biasVec(int N, bool on) { std::vector<float> b(N, 0.f); if (on) for (int n = 0; n < N; n++) b[n] = .01f * n; return b; }
 
+TEST(q5k_matmul_reference) {
+    const int N = 8, K = 256;
+    auto raw = q5kRaw(N, 1, [](int n, int) { return .02f + .001f * n; }, [](int n, int) { return .01f + .0005f * n; },
+                      [](int n, int, int i) { return (n * 37 + i * 13 + 7) & 255; });
+    return runMatmul(GGUF_TYPE_Q5_K, raw, 1, N, K, randnVec(4242, K), biasVec(N, false), false);
+}
+TEST(q5k_matmul_batched4_reference) {
+    const int M = 5, N = 9, K = 512;
+    auto raw = q5kRaw(N, 2, [](int n, int) { return .02f + .001f * n; }, [](int, int b) { return .01f + .0002f * b; },
+                      [](int n, int b, int i) { return n * 29 + b * 11 + i * 19; });
+    return runMatmul(GGUF_TYPE_Q5_K, raw, M, N, K, randnVec(4949, M * K), biasVec(N, true), true);
+}
 TEST(q4k_matmul_reference) {
     const int N = 8, K = 256;
     auto raw = q4kRaw(N, 1, [](int n, int) { return .02f + .001f * n; }, [](int n, int) { return .01f + .0005f * n; },
@@ -170,6 +195,84 @@ TEST(fuse_qkv_rows) {
     readBuffer(by, got.data(), f.N * 4);
     releaseBuffer(bx); releaseBuffer(bw); releaseBuffer(by);
     return assertClose(got.data(), expected.data(), f.N, 2e-4f, 2e-4f);
+}
+
+TEST(fused_down_silu_residual) {
+    // act*mul -> kq_down -> add_inplace (runtime/model_runner.cpp:3748-3793) as one dispatch, against the
+    // oracle's three steps
+    const int N = 24, K = 512;
+    auto raw = q6kRaw(N, 2, [](int n, int b) { return .018f + .0007f * n + .0002f * b; },
+                      [](int n, int b, int i) { return n * 23 + b * 17 + i * 13; });
+    KQuantPacked pk = pack_q6k(raw.data(), N, K);
+    auto gu = randnVec(91, 2 * K), res = randnVec(92, N);
+    std::vector<float> act(K), expected(N), got(N);
+    kqo_prologue(2, gu.data(), nullptr, 0.f, 1, K, act.data());
+    kqo_matmul(KQO_TYPE_Q6_K, act.data(), pk.data.data(), nullptr, expected.data(), 1, N, K, pk.rowStrideWords, 0, 0);
+    for (int n = 0; n < N; n++) expected[n] += res[n];
+    GPUBuffer bx = createBuffer("GateUp", 2 * K * 4), bw = uploadKQWeight("down", pk), by = createBuffer("x", N * 4);
+    writeBuffer(bx, gu.data(), 2 * K * 4);
+    writeBuffer(by, res.data(), N * 4);
+    KQFusedDispatch d;
+    d.base = KQDispatch{GGUF_TYPE_Q6_K, bx, bw, GPUBuffer{}, by, makeKQParams(K, N, pk.nBlocks, pk.rowStrideWords), 1, "down"};
+    d.prologue = BPK_PRO_SILU_MUL;
+    d.Residual = by;   // x += down(...)
+    if (d.run() != BPK_OK) return {false, bpk_last_error()};
+    readBuffer(by, got.data(), N * 4);
+    releaseBuffer(bx); releaseBuffer(bw); releaseBuffer(by);
+    return assertClose(got.data(), expected.data(), N, 2e-4f, 2e-4f);
+}
+TEST(gguf_file_to_fused_weight) {
+    // a two-tensor GGUF written here, read through the GGUFFile mirror, gate|up stacked from it
+    const int K = 256, N = 6;
+    auto rg = q4kRaw(N, 1, [](int n, int) { return .02f + .001f * n; }, [](int, int) { return .01f; },
+                     [](int n, int, int i) { return n * 31 + i * 17; });
+    auto ru = q4kRaw(N, 1, [](int n, int) { return .03f + .001f * n; }, [](int, int) { return .02f; },
+                     [](int n, int, int i) { return n * 7 + i * 5 + 1; });
+    std::vector<uint8_t> f;
+    auto put = [&](const void* p, size_t n) { f.insert(f.end(), (const uint8_t*)p, (const uint8_t*)p + n); };
+    auto u32 = [&](uint32_t v) { put(&v, 4); };
+    auto u64 = [&](uint64_t v) { put(&v, 8); };
+    auto str = [&](const std::string& s) { u64(s.size()); put(s.data(), s.size()); };
+    u32(0x46554747); u32(3); u64(2); u64(2);
+    str("general.architecture"); u32(8); str("llama");
+    str("llama.block_count"); u32(4); u32(32);
+    const size_t bytes = (size_t)N * 144;
+    str("blk.0.ffn_gate.weight"); u32(2); u64(K); u64(N); u32(12); u64(0);
+    str("blk.0.ffn_up.weight"); u32(2); u64(K); u64(N); u32(12); u64((bytes + 31) / 32 * 32);
+    const size_t data_offset = (f.size() + 31) / 32 * 32;
+    f.resize(data_offset, 0);
+    put(rg.data(), bytes);
+    f.resize(data_offset + (bytes + 31) / 32 * 32, 0);
+    put(ru.data(), bytes);
+    const char* path = "/tmp/bpk_kernel_test.gguf";
+    FILE* fp = fopen(path, "wb");
+    if (!fp) return {false, "cannot write the temporary file"};
+    fwrite(f.data(), 1, f.size(), fp);
+    fclose(fp);
+    GGUFFile g;
+    if (!g.open(path)) return {false, bpk_last_error()};
+    if (g.version != 3 || g.n_tensors != 2 || g.data_offset != data_offset) return {false, "header fields"};
+    if (g.getString("general.architecture") != "llama" || g.getU32("llama.block_count") != 32 ||
+        g.getU32("missing", 7) != 7 || g.hasKey("nope"))
+        return {false, "metadata getters"};
+    const GGUFTensorInfo* t = g.find("blk.0.ffn_up.weight");
+    if (!t || t->shape.size() != 2 || t->shape[0] != (uint64_t)K || memcmp(t->data, ru.data(), bytes)) return {false, "tensor table"};
+    GPUBuffer W; KQuantPacked desc; bpk_weight* owner = nullptr;
+    if (!g.loadKQWeight({"blk.0.ffn_gate.weight", "blk.0.ffn_up.weight"}, W, desc, &owner)) return {false, bpk_last_error()};
+    if (desc.N != 2u * N || desc.K != (uint32_t)K) return {false, "stacked descriptor"};
+    KQuantPacked pg = pack_q4k(rg.data(), N, K), pu = pack_q4k(ru.data(), N, K);
+    auto x = randnVec(5, K);
+    std::vector<float> expected(2 * N), got(2 * N);
+    kqo_matmul(KQO_TYPE_Q4_K, x.data(), pg.data.data(), nullptr, expected.data(), 1, N, K, pg.rowStrideWords, 0, 0);
+    kqo_matmul(KQO_TYPE_Q4_K, x.data(), pu.data.data(), nullptr, expected.data() + N, 1, N, K, pu.rowStrideWords, 0, 0);
+    GPUBuffer bx = createBuffer("X", K * 4), by = createBuffer("Y", 2 * N * 4);
+    writeBuffer(bx, x.data(), K * 4);
+    KQDispatch d{desc.type, bx, W, GPUBuffer{}, by, makeKQParams(K, desc.N, desc.nBlocks, desc.rowStrideWords), 1, "gate_up"};
+    if (d.run() != BPK_OK) return {false, bpk_last_error()};
+    readBuffer(by, got.data(), got.size() * 4);
+    releaseBuffer(bx); releaseBuffer(by); releaseWeight(owner);
+    remove(path);
+    return assertClose(got.data(), expected.data(), 2 * N, 2e-4f, 2e-4f);
 }
 
 int main()
