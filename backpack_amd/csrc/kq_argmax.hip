@@ -9,31 +9,20 @@
 #include <hip/hip_runtime.h>
 
 #include "kq_kernels.h"
+#include "kq_wave.h"
 
 namespace kq {
-
-__device__ __forceinline__ void argmax_better(float& v, uint32_t& i, float ov, uint32_t oi)
-{
-    const bool take = ov > v || (ov == v && oi < i);
-    v = take ? ov : v;
-    i = take ? oi : i;
-}
 
 // Best of a workgroup of 256 lanes; valid in thread 0.
 __device__ __forceinline__ void argmax_block(float& v, uint32_t& i, float (&sv)[4], uint32_t (&si)[4])
 {
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const float ov = __shfl_xor(v, o);
-        const uint32_t oi = __shfl_xor(i, o);
-        argmax_better(v, i, ov, oi);
-    }
+    wave_best(v, i);
     if ((threadIdx.x & 63u) == 0) { sv[threadIdx.x >> 6] = v; si[threadIdx.x >> 6] = i; }
     __syncthreads();
     if (threadIdx.x == 0) {
         v = sv[0]; i = si[0];
 #pragma unroll
-        for (int w = 1; w < 4; ++w) argmax_better(v, i, sv[w], si[w]);
+        for (int w = 1; w < 4; ++w) best_of(v, i, sv[w], si[w]);
     }
 }
 
@@ -71,7 +60,7 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const float* logits, u
         const size_t cell = (size_t)row * parts + q;
         const float pv = __hip_atomic_load(&part_val[cell], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const uint32_t pi = __hip_atomic_load(&part_idx[cell], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        argmax_better(v, i, pv, pi);
+        best_of(v, i, pv, pi);
     }
     __syncthreads();   // sv / si are reused
     argmax_block(v, i, sv, si);

@@ -11,34 +11,25 @@
 #include <hip/hip_runtime.h>
 
 #include "kq_kernels.h"
+#include "kq_wave.h"
 
 namespace kq {
 
 constexpr int ROUTE_MAX_PER_LANE = 16;   // n_experts <= 1024
-constexpr int ROUTE_MAX_K = 16;
 constexpr float ROUTE_NEG_INF = -3.4e38f;
 
-// The better of two (value, index) candidates: larger value, then lower index.
-__device__ __forceinline__ void route_better(float& v, uint32_t& i, float ov, uint32_t oi)
-{
-    const bool take = ov > v || (ov == v && oi < i);
-    v = take ? ov : v;
-    i = take ? oi : i;
-}
-
 // One wave selects for one token.  vals[j] is the logit of expert 64*j + lane (-inf beyond n_experts).
+// Lane s ends up holding the s-th pick.  The pass loop is a real loop: these kernels run their code once,
+// and unrolled they spent their time fetching instructions (10 us for a few hundred operations).
 template <int PER_LANE>
 __device__ __forceinline__ void route_select(float (&vals)[PER_LANE], uint32_t lane, uint32_t n_experts, uint32_t k,
                                              int normalize, uint32_t* idx_out, float* wt_out)
 {
-    float sel_v[ROUTE_MAX_K];
-    uint32_t sel_i[ROUTE_MAX_K];
+    float my_v = ROUTE_NEG_INF;
+    uint32_t my_i = 0;
     uint32_t taken = 0;   // bit j: the lane's j-th expert is masked
-#pragma unroll
-    for (int s = 0; s < ROUTE_MAX_K; ++s) {
-        sel_v[s] = ROUTE_NEG_INF;
-        sel_i[s] = 0;
-        if ((uint32_t)s >= k) continue;   // k is uniform: no divergence, and the loop unrolls
+#pragma nounroll
+    for (uint32_t s = 0; s < k; ++s) {
         // lane-local candidate among the unmasked experts; an expert only counts if it beats -3.4e38
         float bv = ROUTE_NEG_INF;
         uint32_t bi = 0xFFFFFFFFu;
@@ -49,36 +40,40 @@ __device__ __forceinline__ void route_select(float (&vals)[PER_LANE], uint32_t l
             bv = ok ? vals[j] : bv;
             bi = ok ? e : bi;
         }
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const float ov = __shfl_xor(bv, o);
-            const uint32_t oi = __shfl_xor(bi, o);
-            route_better(bv, bi, ov, oi);
-        }
+        wave_best(bv, bi);
         // nothing above -3.4e38 left: the reference's scan leaves index 0 and that value
         if (bi == 0xFFFFFFFFu) bi = 0;
-        sel_v[s] = bv;
-        sel_i[s] = bi;
-        if ((bi & 63u) == lane) taken |= 1u << (bi >> 6);
+        else if ((bi & 63u) == lane) taken |= 1u << (bi >> 6);
+        if (lane == s) { my_v = bv; my_i = bi; }
     }
-    float mx = sel_v[0];
+    float mx = lane < k ? my_v : ROUTE_NEG_INF;
 #pragma unroll
-    for (int s = 1; s < ROUTE_MAX_K; ++s)
-        if ((uint32_t)s < k && sel_v[s] > mx) mx = sel_v[s];
-    float sum = 0.0f;
+    for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    const float ex = lane < k ? expf(my_v - mx) : 0.0f;
+    float sum = ex;
 #pragma unroll
-    for (int s = 0; s < ROUTE_MAX_K; ++s)
-        if ((uint32_t)s < k) {
-            sel_v[s] = expf(sel_v[s] - mx);
-            sum += sel_v[s];
-        }
+    for (int o = 1; o < 64; o <<= 1) sum += __shfl_xor(sum, o);
     const float inv = (normalize && sum > 0.0f) ? 1.0f / sum : 1.0f;
-#pragma unroll
-    for (int s = 0; s < ROUTE_MAX_K; ++s)
-        if ((uint32_t)s < k && lane == (uint32_t)s) {
-            idx_out[s] = sel_i[s];
-            wt_out[s] = sel_v[s] * inv;
-        }
+    if (lane < k) {
+        idx_out[lane] = my_i;
+        wt_out[lane] = ex * inv;
+    }
+}
+
+// Picks the scan width by the number of experts (wave-uniform): the lane-local scan is the larger half
+// of a pass.
+__device__ __forceinline__ void route_select_any(float (&vals)[ROUTE_MAX_PER_LANE], uint32_t lane, uint32_t n_experts,
+                                                 uint32_t k, int normalize, uint32_t* idx_out, float* wt_out)
+{
+    if (n_experts <= 128u) {
+        float v2[2] = {vals[0], vals[1]};
+        route_select(v2, lane, n_experts, k, normalize, idx_out, wt_out);
+    } else if (n_experts <= 256u) {
+        float v4[4] = {vals[0], vals[1], vals[2], vals[3]};
+        route_select(v4, lane, n_experts, k, normalize, idx_out, wt_out);
+    } else {
+        route_select(vals, lane, n_experts, k, normalize, idx_out, wt_out);
+    }
 }
 
 // logits [T, n_experts] -> idx, wt [T, k]; a wave per token, four tokens per workgroup.
@@ -94,7 +89,7 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const float* logits, 
         const uint32_t e = 64u * j + lane;
         vals[j] = e < n_experts ? logits[(size_t)tok * n_experts + e] : ROUTE_NEG_INF;
     }
-    route_select(vals, lane, n_experts, k, normalize, idx + (size_t)tok * k, wt + (size_t)tok * k);
+    route_select_any(vals, lane, n_experts, k, normalize, idx + (size_t)tok * k, wt + (size_t)tok * k);
 }
 
 // Logits of experts e0 .. e0+3 for one token: lanes along hidden, four independent load streams.
@@ -155,7 +150,7 @@ __global__ __launch_bounds__(256) void route_kernel(const float* X, const float*
         const uint32_t e = 64u * j + lane;
         vals[j] = e < n_experts ? lg[e] : ROUTE_NEG_INF;
     }
-    route_select(vals, lane, n_experts, k, normalize, idx + (size_t)tok * k, wt + (size_t)tok * k);
+    route_select_any(vals, lane, n_experts, k, normalize, idx + (size_t)tok * k, wt + (size_t)tok * k);
 }
 
 // Few tokens: the experts are spread over workgroups (blockIdx.x takes 16 of them, blockIdx.y is the token)

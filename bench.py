@@ -507,16 +507,30 @@ def moe_leg():
         sec = e0.elapsed_time(e1) * 1e-3 / (reps * len(layers))
         nbytes = touched * per_expert
         flops = 2.0 * T * k * 3 * H * I
-        # the router stage in front of it: fp32 router matvec + top-k softmax
+        # the router stage in front of it: fp32 router matvec + top-k softmax, timed in a replayed graph
         wr = torch.randn(E, H, device="cuda") / H ** 0.5
-        kquant.moe_route(x, wr, k)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(reps * len(layers)):
-            kquant.moe_route(x, wr, k)
-        e1.record()
-        torch.cuda.synchronize()
-        route_us = e0.elapsed_time(e1) * 1e3 / (reps * len(layers))
+        ridx = torch.empty((T, k), dtype=torch.int32, device="cuda")
+        rwt = torch.empty((T, k), dtype=torch.float32, device="cuda")
+        rs = torch.cuda.Stream()
+        with torch.cuda.stream(rs):
+            def route():
+                capi.check(capi.lib().bpk_moe_route(x.data_ptr(), wr.data_ptr(), T, H, E, k, 1, None, ridx.data_ptr(),
+                                                    rwt.data_ptr(), rs.cuda_stream))
+            route()
+            rs.synchronize()
+            rg = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(rg, stream=rs):
+                for _ in range(50):
+                    route()
+            rg.replay()
+            rs.synchronize()
+            r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            r0.record(rs)
+            for _ in range(10):
+                rg.replay()
+            r1.record(rs)
+            rs.synchronize()
+        route_us = r0.elapsed_time(r1) * 1e3 / 500
         res[f"T{T}"] = {"us_per_layer": round(sec * 1e6, 2), "route_us": round(route_us, 2),
                         "experts_touched": touched, "weight_bytes": nbytes,
                         "GBps": round(nbytes / sec / 1e9, 1), "TFLOPs": round(flops / sec / 1e12, 2),
