@@ -38,6 +38,7 @@
 // tiles through LDS at the end.  There is no fold across workgroups.
 #include "kq_format.h"
 #include "kq_kernels.h"
+#include "kq_wave.h"
 
 namespace kq {
 
@@ -137,8 +138,12 @@ struct MtileStager {
             amax = max(amax, __builtin_bit_cast(uint32_t, v[i].z) & 0x7FFFFFFFu);
             amax = max(amax, __builtin_bit_cast(uint32_t, v[i].w) & 0x7FFFFFFFu);
         }
-#pragma unroll
-        for (int off = 1; off < TPP; off <<= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, off, 64));
+        // (DPP moves: an LDS-routed shuffle costs a hundred cycles, and this chain sits in front of the barrier)
+        if constexpr (TPP > 1) amax = max(amax, (uint32_t)group_partner<1>((int)amax));
+        if constexpr (TPP > 2) amax = max(amax, (uint32_t)group_partner<2>((int)amax));
+        if constexpr (TPP > 4) amax = max(amax, (uint32_t)group_partner<4>((int)amax));
+        if constexpr (TPP > 8) amax = max(amax, (uint32_t)group_partner<8>((int)amax));
+        static_assert(TPP <= 16, "the largest magnitude is reduced inside a row of 16 lanes");
         uint32_t e = amax >> 23;                  // biased exponent of the largest |x|
         e = e < 15u ? 15u : (e > 253u ? 253u : e);
         const float s = __builtin_bit_cast(float, (268u - e) << 23);     // 2^(141-e): amax*s in [2^14, 2^15)
@@ -199,13 +204,13 @@ struct MtileStager {
 #pragma unroll
             for (int i = 0; i < EPT / 4; ++i) h += (v[i].x + v[i].y) + (v[i].z + v[i].w);
             constexpr int PER16 = 16 / EPT;   // threads per half run: 1 (EPT 16) or 2 (EPT 8)
-            if (PER16 == 2) h += __shfl_xor(h, 1, 64);
+            if (PER16 == 2) h += group_partner<1>(h);
             const uint32_t half = (sub / PER16) & 1u, run = sub / (2u * PER16);
             float* dst = xs + (bb * 8u + run) * 16u + token;
             if (SPLIT16) {
                 if (sub % PER16 == 0u) dst[8u * half] = h;
             } else {
-                h += __shfl_xor(h, PER16, 64);
+                h += group_partner<PER16>(h);
                 if (sub % (2u * PER16) == 0u) { dst[0] = h; put_sum(run, h); }
             }
         }

@@ -5,6 +5,23 @@
 
 namespace kq {
 
+// One step of an all-reduce over an aligned group of 2, 4, 8 or 16 lanes, taken in the order OFF = 1, 2,
+// 4, 8: the partner's value as a DPP move.  Steps 1 and 2 are lane ^ 1 and lane ^ 2; steps 4 and 8 are the
+// mirrors within 8 and 16 lanes, which pair every lane with one from the other half — the same thing for
+// an all-reduce, since after the earlier steps all lanes of a half hold the same value.
+template <int OFF>
+__device__ __forceinline__ int group_partner(int x)
+{
+    static_assert(OFF == 1 || OFF == 2 || OFF == 4 || OFF == 8, "steps of an all-reduce over up to 16 lanes");
+    constexpr int CTRL = OFF == 1 ? 0xB1 : OFF == 2 ? 0x4E : OFF == 4 ? 0x141 : 0x140;
+    return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xF, 0xF, false);
+}
+template <int OFF>
+__device__ __forceinline__ float group_partner(float x)
+{
+    return __builtin_bit_cast(float, group_partner<OFF>(__builtin_bit_cast(int, x)));
+}
+
 // The better of two (value, index) candidates: larger value, then lower index.
 __device__ __forceinline__ void best_of(float& v, uint32_t& i, float ov, uint32_t oi)
 {
