@@ -397,7 +397,13 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     const bool stream_ok = kq::gemv_stream_supported(a);
     const bool mtile_ok = kq::mtile_supported(a);
     if (t_family == 6 && !mtile_ok) return fail(BPK_ERR_SHAPE, "16x16 tile kernel cannot serve this call");
-    if (t_family == 6 || (t_family == 0 && mtile_ok && M >= 3 && M <= 255)) {
+    // three and four tokens on the smaller matrices stay on the lanes-along-K kernel (four tokens share every
+    // weight load and its unpack).  Measured at M = 4: Q4_K 4096x4096 10.0 against 10.8 us on the tile
+    // kernel, 6144x4096 a tie, 28672x4096 34.5 against 23.0; Q6_K 4096x14336 23.6 against 27.1.
+    const uint64_t weights = (uint64_t)N * K;
+    const bool stream_four = stream_ok && M >= 3 && M <= 4 && N <= 32768u &&
+                             weights <= (type == BPK_TYPE_Q6_K ? (64ull << 20) : (20ull << 20));
+    if (t_family == 6 || (t_family == 0 && mtile_ok && M >= 3 && M <= 255 && !stream_four)) {
         t_kernel = "mtile";
         e = kq::launch_mtile(a, st->split, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
@@ -407,7 +413,7 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     // up to a few tens of thousands of rows the lanes-along-K kernel wins at M = 1
     // (no LDS staging, no K split to fold); longer matrices reach a steady state
     // in which the row-per-lane kernel streams faster
-    if (t_family == 5 || (t_family == 0 && stream_ok && N <= 32768u)) {
+    if (t_family == 5 || (t_family == 0 && stream_ok && N <= 32768u && (M <= 2 || stream_four))) {
         t_kernel = "gemv_stream";
         e = kq::launch_gemv_stream(a, t_gemv, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);

@@ -30,12 +30,13 @@ typedef uint32_t s_u32x4 __attribute__((ext_vector_type(4)));
 // Kernel arguments come in three sizes, and a kernel is compiled for each: the wave's first
 // instructions fetch them, and every further 64 bytes of them cost a launch a measurable fraction of a
 // microsecond, so the dense decode matvec gets the smallest set that describes it.
-struct StreamDense {          // 56 bytes
+struct StreamDense {          // 60 bytes
     const float* X;
     const uint8_t* W;
     const float* bias;
     float* Y;
     uint32_t N, K, n_blocks, row_stride_bytes, y_offset, ldy;
+    uint32_t M;   // tokens; read only by the four-token kernels (three tokens run as four, the last one masked)
     static constexpr bool kGrouped = false, kFused = false;
 };
 
@@ -47,6 +48,7 @@ struct StreamFused {
     const float* bias;
     float* Y;
     uint32_t N, K, n_blocks, row_stride_bytes, y_offset, ldy;
+    uint32_t M;
     int pro;
     float eps;
     const float* norm_w;
@@ -64,6 +66,7 @@ struct StreamGrouped {
     const float* bias;
     float* Y;
     uint32_t N, K, n_blocks, row_stride_bytes, y_offset, ldy;
+    uint32_t M;
     const uint32_t* expert_idx;
     uint32_t k_slots;
     int x_per_slot;
@@ -352,7 +355,8 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
             hoff[pass] = b * BLOCK;
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                const float4* xp = (const float4*)(p.X + (size_t)t * ldx + (size_t)b * KQ_QK + 64u * g + 16u * h);
+                const uint32_t xt = MT > 2 ? min((uint32_t)t, p.M - 1u) : (uint32_t)t;   // a masked token re-reads the last one
+                const float4* xp = (const float4*)(p.X + (size_t)xt * ldx + (size_t)b * KQ_QK + 64u * g + 16u * h);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float4 lo = stream_x4<PRO, PT::kFused>(xp + i, x2_off), hi = stream_x4<PRO, PT::kFused>(xp + 8 + i, x2_off);
@@ -462,6 +466,7 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
             const float bias = p.bias ? p.bias[r] : 0.0f;
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
+                if (MT > 2 && (uint32_t)t >= p.M) continue;
                 const size_t at = (size_t)t * p.ldy + p.y_offset + r;
                 float y = res[t];
                 if (KW > 1) {
@@ -613,7 +618,8 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(PT p)
             boff[pass] = b * KQ_Q6K_BYTES;
 #pragma unroll
             for (int tk = 0; tk < MT; ++tk) {
-                const float4* xp = (const float4*)(p.X + (size_t)tk * ldx + (size_t)b * KQ_QK + 128u * n + 8u * lg);
+                const uint32_t xt = MT > 2 ? min((uint32_t)tk, p.M - 1u) : (uint32_t)tk;
+                const float4* xp = (const float4*)(p.X + (size_t)xt * ldx + (size_t)b * KQ_QK + 128u * n + 8u * lg);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     float4 lo = stream_x4<PRO, PT::kFused>(xp + 8 * k, x2_off), hi = stream_x4<PRO, PT::kFused>(xp + 8 * k + 1, x2_off);
@@ -732,6 +738,7 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(PT p)
 #pragma unroll
                     for (int w = 1; w < KW; ++w) y += part[w][tk][lane];
                 }
+                if (MT > 2 && (uint32_t)tk >= p.M) continue;
                 const size_t at = (size_t)tk * p.ldy + p.y_offset + r;
                 y += bias;
                 if constexpr (PT::kFused) y += stream_residual(p) ? stream_residual(p)[at] : 0.0f;
@@ -759,7 +766,11 @@ static uint32_t stream_workgroups(uint32_t N, uint32_t per_cu, int rows_override
 bool gemv_stream_supported(const MatmulArgs& a)
 {
     // grouped calls: M counts (token, slot) pairs, each a matvec of its own
-    if (!a.expert_idx && (a.M < 1 || a.M > 2)) return false;
+    if (!a.expert_idx && (a.M < 1 || a.M > 4)) return false;
+    // three and four tokens: Q4_K / Q6_K, plain calls, rows of at most 56 superblocks
+    if (!a.expert_idx && a.M > 2 &&
+        (a.n_blocks > 56 || a.pro != 0 || a.residual || (a.type != KQ_TYPE_Q4_K && a.type != KQ_TYPE_Q6_K)))
+        return false;
     if (a.expert_idx && (a.M < 1 || a.M > 65535u || a.bias)) return false;
     if (((uintptr_t)a.X & 15u)) return false;
     if (a.n_blocks < 1) return false;
@@ -811,12 +822,38 @@ static void launch_q4k_sliced(dim3 grid, hipStream_t s, const PT& p)
     if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, 1, 2, MT, PT, Q5, KW>), grid, dim3(64 * KW), 0, s, p);
 }
 
+// Three or four tokens (dense calls): every wave holds a K slice of eight superblocks for four tokens (128
+// activations per lane), so rows of any length up to 56 superblocks are cut over 1, 2, 4 or 7 waves; two
+// rows in flight.  Three tokens run as four with the last one masked.
+template <typename PT>
+static hipError_t launch_stream_four(const MatmulArgs& a, hipStream_t s, const PT& p)
+{
+    const uint32_t nb = a.n_blocks;
+    const int kw = nb <= 8u ? 1 : nb <= 16u ? 2 : nb <= 32u ? 4 : 7;
+    const uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 8u / (uint32_t)kw, 0);
+    const dim3 grid(wgs, 1, 1);
+    if (a.type == KQ_TYPE_Q6_K) {
+        if (kw == 1) hipLaunchKernelGGL((q6k_stream_kernel<1, 1, 2, 4, PT>), grid, dim3(64), 0, s, p);
+        else if (kw == 2) hipLaunchKernelGGL((q6k_stream_kernel<1, 2, 2, 4, PT>), grid, dim3(128), 0, s, p);
+        else if (kw == 4) hipLaunchKernelGGL((q6k_stream_kernel<1, 4, 2, 4, PT>), grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((q6k_stream_kernel<1, 7, 2, 4, PT>), grid, dim3(448), 0, s, p);
+    } else {
+        if (kw == 1) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 1>), grid, dim3(64), 0, s, p);
+        else if (kw == 2) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 2>), grid, dim3(128), 0, s, p);
+        else if (kw == 4) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 4>), grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 7>), grid, dim3(448), 0, s, p);
+    }
+    return hipGetLastError();
+}
+
 template <typename PT>
 static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, hipStream_t s, const PT& p,
                                      uint32_t pairs, uint32_t twins)
 {
     const bool two = !PT::kGrouped && a.M == 2;       // two tokens share every weight load
-    const dim3 grid_yz(1, pairs, twins);
+    if constexpr (!PT::kGrouped && !PT::kFused) {
+        if (a.M > 2) return launch_stream_four(a, s, p);
+    }
     // Measured on MI355X: these kernels run best with about 40 KB of weight loads
     // in flight per CU: 4 to 8 waves, two to four rows in flight each.  More waves
     // or deeper rings are slower.
@@ -910,6 +947,7 @@ static void stream_fill_common(PT& p, const MatmulArgs& a)
     p.row_stride_bytes = a.row_stride_bytes;
     p.y_offset = a.y_offset;
     p.ldy = a.ldy;
+    p.M = a.M;
 }
 
 hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStream_t s)

@@ -91,6 +91,28 @@ def test_reference_recipe(gpu, kqo, name, family):
     assert bad == 0, f"{name}: {bad} elements outside atol={atol} rtol={rtol}, worst excess {worst}"
 
 
+# ---- three and four tokens on the lanes-along-K kernel ---------------------------------
+@pytest.mark.parametrize("type_,M,N,K", [
+    (Q4_K, 3, 130, 2048), (Q4_K, 4, 300, 4096), (Q4_K, 3, 200, 8192), (Q4_K, 4, 100, 14336), (Q4_K, 4, 4096, 4096),
+    (Q4_K, 3, 77, 6400),                       # 25 superblocks: the fourth K slice is partial
+    (Q6_K, 4, 33, 768), (Q6_K, 3, 150, 4096), (Q6_K, 4, 120, 8192), (Q6_K, 3, 4096, 14336), (Q6_K, 4, 64, 2048),
+])
+def test_four_token_stream_kernels(gpu, kqo, type_, M, N, K):
+    """Every K-slice count (1, 2, 4, 7 waves), three tokens run as four with the last masked: the rows of Y
+    beyond M must stay untouched."""
+    from backpack_amd import capi, kquant
+    _say("four-token stream", type_, M, N, K)
+    raw, packed, w = gpu.make_weight(type_, N, K, seed=M * 31 + N)
+    X = np.random.default_rng(N + K).standard_normal((M, K)).astype(np.float32)
+    bias = np.random.default_rng(2).standard_normal(N).astype(np.float32)
+    out = gpu.dev(np.full((M + 1, N), 7.5, np.float32))
+    kquant.matmul(gpu.dev(X), w, bias=gpu.dev(bias), out=out[:M])
+    assert capi.last_kernel() == "gemv_stream"
+    got = out.cpu().numpy()
+    assert np.all(got[M] == 7.5)
+    gpu.check_matmul(kqo, type_, got[:M], X, packed, N, K, bias=bias, label=f"four {type_} {M}x{N}x{K}")
+
+
 # ---- Q5_K: packers, rows and the fp32 matmul (generic kernel) ------------------------
 @pytest.mark.parametrize("M,N,K,kernel", [(1, 300, 4096, "gemv_stream"), (2, 64, 768, "gemv_stream"),
                                           (1, 4096, 4096, "gemv_stream"), (2, 6144, 4096, "gemv_stream"),
