@@ -187,7 +187,6 @@ bool read_value(Cursor& c, uint32_t t, MetaValue& v, int depth)
 }  // namespace
 
 struct bpk_gguf {
-    int fd = -1;
     const uint8_t* map = nullptr;
     uint64_t size = 0;
     uint32_t version = 0;
@@ -229,14 +228,13 @@ int bpk_gguf_open(const char* path, bpk_gguf** out)
     struct stat st;
     if (fstat(fd, &st) != 0 || st.st_size < 24) { close(fd); return fail(BPK_ERR_FORMAT, "%s is too short to be a GGUF file", path); }
     void* m = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
-    if (m == MAP_FAILED) { close(fd); return fail(BPK_ERR_IO, "cannot map %s", path); }
+    close(fd);   // the mapping outlives the descriptor
+    if (m == MAP_FAILED) return fail(BPK_ERR_IO, "cannot map %s", path);
     bpk_gguf* g = new bpk_gguf;
-    g->fd = fd;
     g->map = (const uint8_t*)m;
     g->size = (uint64_t)st.st_size;
     auto bail = [&](int code, const char* what) {
         munmap((void*)g->map, (size_t)g->size);
-        close(g->fd);
         delete g;
         return fail(code, "%s: %s", path, what);
     };
@@ -296,7 +294,6 @@ int bpk_gguf_close(bpk_gguf* g)
 {
     if (!g) return BPK_OK;
     munmap((void*)g->map, (size_t)g->size);
-    close(g->fd);
     delete g;
     return BPK_OK;
 }

@@ -61,7 +61,8 @@ BPK_API const char *bpk_last_error(void);
 
 /* Checks that `device` is a gfx950 part and creates the library's per-device
  * state (split-K scratch, counters).  Optional: the first launch on a device
- * does the same.  Replaces GPUContext device bring-up for this path
+ * does the same — but it allocates, so call it before capturing a HIP graph
+ * on that device.  Replaces GPUContext device bring-up for this path
  * (runtime/gpu_context.h:86-145). */
 BPK_API int bpk_init(int device);
 
