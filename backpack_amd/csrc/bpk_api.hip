@@ -120,8 +120,8 @@ int current_state(DeviceState** out)
 }
 
 bool known_type(int type) { return type == BPK_TYPE_Q4_K || type == BPK_TYPE_Q5_K || type == BPK_TYPE_Q6_K; }
-// Q5_K is served by the packers, the row dequantiser and the fp32 matmul (generic kernel); the bf16 GEMM
-// and the MoE entry points take the two types their kernels are written for.
+// Q5_K is served by the packers, the row dequantiser, the fp32 matmul and the 128-tile bf16 GEMM; the MoE
+// entry points take the two types their kernels are written for.
 bool fast_type(int type) { return type == BPK_TYPE_Q4_K || type == BPK_TYPE_Q6_K; }
 
 int check_matmul(int type, const void* X, const void* W, const void* Y, uint32_t M, uint32_t N, uint32_t K,
@@ -499,7 +499,6 @@ int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bi
 int bpk_kq_matmul_bf16(int type, const uint16_t* X, const void* W, const float* bias, float* Y, uint32_t M,
                        uint32_t N, uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, void* stream)
 {
-    if (type == BPK_TYPE_Q5_K) return fail(BPK_ERR_TYPE, "the bf16 GEMM takes Q4_K and Q6_K");
     if (int rc = check_matmul(type, X, W, Y, M, N, K, n_blocks, row_stride_words)) return rc;
     if (M == 0) return BPK_OK;
     if (int rc = current_state(nullptr)) return rc;

@@ -100,6 +100,49 @@ __device__ __forceinline__ void q4k_expand(const uint32_t (&raw)[12], uint32_t k
     }
 }
 
+// Q5_K: the Q4_K layout with the quants 32 bytes further on and, before them, the 32 bytes of fifth bits
+// (bit sb of byte i belongs to element i of sub-block sb).
+__device__ __forceinline__ void q5k_load(const uint8_t* row, uint32_t kc, uint32_t (&raw)[20])
+{
+    const uint8_t* blk = row + (size_t)(kc >> 2) * KQ_Q5K_BYTES;
+    const u32x4 h = *(const u32x4*)blk;
+    const u32x4 b0 = *(const u32x4*)(blk + 16), b1 = *(const u32x4*)(blk + 32);
+    const u32x4* q = (const u32x4*)(blk + 48 + (kc & 3u) * 32u);
+    const u32x4 q0 = q[0], q1 = q[1];
+    raw[0] = h.x; raw[1] = h.y; raw[2] = h.z; raw[3] = h.w;
+    raw[4] = q0.x; raw[5] = q0.y; raw[6] = q0.z; raw[7] = q0.w;
+    raw[8] = q1.x; raw[9] = q1.y; raw[10] = q1.z; raw[11] = q1.w;
+    raw[12] = b0.x; raw[13] = b0.y; raw[14] = b0.z; raw[15] = b0.w;
+    raw[16] = b1.x; raw[17] = b1.y; raw[18] = b1.z; raw[19] = b1.w;
+}
+
+__device__ __forceinline__ void q5k_expand(const uint32_t (&raw)[20], uint32_t kc, uint32_t hf, uint8_t* dst)
+{
+    const float d = half_bits_to_float(raw[0] & 0xFFFFu);
+    const float dmin = half_bits_to_float(raw[0] >> 16);
+    const uint32_t sb = (kc & 3u) * 2u + hf;
+    uint32_t sc, mn;
+    q4k_scale_min(raw[1], raw[2], raw[3], (int)sb, sc, mn);
+    const float a = d * (float)sc;
+    const float nb = -(dmin * (float)mn);
+    const uint32_t sh = hf * 4u;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        u32x4 out;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t w = ((raw[4 + v * 2 + j] >> sh) & 0x0F0F0F0Fu) | (((raw[12 + v * 2 + j] >> sb) & 0x01010101u) << 4);
+            const float f0 = fmaf(a, (float)(w & 255u), nb);
+            const float f1 = fmaf(a, (float)((w >> 8) & 255u), nb);
+            const float f2 = fmaf(a, (float)((w >> 16) & 255u), nb);
+            const float f3 = fmaf(a, (float)(w >> 24), nb);
+            out[j * 2] = pack_bf16(f0, f1);
+            out[j * 2 + 1] = pack_bf16(f2, f3);
+        }
+        *(u32x4*)(dst + v * 16) = out;
+    }
+}
+
 // Q6_K: chunk kc of the row covers elements 64*kc .. 64*kc+63 = (half h, t pair);
 // hf picks t.  Blocks are only 2-byte aligned, so bytes are fetched as u16.
 struct Q6Raw {
@@ -241,15 +284,17 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm_bf16_kernel(GemmParams p)
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     u32x4 xr[XP];
-    uint32_t w4[WI][12];
-    Q6Raw w6[WI];
+    uint32_t w4[TYPE == KQ_TYPE_Q4_K ? WI : 1][12];
+    uint32_t w5[TYPE == KQ_TYPE_Q5_K ? WI : 1][20];
+    Q6Raw w6[TYPE == KQ_TYPE_Q6_K ? WI : 1];
 
     auto load_tile = [&](uint32_t kt) {
 #pragma unroll
         for (int i = 0; i < XP; ++i) xr[i] = *(const u32x4*)(xsrc[i] + (size_t)kt * (GEMM_BK * 2));
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
-            if (TYPE == KQ_TYPE_Q4_K) q4k_load(wsrc[i], kt, w4[i]);
+            if constexpr (TYPE == KQ_TYPE_Q4_K) q4k_load(wsrc[i], kt, w4[i]);
+            else if constexpr (TYPE == KQ_TYPE_Q5_K) q5k_load(wsrc[i], kt, w5[i]);
             else q6k_load(wsrc[i], kt, whf[i], w6[i]);
         }
     };
@@ -262,7 +307,8 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm_bf16_kernel(GemmParams p)
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
             uint8_t* dst = b + wrow[i] * GEMM_LD + whf[i] * 64u;
-            if (TYPE == KQ_TYPE_Q4_K) q4k_expand(w4[i], kt, whf[i], dst);
+            if constexpr (TYPE == KQ_TYPE_Q4_K) q4k_expand(w4[i], kt, whf[i], dst);
+            else if constexpr (TYPE == KQ_TYPE_Q5_K) q5k_expand(w5[i], kt, whf[i], dst);
             else q6k_expand(w6[i], kt, whf[i], dst);
         }
     };
@@ -558,9 +604,9 @@ __global__ __launch_bounds__(256) void gemm_clear_split_tiles_kernel(GemmParams 
 bool gemm_bf16_supported(const MatmulArgs& a)
 {
     if (a.expert_idx) return false;
-    if (a.type != KQ_TYPE_Q4_K && a.type != KQ_TYPE_Q6_K) return false;
+    if (a.type != KQ_TYPE_Q4_K && a.type != KQ_TYPE_Q5_K && a.type != KQ_TYPE_Q6_K) return false;
     if ((uintptr_t)a.X & 15u) return false;            // 128-bit loads of bf16 rows (K % 256 == 0 already)
-    if (a.type == KQ_TYPE_Q4_K && (((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u))) return false;
+    if (a.type != KQ_TYPE_Q6_K && (((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u))) return false;
     if (a.type == KQ_TYPE_Q6_K && ((uintptr_t)a.W & 1u)) return false;
     return true;
 }
@@ -620,6 +666,9 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, hipStream_
     p.row_stride_bytes = a.row_stride_bytes;
     p.ldy = a.ldy;
     const bool q4 = a.type == KQ_TYPE_Q4_K;
+    // Q5_K runs on the 128-tile kernel whatever the shape (the persistent kernel's dequantiser is written
+    // for the other two types)
+    if (a.type == KQ_TYPE_Q5_K) return launch_gemm<KQ_TYPE_Q5_K, 128, 128, 4>(p, s);
     // Measured on M = 2048: 256-tiles win once they occupy more than half the CUs.  Below that, a long K is
     // worth cutting (the epilogue of a cut tile costs about 15 k steps), a short one runs on 128-tiles, two
     // workgroups per CU.  With many tiles per CU, equal shares also remove the ragged last round.

@@ -143,10 +143,6 @@ def test_q5k_is_refused_where_no_kernel_serves_it(gpu):
     from backpack_amd import capi, kquant
     raw, packed, w = gpu.make_weight(Q5_K, 64, 512, seed=1)
     import torch
-    xb = torch.zeros(256, 512, dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(capi.BpkError) as e:
-        kquant.matmul(xb, w)
-    assert e.value.code == -1
     idx = torch.zeros(2, 2, dtype=torch.int32, device="cuda")
     with pytest.raises(capi.BpkError) as e:
         kquant.moe_matmul(torch.zeros(2, 512, device="cuda"), w, idx, 4)
@@ -389,6 +385,11 @@ GEMM_SHAPES = [
     (Q6_K, 256, 256, 768, 256),      # odd block count: rows only 8-byte aligned
     (Q6_K, 190, 260, 1024, 128),
     (Q6_K, 512, 512, 4096, 0),
+    # Q5_K: the 128-tile kernel whatever is asked for
+    (Q5_K, 128, 128, 256, 0),
+    (Q5_K, 200, 300, 1024, 0),
+    (Q5_K, 512, 1024, 4096, 0),
+    (Q5_K, 300, 520, 768, 256),
     # 256-tile with the walk cut into equal shares per CU (tiles summed with atomics)
     (Q4_K, 256, 256, 256, 258),
     (Q4_K, 300, 520, 768, 258),
