@@ -401,12 +401,30 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     // weight load and its unpack).  Measured at M = 4: Q4_K 4096x4096 10.0 against 10.8 us on the tile
     // kernel, 6144x4096 a tie, 28672x4096 34.5 against 23.0; Q6_K 4096x14336 23.6 against 27.1.
     const uint64_t weights = (uint64_t)N * K;
+    // (Q5_K has no tile kernel to fall back on: it takes this path whatever the size)
     const bool stream_four = stream_ok && M >= 3 && M <= 4 && N <= 32768u &&
-                             weights <= (type == BPK_TYPE_Q6_K ? (64ull << 20) : (20ull << 20));
+                             (type == BPK_TYPE_Q5_K || weights <= (type == BPK_TYPE_Q6_K ? (64ull << 20) : (20ull << 20)));
     if (t_family == 6 || (t_family == 0 && mtile_ok && M >= 3 && M <= 255 && !stream_four)) {
         t_kernel = "mtile";
         e = kq::launch_mtile(a, st->split, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+    }
+    // Q5_K beyond four tokens: groups of four on the lanes-along-K kernel (the tile kernel does not take the
+    // type; re-reading the weights per group is still many times faster than the generic kernel)
+    if (t_family == 0 && type == BPK_TYPE_Q5_K && M > 4u && M <= 64u && N <= 32768u) {
+        kq::MatmulArgs g = a;
+        g.M = 4;
+        if (kq::gemv_stream_supported(g)) {
+            t_kernel = "gemv_stream";
+            for (uint32_t m0 = 0; m0 < M; m0 += 4u) {
+                g.M = M - m0 < 4u ? M - m0 : 4u;
+                g.X = X + (size_t)m0 * K;
+                g.Y = Y + (size_t)m0 * N;
+                e = kq::launch_gemv_stream(g, t_gemv, s);
+                if (e != hipSuccess) return hip_fail(e, t_kernel);
+            }
+            return BPK_OK;
+        }
     }
     if (t_family == 5 && !stream_ok) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");
     if (t_family == 4) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);

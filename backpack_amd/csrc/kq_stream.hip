@@ -767,10 +767,8 @@ bool gemv_stream_supported(const MatmulArgs& a)
 {
     // grouped calls: M counts (token, slot) pairs, each a matvec of its own
     if (!a.expert_idx && (a.M < 1 || a.M > 4)) return false;
-    // three and four tokens: Q4_K / Q6_K, plain calls, rows of at most 56 superblocks
-    if (!a.expert_idx && a.M > 2 &&
-        (a.n_blocks > 56 || a.pro != 0 || a.residual || (a.type != KQ_TYPE_Q4_K && a.type != KQ_TYPE_Q6_K)))
-        return false;
+    // three and four tokens: plain calls, rows of at most 56 superblocks
+    if (!a.expert_idx && a.M > 2 && (a.n_blocks > 56 || a.pro != 0 || a.residual)) return false;
     if (a.expert_idx && (a.M < 1 || a.M > 65535u || a.bias)) return false;
     if (((uintptr_t)a.X & 15u)) return false;
     if (a.n_blocks < 1) return false;
@@ -837,6 +835,11 @@ static hipError_t launch_stream_four(const MatmulArgs& a, hipStream_t s, const P
         else if (kw == 2) hipLaunchKernelGGL((q6k_stream_kernel<1, 2, 2, 4, PT>), grid, dim3(128), 0, s, p);
         else if (kw == 4) hipLaunchKernelGGL((q6k_stream_kernel<1, 4, 2, 4, PT>), grid, dim3(256), 0, s, p);
         else hipLaunchKernelGGL((q6k_stream_kernel<1, 7, 2, 4, PT>), grid, dim3(448), 0, s, p);
+    } else if (a.type == KQ_TYPE_Q5_K) {
+        if (kw == 1) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, true, 1>), grid, dim3(64), 0, s, p);
+        else if (kw == 2) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, true, 2>), grid, dim3(128), 0, s, p);
+        else if (kw == 4) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, true, 4>), grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, true, 7>), grid, dim3(448), 0, s, p);
     } else {
         if (kw == 1) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 1>), grid, dim3(64), 0, s, p);
         else if (kw == 2) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 2>), grid, dim3(128), 0, s, p);

@@ -96,6 +96,7 @@ def test_reference_recipe(gpu, kqo, name, family):
     (Q4_K, 3, 130, 2048), (Q4_K, 4, 300, 4096), (Q4_K, 3, 200, 8192), (Q4_K, 4, 100, 14336), (Q4_K, 4, 4096, 4096),
     (Q4_K, 3, 77, 6400),                       # 25 superblocks: the fourth K slice is partial
     (Q6_K, 4, 33, 768), (Q6_K, 3, 150, 4096), (Q6_K, 4, 120, 8192), (Q6_K, 3, 4096, 14336), (Q6_K, 4, 64, 2048),
+    (Q5_K, 3, 90, 1024), (Q5_K, 4, 300, 4096), (Q5_K, 4, 60, 8192), (Q5_K, 3, 50, 14336), (Q5_K, 4, 28672, 4096),
 ])
 def test_four_token_stream_kernels(gpu, kqo, type_, M, N, K):
     """Every K-slice count (1, 2, 4, 7 waves), three tokens run as four with the last masked: the rows of Y
@@ -117,7 +118,8 @@ def test_four_token_stream_kernels(gpu, kqo, type_, M, N, K):
 @pytest.mark.parametrize("M,N,K,kernel", [(1, 300, 4096, "gemv_stream"), (2, 64, 768, "gemv_stream"),
                                           (1, 4096, 4096, "gemv_stream"), (2, 6144, 4096, "gemv_stream"),
                                           (1, 77, 256, "gemv_stream"), (1, 500, 3072, "gemv_stream"),
-                                          (5, 130, 2048, "generic"), (17, 40, 512, "generic"),
+                                          (5, 130, 2048, "gemv_stream"), (17, 40, 512, "gemv_stream"), (4, 64, 768, "gemv_stream"),
+                                          (13, 700, 4096, "gemv_stream"), (70, 40, 512, "generic"),
                                           (1, 1000, 14336, "gemv_stream"), (2, 300, 8192, "gemv_stream"),
                                           (1, 200, 28672, "gemv_stream"), (2, 200, 28672, "generic"),
                                           (1, 50, 32768, "generic")])
