@@ -31,10 +31,12 @@ class WeightDesc(C.Structure):
 
 
 class Fusion(C.Structure):
-    _fields_ = [("prologue", C.c_int), ("norm_w", C.c_void_p), ("eps", C.c_float), ("residual", C.c_void_p)]
+    _fields_ = [("prologue", C.c_int), ("norm_w", C.c_void_p), ("eps", C.c_float), ("residual", C.c_void_p),
+                ("epilogue", C.c_int)]
 
 
 PRO_NONE, PRO_RMS_NORM, PRO_SILU_MUL, PRO_GELU_MUL = range(4)
+EPI_NONE, EPI_SILU_MUL, EPI_GELU_MUL = 0, 2, 3
 
 
 class GgufTensor(C.Structure):

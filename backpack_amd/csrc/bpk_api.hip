@@ -455,8 +455,9 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
 
 size_t bpk_kq_matmul_fused_workspace_bytes(uint32_t M, uint32_t N, uint32_t K)
 {
+    // the prologue's output [M, K] and the matmul's own output: [M, N], or [M, 2N] in front of an epilogue
     const size_t x = ((size_t)M * K * sizeof(float) + 255u) & ~(size_t)255u;
-    return x + (size_t)M * N * sizeof(float);
+    return x + 2u * (size_t)M * N * sizeof(float);
 }
 
 int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bias, float* Y, uint32_t M, uint32_t N,
@@ -466,10 +467,16 @@ int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bi
     if (!f) return fail(BPK_ERR_NULL, "fusion descriptor must be non-null");
     if (f->prologue < BPK_PRO_NONE || f->prologue > BPK_PRO_GELU_MUL)
         return fail(BPK_ERR_SHAPE, "prologue %d unknown", f->prologue);
+    if (f->epilogue != BPK_EPI_NONE && f->epilogue != BPK_EPI_SILU_MUL && f->epilogue != BPK_EPI_GELU_MUL)
+        return fail(BPK_ERR_SHAPE, "epilogue %d unknown", f->epilogue);
     if (f->prologue == BPK_PRO_RMS_NORM && !f->norm_w) return fail(BPK_ERR_NULL, "norm_w must be non-null for the norm prologue");
-    if (f->prologue == BPK_PRO_NONE && !f->residual)
+    const bool epi = f->epilogue != BPK_EPI_NONE;
+    if (epi && f->residual) return fail(BPK_ERR_SHAPE, "an epilogue takes no residual");
+    if (epi && N > 0x7FFFFFFFu) return fail(BPK_ERR_SHAPE, "N too large");
+    if (f->prologue == BPK_PRO_NONE && !f->residual && !epi)
         return bpk_kq_matmul(type, X, W, bias, Y, M, N, K, n_blocks, row_stride_words, y_offset, stream);
-    if (int rc = check_matmul(type, X, W, Y, M, N, K, n_blocks, row_stride_words)) return rc;
+    const uint32_t w_rows = epi ? 2u * N : N;   // rows of W
+    if (int rc = check_matmul(type, X, W, Y, M, w_rows, K, n_blocks, row_stride_words)) return rc;
     if (((uintptr_t)f->norm_w | (uintptr_t)f->residual) & 3u) return fail(BPK_ERR_ALIGN, "norm_w and residual must be 4-byte aligned");
     if (M == 0) return BPK_OK;
     DeviceState* st;
@@ -477,14 +484,14 @@ int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bi
     hipStream_t s = (hipStream_t)stream;
     kq::MatmulArgs a{};
     a.type = type; a.X = X; a.W = (const uint8_t*)W; a.bias = bias; a.Y = Y;
-    a.M = M; a.N = N; a.K = K; a.n_blocks = n_blocks;
+    a.M = M; a.N = w_rows; a.K = K; a.n_blocks = n_blocks;
     a.row_stride_bytes = row_stride_words * 4u;
     a.y_offset = y_offset;
     a.ldy = N;
     // one launch where the lanes-along-K kernel takes the shape
     if (!t_fused_separate && (t_family == 0 || t_family == 5)) {
-        a.pro = f->prologue; a.norm_w = f->norm_w; a.eps = f->eps; a.residual = f->residual;
-        if (kq::gemv_stream_supported(a) && N <= 32768u) {
+        a.pro = f->prologue; a.norm_w = f->norm_w; a.eps = f->eps; a.residual = f->residual; a.epi = f->epilogue;
+        if (kq::gemv_stream_supported(a) && w_rows <= 32768u) {
             t_kernel = "gemv_stream_fused";
             const hipError_t e = kq::launch_gemv_stream(a, t_gemv, s);
             return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
@@ -493,8 +500,8 @@ int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bi
     }
     // otherwise the same function in up to three launches through the caller's workspace
     const size_t x_bytes = ((size_t)M * K * sizeof(float) + 255u) & ~(size_t)255u;
-    const bool need_x = f->prologue != BPK_PRO_NONE, need_y = f->residual != nullptr;
-    const size_t need = (need_x ? x_bytes : 0) + (need_y ? (size_t)M * N * sizeof(float) : 0);
+    const bool need_x = f->prologue != BPK_PRO_NONE, need_y = f->residual != nullptr || epi;
+    const size_t need = (need_x ? x_bytes : 0) + (need_y ? (size_t)M * w_rows * sizeof(float) : 0);
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15u))
         return fail(BPK_ERR_WORKSPACE, "this shape needs a 16-byte aligned workspace of %zu bytes (given %zu)", need,
                     workspace ? workspace_bytes : (size_t)0);
@@ -504,10 +511,14 @@ int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bi
         const hipError_t e = kq::launch_prologue_rows(f->prologue, X, f->norm_w, f->eps, M, K, wx, s);
         if (e != hipSuccess) return hip_fail(e, "prologue_rows");
     }
-    if (int rc = bpk_kq_matmul(type, need_x ? wx : X, W, bias, need_y ? wy : Y, M, N, K, n_blocks, row_stride_words,
+    if (int rc = bpk_kq_matmul(type, need_x ? wx : X, W, bias, need_y ? wy : Y, M, w_rows, K, n_blocks, row_stride_words,
                                need_y ? 0u : y_offset, stream))
         return rc;
-    if (need_y) {
+    if (epi) {
+        // act(gate) * up of the [M, 2N] product rows -> Y rows (N apart, at y_offset)
+        const hipError_t e = kq::launch_prologue_rows(f->epilogue, wy, nullptr, 0.0f, M, N, Y + y_offset, s);
+        if (e != hipSuccess) return hip_fail(e, "act_mul_rows");
+    } else if (need_y) {
         const hipError_t e = kq::launch_add_residual(wy, f->residual, Y, M, N, N, y_offset, s);
         if (e != hipSuccess) return hip_fail(e, "add_residual");
     }

@@ -97,7 +97,7 @@ int gatherKQ(GGUFType type, const GPUBuffer& W, uint32_t rowStrideWords, const G
 int KQFusedDispatch::run(void* stream) const
 {
     const KQDispatch& d = base;
-    bpk_kq_fusion f{prologue, (const float*)NormW.ptr(), eps, (const float*)Residual.ptr()};
+    bpk_kq_fusion f{prologue, (const float*)NormW.ptr(), eps, (const float*)Residual.ptr(), epilogue};
     const int rc = bpk_kq_matmul_fused((int)d.type, (const float*)d.X.ptr(), d.W.ptr(), (const float*)d.Bias.ptr(),
                                        (float*)d.Y.ptr(), d.M, d.P.v[1], d.P.v[0], d.P.v[2], d.P.v[3], d.P.v[4], &f,
                                        Workspace.ptr(), Workspace.handle ? Workspace.size - Workspace.offset : 0, stream);

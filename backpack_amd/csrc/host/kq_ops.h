@@ -76,6 +76,7 @@ struct KQDispatch {
 struct KQFusedDispatch {
     KQDispatch base;
     int prologue = BPK_PRO_NONE;
+    int epilogue = BPK_EPI_NONE;   // base.W is then gate|up stacked and base.P.v[1] the number of outputs
     GPUBuffer NormW, Residual, Workspace;   // Workspace only for shapes that need separate launches
     float eps = 0.0f;
     int run(void* stream = nullptr) const;

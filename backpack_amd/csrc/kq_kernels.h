@@ -34,6 +34,9 @@ struct MatmulArgs {
     const float* norm_w = nullptr;
     float eps = 0.0f;
     const float* residual = nullptr;
+    // 2 / 3: W is gate | up stacked (N rows, N/2 outputs), Y[n] = silu / gelu_tanh (gate_n . x) * (up_n . x);
+    // Y rows are ldy apart
+    int epi = 0;
 };
 
 // Per-device scratch for split-K partial sums and arrival counters.

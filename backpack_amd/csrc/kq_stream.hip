@@ -20,6 +20,7 @@
 // its 16 activations, a per-lane constant.
 #include "kq_format.h"
 #include "kq_kernels.h"
+#include "kq_wave.h"
 #include <type_traits>
 
 namespace kq {
@@ -53,6 +54,9 @@ struct StreamFused {
     float eps;
     const float* norm_w;
     const float* residual;
+    // 0, or STREAM_PRO_SILU / STREAM_PRO_GELU: W is gate | up stacked (N rows in all, N/2 outputs) and
+    // Y[n] = act(gate_n . x) * (up_n . x): a wave takes both rows of a pair, one after the other
+    int epi;
     static constexpr bool kGrouped = false, kFused = true;
 };
 
@@ -108,6 +112,8 @@ __device__ __forceinline__ float stream_eps(const StreamFused& p) { return p.eps
 template <typename PT> __device__ __forceinline__ const float* stream_norm_w(const PT&) { return nullptr; }
 template <typename PT> __device__ __forceinline__ float stream_eps(const PT&) { return 0.0f; }
 __device__ __forceinline__ const float* stream_residual(const StreamFused& p) { return p.residual; }
+__device__ __forceinline__ int stream_epi(const StreamFused& p) { return p.epi; }
+template <typename PT> __device__ __forceinline__ int stream_epi(const PT&) { return 0; }
 template <typename PT> __device__ __forceinline__ const float* stream_residual(const PT&) { return nullptr; }
 __device__ __forceinline__ uint32_t stream_ldx(const StreamDense& p) { return p.K; }
 __device__ __forceinline__ uint32_t stream_ldx(const StreamFused& p) { return p.pro >= STREAM_PRO_SILU ? 2u * p.K : p.K; }
@@ -334,8 +340,18 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
     // rows gw, gw + stride, ...: at any moment the waves of the grid read
     // consecutive rows, one contiguous stream across the memory channels
     const uint32_t stride = KW > 1 ? gridDim.x : gridDim.x * NW;
-    if (gw >= p.N) return;   // KW > 1: the whole workgroup
-    const uint32_t n_rows = (p.N - gw + stride - 1u) / stride;
+    // pair mode (fused kernels only): the wave walks pairs gw, gw + stride, ... of the N/2 outputs and its
+    // ring alternates between a pair's gate row and its up row, N/2 rows further on
+    const bool pairs = PT::kFused && stream_epi(p) != 0;
+    const uint32_t n_walk_all = pairs ? p.N / 2u : p.N;
+    if (gw >= n_walk_all) return;   // KW > 1: the whole workgroup
+    const uint32_t n_walk = (n_walk_all - gw + stride - 1u) / stride;
+    const uint32_t n_rows = pairs ? 2u * n_walk : n_walk;
+    auto row_of = [&](uint32_t i) -> size_t {
+        i = min(i, n_rows - 1u);
+        if (PT::kFused && pairs) return (size_t)(gw + (i >> 1) * stride) + (size_t)(i & 1u) * n_walk_all;
+        return (size_t)(gw + i * stride);
+    };
     const uint32_t bl = lane >> 3, j = lane & 7u, g = j >> 1, h = j & 1u;
     const bool sel_hi = g >= 2u;
     const uint32_t sh = 16u * (g & 1u);
@@ -428,7 +444,7 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
     // must stay where they are, and across the prologue's arithmetic the compiler moves them.)
 #pragma unroll
     for (int d = 0; d < D; ++d)
-        ring[d].fill(p.W + (size_t)(gw + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, hoff, j);
+        ring[d].fill(p.W + row_of((uint32_t)d) * p.row_stride_bytes, hoff, j);
     // Rows are taken 64 at a time: lane i keeps the sums of the chunk's row i, and the
     // chunk is stored (bias added) after its last row.
     for (uint32_t c0 = 0; c0 < n_rows; c0 += 64u) {
@@ -448,7 +464,7 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
                 for (int pass = 0; pass < P; ++pass)
                     q4k_piece_dot<MT, Q5>(ring[d].hdr[pass], ring[d].q[pass], xlo[pass], xhi[pass], xs_lo[pass],
                                           xs_hi[pass], sel_hi, sh, acc, ring[d].qh[Q5 ? pass : 0], 2u * g);
-                ring[d].fill(p.W + (size_t)(gw + min(c0 + i + D, n_rows - 1u) * stride) * p.row_stride_bytes, hoff, j);
+                ring[d].fill(p.W + row_of(c0 + i + D) * p.row_stride_bytes, hoff, j);
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
                     const float tot = wave_sum(acc[t]);
@@ -461,13 +477,11 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
             for (int t = 0; t < MT; ++t) part[wave][t][lane] = res[t];
             __syncthreads();
         }
-        if ((KW == 1 || wave == 0) && lane < cnt) {
-            const uint32_t r = gw + (c0 + lane) * stride;
-            const float bias = p.bias ? p.bias[r] : 0.0f;
+        if (KW == 1 || wave == 0) {
+            const uint32_t r = (uint32_t)row_of(c0 + lane);   // (clamped past the end; those lanes do not store)
+            const float bias = (p.bias && lane < cnt) ? p.bias[r] : 0.0f;
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                if (MT > 2 && (uint32_t)t >= p.M) continue;
-                const size_t at = (size_t)t * p.ldy + p.y_offset + r;
                 float y = res[t];
                 if (KW > 1) {
                     y = part[0][t][lane];
@@ -475,6 +489,17 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
                     for (int w = 1; w < KW; ++w) y += part[w][t][lane];
                 }
                 y += bias;
+                if (PT::kFused && pairs) {
+                    // lanes 2j and 2j + 1 hold a pair's gate and up products: the even lane stores the output
+                    const float up = group_partner<1>(y);
+                    y = stream_epi(p) == STREAM_PRO_SILU ? stream_act<STREAM_PRO_SILU, true>(y, up)
+                                                         : stream_act<STREAM_PRO_GELU, true>(y, up);
+                    if (lane < cnt && !(lane & 1u)) p.Y[(size_t)t * p.ldy + p.y_offset + r] = y;
+                    continue;
+                }
+                if (MT > 2 && (uint32_t)t >= p.M) continue;
+                if (lane >= cnt) continue;
+                const size_t at = (size_t)t * p.ldy + p.y_offset + r;
                 if constexpr (PT::kFused) y += stream_residual(p) ? stream_residual(p)[at] : 0.0f;
                 p.Y[at] = y;
             }
@@ -778,10 +803,11 @@ bool gemv_stream_supported(const MatmulArgs& a)
         // the longest rows has no registers for Q5_K's third load or the fused forms
         if (a.n_blocks > 16 && a.expert_idx) return false;
         if (a.n_blocks > 112) return false;
-        if (a.n_blocks > 56 && a.M == 2 && (a.type == KQ_TYPE_Q5_K || a.pro != 0 || a.residual)) return false;
+        if (a.n_blocks > 56 && a.M == 2 && (a.type == KQ_TYPE_Q5_K || a.pro != 0 || a.residual || a.epi)) return false;
         if (((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u)) return false;
         return true;
     }
+    if (a.epi && (a.type == KQ_TYPE_Q6_K || a.expert_idx || a.M > 2 || (a.N & 1u))) return false;   // pair mode: Q4_K / Q5_K
     if (a.type == KQ_TYPE_Q6_K) {
         if (a.n_blocks > 112) return false;
         // the two-token kernel for the longest rows has no registers to spare for the fused forms
@@ -966,13 +992,14 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
         p.X2 = a.X2;
         return launch_stream_with(a, t, s, p, a.M, p.W2 ? 2u : 1u);   // grid.y = pairs, grid.z = twins
     }
-    if (a.pro != STREAM_PRO_NONE || a.residual) {
+    if (a.pro != STREAM_PRO_NONE || a.residual || a.epi) {
         StreamFused p;
         stream_fill_common(p, a);
         p.pro = a.pro;
         p.eps = a.eps;
         p.norm_w = a.norm_w;
         p.residual = a.residual;
+        p.epi = a.epi;
         return launch_stream_with(a, t, s, p, 1u, 1u);
     }
     StreamDense p;

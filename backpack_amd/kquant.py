@@ -131,24 +131,26 @@ def matmul(x: torch.Tensor, w: KQuantPacked, bias: torch.Tensor | None = None,
 def matmul_fused(x: torch.Tensor, w: KQuantPacked, prologue: int = capi.PRO_NONE, norm_w: torch.Tensor | None = None,
                  eps: float = 0.0, residual: torch.Tensor | None = None, bias: torch.Tensor | None = None,
                  out: torch.Tensor | None = None, workspace: torch.Tensor | None = None,
-                 allow_workspace: bool = True) -> torch.Tensor:
+                 allow_workspace: bool = True, epilogue: int = capi.EPI_NONE) -> torch.Tensor:
     """The decode matvec with what surrounds it folded in: RMSNorm of x, or act(gate)*up of a gate|up
-    row (x is then [M, 2K]), and a residual added to the output (residual may be `out`)."""
+    row (x is then [M, 2K]), and a residual added to the output (residual may be `out`).  With an
+    epilogue, w is the stacked gate|up matrix and the result is act(gate.x) * (up.x), [M, w.N / 2]."""
     assert x.is_cuda and x.is_contiguous() and x.dtype == torch.float32
     xk = w.K * (2 if prologue in (capi.PRO_SILU_MUL, capi.PRO_GELU_MUL) else 1)
     assert x.shape[-1] == xk
     M = x.numel() // xk
+    n_out = w.N // 2 if epilogue else w.N
     if out is None:
-        out = torch.empty((M, w.N), dtype=torch.float32, device=x.device)
+        out = torch.empty((M, n_out), dtype=torch.float32, device=x.device)
     L = capi.lib()
-    f = capi.Fusion(prologue, _ptr(norm_w), eps, _ptr(residual))
+    f = capi.Fusion(prologue, _ptr(norm_w), eps, _ptr(residual), epilogue)
     nbytes = 0
     if workspace is None and allow_workspace:
-        nbytes = L.bpk_kq_matmul_fused_workspace_bytes(M, w.N, w.K)
+        nbytes = L.bpk_kq_matmul_fused_workspace_bytes(M, n_out, w.K)
         workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
     elif workspace is not None:
         nbytes = workspace.numel() * workspace.element_size()
-    capi.check(L.bpk_kq_matmul_fused(w.type, _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out), M, w.N, w.K, w.n_blocks,
+    capi.check(L.bpk_kq_matmul_fused(w.type, _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out), M, n_out, w.K, w.n_blocks,
                                      w.row_stride_words, 0, f, _ptr(workspace), nbytes, _stream()))
     return out
 

@@ -297,9 +297,9 @@ def main():
 
 
 def fused_leg(mats, use_graph):
-    """The decode layer set with what surrounds two of its matvecs folded in: qkv reads x through RMSNorm,
-    down reads silu(gate)*up from the gate|up output and adds the residual in place.  Timed three ways on
-    the same weights: plain matvecs only (what the headline measures), fused (one launch each), and the
+    """The decode layer set with the dispatches around its matvecs folded in: qkv and gate|up read x through
+    RMSNorm, gate|up writes silu(gate)*up directly, o and down add the residual in place.  Timed three ways
+    on the same weights: plain matvecs only (what the headline measures), fused (one launch each), and the
     same function as separate launches (norm, act*mul, add beside the matvecs)."""
     import torch
     from backpack_amd import capi, kquant
@@ -311,12 +311,21 @@ def fused_leg(mats, use_graph):
     ws = torch.empty(capi.lib().bpk_kq_matmul_fused_workspace_bytes(1, max(w.N for _, w, _, _ in mats), inter),
                      dtype=torch.uint8, device="cuda")
 
+    act = torch.zeros(1, inter, device="cuda")
+
     def fused_pass():
+        # a layer's four matvecs with the five dispatches around them folded in: attn_norm -> qkv,
+        # o -> + residual, ffn_norm -> gate|up -> act * up, down -> + residual
         for name, w, x, y in mats:
             if name == "qkv":
                 kquant.matmul_fused(x, w, capi.PRO_RMS_NORM, norm_w=norm_w, eps=1e-5, out=y, workspace=ws)
+            elif name == "o":
+                kquant.matmul_fused(x, w, residual=resid, out=resid, workspace=ws)
+            elif name == "gate_up":
+                kquant.matmul_fused(x, w, capi.PRO_RMS_NORM, norm_w=norm_w, eps=1e-5, out=act, workspace=ws,
+                                    epilogue=capi.EPI_SILU_MUL)
             elif name == "down":
-                kquant.matmul_fused(gate_up, w, capi.PRO_SILU_MUL, residual=resid, out=resid, workspace=ws)
+                kquant.matmul_fused(act, w, residual=resid, out=resid, workspace=ws)
             else:
                 kquant.matmul(x, w, out=y)
 
@@ -360,8 +369,8 @@ def fused_leg(mats, use_graph):
             capi.check(capi.lib().bpk_argmax_rows(logits.data_ptr(), 1, logits.shape[1], logits.shape[1], idx.data_ptr(),
                                                   val.data_ptr(), torch.cuda.current_stream().cuda_stream))
     res["argmax_us"] = round(timed(picks) * 1e3 / 50, 2)
-    n = sum(1 for name, *_ in mats if name in ("qkv", "down"))
-    res["launches_saved"] = int(n * 1.5)     # norm per qkv; act*mul and add per down
+    n = sum(1 for name, *_ in mats if name == "qkv")
+    res["launches_saved"] = 5 * n     # per layer: two norms, act*mul, two residual adds
     return res
 
 

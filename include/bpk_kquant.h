@@ -221,17 +221,27 @@ BPK_API int bpk_kq_matmul(int type, const float *X, const void *W,
  * 0.044715 g^3))).  residual may be NULL (= zeros) and may be Y itself (the
  * in-place add).  M <= 2 with rows the decode kernel holds in registers
  * (K <= 28672 for one token, K <= 14336 for two; N <= 32768) is one launch
- * and needs no workspace.  Other shapes run the same function as prologue, matmul and add
- * launches through `workspace` (device memory, 16-byte aligned, at least
- * bpk_kq_matmul_fused_workspace_bytes(M, N, K) bytes) and fail with
- * BPK_ERR_WORKSPACE without it. */
+ * and needs no workspace.  Other shapes run the same function as prologue,
+ * matmul and add launches through `workspace` (device memory, 16-byte aligned,
+ * at least bpk_kq_matmul_fused_workspace_bytes(M, N, K) bytes) and fail with
+ * BPK_ERR_WORKSPACE without it.
+ *
+ * Epilogue BPK_EPI_SILU_MUL / BPK_EPI_GELU_MUL folds the same activation into
+ * the gate|up matvec instead: W is the stacked gate|up matrix of 2N rows
+ * (gate rows first), N counts the outputs, and
+ *   Y[m*N + y_offset + n] = act(bias[n] + gate_n . x[m]) * (bias[N+n] + up_n . x[m])
+ * so the 2N-float gate|up buffer is never written (the down matvec then takes
+ * Y as a plain X).  bias is f32 [2N] or NULL; residual must be NULL.  One launch
+ * for Q4_K / Q5_K with M <= 2; other shapes go through the workspace. */
 enum { BPK_PRO_NONE = 0, BPK_PRO_RMS_NORM = 1, BPK_PRO_SILU_MUL = 2, BPK_PRO_GELU_MUL = 3 };
+enum { BPK_EPI_NONE = 0, BPK_EPI_SILU_MUL = 2, BPK_EPI_GELU_MUL = 3 };
 
 typedef struct bpk_kq_fusion {
     int prologue;          /* BPK_PRO_*                               */
     const float *norm_w;   /* f32 [K] (device), BPK_PRO_RMS_NORM only */
     float eps;             /* BPK_PRO_RMS_NORM only                   */
     const float *residual; /* f32 (device), indexed like Y, or NULL   */
+    int epilogue;          /* BPK_EPI_*                               */
 } bpk_kq_fusion;
 
 BPK_API size_t bpk_kq_matmul_fused_workspace_bytes(uint32_t M, uint32_t N,

@@ -135,7 +135,67 @@ def test_fused_argument_checks(gpu):
         return L.bpk_kq_matmul_fused(Q4_K, x.data_ptr(), w.data.data_ptr(), None, y.data_ptr(), 1, 8, 256, 1, 36, 0,
                                      f, None, 0, None)
     assert call(None) == -3
-    assert call(C.byref(capi.Fusion(7, None, 0.0, None))) == -2
-    assert call(C.byref(capi.Fusion(capi.PRO_RMS_NORM, None, 1e-5, None))) == -3
-    assert call(C.byref(capi.Fusion(capi.PRO_NONE, None, 0.0, None))) == 0     # plain matmul
-    assert L.bpk_kq_matmul_fused_workspace_bytes(3, 10, 256) == 3 * 256 * 4 + 3 * 10 * 4
+    assert call(C.byref(capi.Fusion(7, None, 0.0, None, 0))) == -2
+    assert call(C.byref(capi.Fusion(capi.PRO_RMS_NORM, None, 1e-5, None, 0))) == -3
+    assert call(C.byref(capi.Fusion(capi.PRO_NONE, None, 0.0, None, 0))) == 0     # plain matmul
+    assert L.bpk_kq_matmul_fused_workspace_bytes(3, 10, 256) == 3 * 256 * 4 + 2 * 3 * 10 * 4
+
+
+# ---- epilogue: act(gate . x) * (up . x) out of the stacked gate|up matvec -------------------------
+EPI = [
+    # type, M, N outputs, K, epilogue, prologue, bias, expected kernel
+    (Q4_K, 1, 14336, 4096, SILU, NONE, False, "gemv_stream_fused"),     # the decode FFN head at its real shape
+    (Q4_K, 2, 300, 4096, GELU, NONE, True, "gemv_stream_fused"),
+    (Q4_K, 1, 257, 2048, SILU, NORM, False, "gemv_stream_fused"),       # ffn_norm folded in as well
+    (Q4_K, 1, 100, 8192, SILU, NONE, False, "gemv_stream_fused"),       # K slices over four waves
+    (Q4_K, 2, 64, 14336, GELU, NORM, True, "gemv_stream_fused"),        # ... over seven, two tokens
+    (13, 1, 500, 4096, SILU, NONE, False, "gemv_stream_fused"),         # Q5_K
+    (Q4_K, 1, 33, 256, SILU, NONE, False, "gemv_stream_fused"),         # fewer pairs than waves
+    (Q6_K, 1, 200, 2048, SILU, NONE, False, None),                      # workspace path: Q6_K gate|up
+    (Q4_K, 5, 120, 1024, GELU, NORM, True, None),                       # ... more than two tokens
+]
+
+
+@pytest.mark.parametrize("type_,M,N,K,epi,pro,with_bias,kernel", EPI)
+def test_fused_gate_up_epilogue(gpu, kqo, type_, M, N, K, epi, pro, with_bias, kernel):
+    from backpack_amd import capi, kquant
+    print("fused epilogue", type_, M, N, K, epi, pro, with_bias, flush=True)
+    rng = np.random.default_rng(N + K + M)
+    raw, packed, w = gpu.make_weight(type_, 2 * N, K, seed=N)            # gate rows, then up rows
+    X = rng.standard_normal((M, K)).astype(np.float32)
+    norm_w = (1 + 0.1 * rng.standard_normal(K)).astype(np.float32) if pro == NORM else None
+    bias = (0.1 * rng.standard_normal(2 * N)).astype(np.float32) if with_bias else None
+    xp = X if pro == NONE else kqo.prologue(pro, X, K, norm_w=norm_w, eps=1e-5)
+    gate_up = kqo.matmul(type_, xp, packed, 2 * N, K, bias=bias)          # [M, 2N] = gate | up
+    want = kqo.prologue(epi, gate_up, N)
+    args = dict(norm_w=gpu.dev(norm_w) if norm_w is not None else None, eps=1e-5,
+                bias=gpu.dev(bias) if bias is not None else None, epilogue=epi)
+    if kernel is None:
+        with pytest.raises(capi.BpkError) as e:
+            kquant.matmul_fused(gpu.dev(X), w, pro, allow_workspace=False, **args)
+        assert e.value.code == -7
+    y = kquant.matmul_fused(gpu.dev(X), w, pro, allow_workspace=kernel is None, **args)
+    if kernel is not None:
+        assert capi.last_kernel() == kernel
+    got = y.cpu().numpy()
+    assert got.shape == (M, N)
+    # the product of two fp32 matvec results, each good to ~1e-6 of its rms: 2e-4 of the output's scale
+    # leaves room for the device's exponential as well
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    assert np.all(np.abs(got - want) <= 2e-4 * (rms + np.abs(want))), float(np.abs(got - want).max())
+
+
+def test_fused_epilogue_argument_checks(gpu):
+    import ctypes as C
+    from backpack_amd import capi
+    raw, packed, w = gpu.make_weight(Q4_K, 16, 256, seed=1)
+    x = gpu.dev(np.zeros((1, 256), np.float32))
+    y = gpu.dev(np.zeros((1, 8), np.float32))
+    L = capi.lib()
+
+    def call(f):
+        return L.bpk_kq_matmul_fused(Q4_K, x.data_ptr(), w.data.data_ptr(), None, y.data_ptr(), 1, 8, 256, 1, 36, 0,
+                                     C.byref(f), None, 0, None)
+    assert call(capi.Fusion(capi.PRO_NONE, None, 0.0, None, 1)) == -2                  # unknown epilogue
+    assert call(capi.Fusion(capi.PRO_NONE, None, 0.0, y.data_ptr(), capi.EPI_SILU_MUL)) == -2   # residual with epilogue
+    assert call(capi.Fusion(capi.PRO_NONE, None, 0.0, None, capi.EPI_SILU_MUL)) == 0
