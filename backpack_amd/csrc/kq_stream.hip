@@ -477,9 +477,11 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
             for (int t = 0; t < MT; ++t) part[wave][t][lane] = res[t];
             __syncthreads();
         }
-        if (KW == 1 || wave == 0) {
-            const uint32_t r = (uint32_t)row_of(c0 + lane);   // (clamped past the end; those lanes do not store)
-            const float bias = (p.bias && lane < cnt) ? p.bias[r] : 0.0f;
+        // (the lane guard stays outside: with it inside, the gate|up launch measured 3 us slower.  In pair
+        // mode cnt is even, so a lane inside the guard finds its partner there too.)
+        if ((KW == 1 || wave == 0) && lane < cnt) {
+            const uint32_t r = (uint32_t)row_of(c0 + lane);
+            const float bias = p.bias ? p.bias[r] : 0.0f;
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 float y = res[t];
@@ -494,11 +496,10 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
                     const float up = group_partner<1>(y);
                     y = stream_epi(p) == STREAM_PRO_SILU ? stream_act<STREAM_PRO_SILU, true>(y, up)
                                                          : stream_act<STREAM_PRO_GELU, true>(y, up);
-                    if (lane < cnt && !(lane & 1u)) p.Y[(size_t)t * p.ldy + p.y_offset + r] = y;
+                    if (!(lane & 1u)) p.Y[(size_t)t * p.ldy + p.y_offset + r] = y;
                     continue;
                 }
                 if (MT > 2 && (uint32_t)t >= p.M) continue;
-                if (lane >= cnt) continue;
                 const size_t at = (size_t)t * p.ldy + p.y_offset + r;
                 if constexpr (PT::kFused) y += stream_residual(p) ? stream_residual(p)[at] : 0.0f;
                 p.Y[at] = y;
@@ -819,7 +820,7 @@ bool gemv_stream_supported(const MatmulArgs& a)
 }
 
 // Launches of one instantiation.  Not every combination exists: grouped launches are one token per
-// pair, the fused forms run two rows in flight per wave whatever the depth option says, and the
+// pair, the fused forms run two rows in flight per wave (the Q4_K kernel also four, for one token), and the
 // two-token Q6_K kernel for the longest rows has no registers to spare for the fused forms
 // (gemv_stream_supported declines those calls).
 template <int P, int KW, int D, int MT, typename PT>
@@ -834,7 +835,8 @@ static void launch_q6k_one(dim3 grid, hipStream_t s, const PT& p)
 template <int P, int NW, int D, int MT, typename PT, bool Q5>
 static void launch_q4k_one(dim3 grid, hipStream_t s, const PT& p)
 {
-    constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && D != 2) || (Q5 && (PT::kGrouped || D > 2));
+    constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && (D == 1 || (D == 4 && MT == 2))) ||
+                            (Q5 && (PT::kGrouped || D > 2));
     if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT, Q5>), grid, dim3(64 * NW), 0, s, p);
 }
 
@@ -941,8 +943,9 @@ static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, h
     uint32_t wgs = t.splits > 0 ? ((a.N + (uint32_t)t.splits - 1u) / (uint32_t)t.splits + NW - 1u) / NW
                                 : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
     wgs = (wgs + pairs * twins - 1u) / (pairs * twins);
-    int depth = PT::kFused ? 2 : t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
+    int depth = t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
     if (q5 && depth > 2) depth = 2;
+    if (PT::kFused) depth = depth >= 4 && !two ? 4 : 2;   // the fused forms come with two or four rows in flight
     const dim3 grid(wgs, pairs, twins);
 #define KQ_STREAM_LAUNCH(P, D) \
     do { \
