@@ -428,10 +428,12 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     }
     if (t_family == 5 && !stream_ok) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");
     if (t_family == 4) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
-    // up to a few tens of thousands of rows the lanes-along-K kernel wins at M = 1
-    // (no LDS staging, no K split to fold); longer matrices reach a steady state
-    // in which the row-per-lane kernel streams faster
-    if (t_family == 5 || (t_family == 0 && stream_ok && N <= 32768u && (M <= 2 || stream_four))) {
+    // The lanes-along-K kernel (no LDS staging, no K split to fold) wins everywhere except on Q6_K matrices
+    // of more than a few tens of thousands of rows at one token, where the row-per-lane kernel reaches a
+    // faster steady state (128256 x 4096: 90 against 97 us; at two tokens 129 against 102 us, and Q4_K of
+    // that size 152 against 82 us).
+    const bool stream_rows_ok = N <= 32768u || M == 2u || type != BPK_TYPE_Q6_K;
+    if (t_family == 5 || (t_family == 0 && stream_ok && ((M <= 2 && stream_rows_ok) || stream_four))) {
         t_kernel = "gemv_stream";
         e = kq::launch_gemv_stream(a, t_gemv, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
