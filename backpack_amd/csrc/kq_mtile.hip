@@ -80,6 +80,7 @@ struct MtileParams {
     // 16 (Q4_K) / 8 (Q6_K) (token, slot) pairs that share an expert; N is the rows of one expert
     const uint32_t* tiles;
     const uint32_t* n_tiles;
+    uint32_t tile_iters;    // grouped calls whose K is a single chunk: tiles a wave walks with X staged once
     uint32_t tile_stride;   // words per record
     uint32_t k_slots;
     int x_per_slot;         // X row of a pair: the pair itself (1) or its token, pair / k_slots (0)
@@ -521,6 +522,30 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     stager.init(p, rec, count);
     stager.fetch(p, c_begin);
     t_f32x4 tot = {0, 0, 0, 0};
+    // a finished tile: lane l holds tokens 4*(l/16) .. +3 of weight row row_t
+    auto put_tile = [&](uint32_t row_t, const t_f32x4& t) {
+        if (row_t < p.N && (!Q6 || kq < 2u)) {
+            const float bias = p.bias ? p.bias[row_t] : 0.0f;
+            const float t4[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t token = 4u * kq + r;
+                if (token < count) {
+                    const uint32_t yrow = rec ? rec[2u + token] : token;
+                    p.Y[(size_t)yrow * p.ldy + p.y_offset + row_t] = t4[r] + bias;
+                }
+            }
+        }
+    };
+    auto store_tile = [&](uint32_t row_t, t_f32x4 t) {
+        if constexpr (Q6) {   // lanes l and l + 32 hold the two 16-element halves of the same tokens
+            t.x += __shfl_xor(t.x, 32, 64);
+            t.y += __shfl_xor(t.y, 32, 64);
+            t.z += __shfl_xor(t.z, 32, 64);
+            t.w += __shfl_xor(t.w, 32, 64);
+        }
+        put_tile(row_t, t);
+    };
     if constexpr (STAGED) {
 #pragma unroll
     for (int h = 0; h < PASSES; ++h) ws[h].load(pass_block(c_begin, h) * BB, row_bytes);
@@ -569,8 +594,15 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     for (uint32_t i = threadIdx.x; i < MT_STAGE_BYTES / 16; i += 64 * NW)
         ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
     __syncthreads();
-    const uint8_t* wrow = wmat + (size_t)min(row, p.N - 1u) * p.row_stride_bytes;
+    // A grouped call whose K fits one chunk stages the record's X once and lets every wave walk `iters` tiles
+    // with it (no barrier after the first): such workgroups are otherwise mostly set-up.
+    const uint32_t iters = (R == NW && p.tiles) ? p.tile_iters : 1u;
     constexpr int BPC = R == 1 ? (MT_KC + NW - 1) / NW : MT_KC;   // superblocks of a chunk this wave takes
+    for (uint32_t it = 0; it < iters; ++it) {
+    const uint32_t tile_i = iters > 1u ? (blockIdx.x * iters + it) * p.tiles_per_wg + wave : tile;
+    const uint32_t row_i = has_tile ? tile_i * 16u + (lane & 15u) : p.N;
+    if (iters > 1u) tot = t_f32x4{0, 0, 0, 0};
+    const uint8_t* wrow = wmat + (size_t)min(row_i, p.N - 1u) * p.row_stride_bytes;
     for (uint32_t c0 = c_begin; c0 < c_end; c0 += MT_KC) {
         // the chunk's weights are requested first, so that their latency runs under the conversion of X
         t_u32x4 hdr[BPC];
@@ -589,9 +621,11 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                 for (int g = 0; g < 4; ++g) w[i][g] = *(const t_u32x2*)(blk + 16u + 32u * g + 8u * kq);
             }
         }
-        stager.park(xa, xs, xinv, xv);
-        __syncthreads();
-        if (c0 + MT_KC < c_end) stager.fetch(p, c0 + MT_KC);   // the next chunk of X travels while this one is multiplied
+        if (it == 0u) {
+            stager.park(xa, xs, xinv, xv);
+            __syncthreads();
+            if (c0 + MT_KC < c_end) stager.fetch(p, c0 + MT_KC);   // the next chunk of X travels while this one is multiplied
+        }
         if (has_tile) {
 #pragma unroll
             for (int i = 0; i < BPC; ++i) {
@@ -604,8 +638,11 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                 }
             }
         }
-        __syncthreads();
+        if (iters == 1u) __syncthreads();   // (with iters > 1 there is one chunk and X stays where it is)
     }
+    if (iters > 1u) store_tile(row_i, tot);
+    }
+    if (iters > 1u) return;
     }
 
     if (R == 1) {
@@ -658,18 +695,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         }
         if (threadIdx.x == 0) __hip_atomic_store(&p.counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (row < p.N && (!Q6 || kq < 2u)) {
-        const float bias = p.bias ? p.bias[row] : 0.0f;
-        const float t4[4] = {tot.x, tot.y, tot.z, tot.w};
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t token = 4u * kq + r;
-            if (token < count) {
-                const uint32_t yrow = rec ? rec[2u + token] : token;
-                p.Y[(size_t)yrow * p.ldy + p.y_offset + row] = t4[r] + bias;
-            }
-        }
-    }
+    put_tile(row, tot);
 }
 
 bool mtile_supported(const MatmulArgs& a)
@@ -728,12 +754,18 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
     // one or two chunks and are bound by their latencies, so two must share a CU: Q4_K runs 8 tiles per
     // workgroup at 128 registers, Q6_K (160 registers) 4 tiles per workgroup of 4 waves.
     const uint32_t row_tiles = (a.N + 15u) / 16u;
-    if (a.type == KQ_TYPE_Q6_K) {
-        p.tiles_per_wg = 4;
-        return launch_mtile_one<KQ_TYPE_Q6_K, 4, 4, false>(p, (row_tiles + 3u) / 4u, tiles_bound, s, slices);
+    const uint32_t tpw = a.type == KQ_TYPE_Q6_K ? 4u : 8u;
+    p.tiles_per_wg = tpw;
+    // one chunk of K: every wave walks up to 8 tiles with the record's X staged once, as long as a record
+    // still spreads over four workgroups
+    p.tile_iters = 1;
+    if (p.chunks_per_split == 1u) {
+        const uint32_t groups = (row_tiles + tpw - 1u) / tpw;
+        p.tile_iters = groups >= 32u ? 8u : groups >= 16u ? 4u : groups >= 8u ? 2u : 1u;
     }
-    p.tiles_per_wg = 8;
-    return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, false>(p, (row_tiles + 7u) / 8u, tiles_bound, s, slices);
+    const uint32_t wgs = (row_tiles + tpw * p.tile_iters - 1u) / (tpw * p.tile_iters);
+    if (a.type == KQ_TYPE_Q6_K) return launch_mtile_one<KQ_TYPE_Q6_K, 4, 4, false>(p, wgs, tiles_bound, s, slices);
+    return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, false>(p, wgs, tiles_bound, s, slices);
 }
 
 hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s)
@@ -781,7 +813,7 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
         p.y_offset = a.y_offset;
         p.ldy = a.ldy;
         p.tiles_per_wg = 1;
-        p.tiles = nullptr; p.n_tiles = nullptr; p.tile_stride = 0; p.k_slots = 1; p.x_per_slot = 0;
+        p.tiles = nullptr; p.n_tiles = nullptr; p.tile_stride = 0; p.tile_iters = 1; p.k_slots = 1; p.x_per_slot = 0;
         p.n_splits = 1; p.chunks_per_split = n_chunks; p.partial = sc.partial; p.counters = sc.counters;
         hipError_t e;
         if (shared_tile) {

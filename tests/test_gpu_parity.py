@@ -564,7 +564,10 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
 
 
 @pytest.mark.parametrize("family,kernel", [(0, "mtile_grouped"), (3, "mrow_grouped")])
-@pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True)])
+@pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True),
+                                                 # K of one chunk: waves walk several tiles per staged X; ragged last tile
+                                                 (Q6_K, 2000, 768, True), (Q4_K, 1104, 1024, False),
+                                                 (Q6_K, 520, 512, False)])
 def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot, family, kernel):
     """Ragged lists: some experts get many pairs, some none; repeated experts inside a token."""
     from backpack_amd import capi, kquant
