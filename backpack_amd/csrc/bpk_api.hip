@@ -20,6 +20,8 @@ namespace {
 constexpr int kMaxDevices = 16;
 constexpr size_t kPartialFloats = size_t(4) << 20;  // 16 MiB of split-K partial sums
 constexpr uint32_t kCounters = 1u << 16;
+// bf16 GEMM: two 256 x 256 fp32 slots per workgroup for the runs of cut tiles, a workgroup per CU
+constexpr size_t kGemmPartialFloats = size_t(2) * 256 * 65536;  // 128 MiB
 constexpr size_t kMoeWords = size_t(4) << 20;       // 16 MiB of tile records for bpk_kq_moe_matmul
 
 thread_local char t_err[512] = "";
@@ -69,6 +71,7 @@ struct UploadStage {
 struct DeviceState {
     bool ready = false;
     kq::SplitScratch split{};
+    kq::SplitScratch gemm_split{};   // of the bf16 GEMM's cut tiles (its own, so that it can run beside a GEMV)
     uint32_t* moe_tiles = nullptr;   // kMoeWords words
     uint32_t* argmax_scratch = nullptr;   // partial values | partial indices | tickets of bpk_argmax_rows
     float* route_logits = nullptr;   // ROUTE_SPREAD_TOKENS x 1024 router logits of a small-T route call
@@ -96,6 +99,9 @@ int ensure_device(int device, DeviceState** out)
         e = hipMalloc((void**)&st.split.partial, kPartialFloats * sizeof(float));
         if (e == hipSuccess) e = hipMalloc((void**)&st.split.counters, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMemset(st.split.counters, 0, kCounters * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipMalloc((void**)&st.gemm_split.partial, kGemmPartialFloats * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc((void**)&st.gemm_split.counters, kCounters * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipMemset(st.gemm_split.counters, 0, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMalloc((void**)&st.moe_tiles, kMoeWords * sizeof(uint32_t));
         constexpr size_t kArgmaxWords = (size_t)kq::ARGMAX_MAX_ROWS * (2u * kq::ARGMAX_PARTS + 1u);
         if (e == hipSuccess) e = hipMalloc((void**)&st.argmax_scratch, kArgmaxWords * sizeof(uint32_t));
@@ -105,6 +111,8 @@ int ensure_device(int device, DeviceState** out)
         if (e != hipSuccess) return hip_fail(e, "allocating split-K scratch");
         st.split.capacity_floats = kPartialFloats;
         st.split.n_counters = kCounters;
+        st.gemm_split.capacity_floats = kGemmPartialFloats;
+        st.gemm_split.n_counters = kCounters;
         st.ready = true;
     }
     if (out) *out = &st;
@@ -532,7 +540,8 @@ int bpk_kq_matmul_bf16(int type, const uint16_t* X, const void* W, const float* 
 {
     if (int rc = check_matmul(type, X, W, Y, M, N, K, n_blocks, row_stride_words)) return rc;
     if (M == 0) return BPK_OK;
-    if (int rc = current_state(nullptr)) return rc;
+    DeviceState* st = nullptr;
+    if (int rc = current_state(&st)) return rc;
     kq::MatmulArgs a{};
     a.type = type; a.X = X; a.W = (const uint8_t*)W; a.bias = bias; a.Y = Y;
     a.M = M; a.N = N; a.K = K; a.n_blocks = n_blocks;
@@ -542,7 +551,7 @@ int bpk_kq_matmul_bf16(int type, const uint16_t* X, const void* W, const float* 
     if (!kq::gemm_bf16_supported(a))
         return fail(BPK_ERR_ALIGN, "bf16 GEMM needs 16-byte aligned X and (for Q4_K) 16-byte aligned W rows");
     t_kernel = "gemm_bf16";
-    hipError_t e = kq::launch_gemm_bf16(a, t_gemm_tile, t_gemm_split, (hipStream_t)stream);
+    hipError_t e = kq::launch_gemm_bf16(a, t_gemm_tile, t_gemm_split, st->gemm_split, (hipStream_t)stream);
     return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
 }
 

@@ -38,6 +38,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GEMM_BK = 64;
@@ -52,6 +53,8 @@ struct GemmParams {
     // walk of the persistent kernel: units = k steps (of 64) of all 256 x 256 tiles, tile after tile
     // (tiles of one token block next to each other), cut into equal shares
     uint32_t tiles_n, units, units_per_wg;
+    // runs that cover part of a tile leave their sums here: two slots of 256 x 256 floats per workgroup
+    float* partial;
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
@@ -572,33 +575,62 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
         slice_schedule();
     }
 
-    // a tile walked in one piece is stored; a tile cut between workgroups is summed into Y, which the
-    // launcher cleared for exactly those tiles (the bias goes in with the segment that starts at k = 0)
-    if (nk == nk_all) store_acc<TM, TN, false>(p, acc, m0 + wm * WM, n0 + wn * WN, lane);
-    else store_acc<TM, TN, true>(p, acc, m0 + wm * WM, n0 + wn * WN, lane, k_first == 0u);
+    // A tile walked in one piece is stored.  A run over part of a tile leaves its sums in the workspace, in
+    // register order (a wave writes 1 KB per instruction): slot 2b of workgroup b if the run starts the
+    // workgroup's share, slot 2b+1 if it ends it.  gemm_sum_cut_tiles_kernel adds the runs of each cut tile
+    // in the order of the walk afterwards, so the result does not depend on timing.
+    if (nk == nk_all) {
+        store_acc<TM, TN>(p, acc, m0 + wm * WM, n0 + wn * WN, lane);
+    } else {
+        const uint32_t slot = 2u * blockIdx.x + (blockIdx.x * p.units_per_wg < tile * nk_all ? 1u : 0u);
+        f32x4* dst = (f32x4*)(p.partial + (size_t)slot * 65536u) + wave * 2048u + lane;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    dst[((i * TN + j) * 4 + r) * 64] =
+                        f32x4{acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2], acc[i][j][4 * r + 3]};
+    }
     __syncthreads();   // the next segment's prologue overwrites LDS
     }
 }
 
-// Clears the tiles of Y that the persistent kernel's cut points split: block b looks at the boundary
-// between workgroups b and b+1.
-__global__ __launch_bounds__(256) void gemm_clear_split_tiles_kernel(GemmParams p)
+// Sums the runs of the tiles that the persistent kernel's cut points split, adds the bias and stores Y.
+// blockIdx.x = cut point (between workgroups b and b+1 of the walk), blockIdx.y = which of the 8
+// accumulator blocks of every wave's 128 x 64 share; thread = (wave, lane) of the persistent kernel.  The
+// first cut point inside a tile serves the tile.
+__global__ __launch_bounds__(512) void gemm_sum_cut_tiles_kernel(GemmParams p)
 {
-    const uint32_t nk_all = p.K / GEMM_BK;
-    const uint32_t cut = (blockIdx.x + 1u) * p.units_per_wg;
+    const uint32_t nk_all = p.K / GEMM_BK, share = p.units_per_wg;
+    const uint32_t cut = (blockIdx.x + 1u) * share;
     if (cut >= p.units || cut % nk_all == 0u) return;
-    const uint32_t tile = cut / nk_all;
-    const uint32_t m0 = (tile / p.tiles_n) * 256u, n0 = (tile % p.tiles_n) * 256u;
-    const uint32_t rows = min(256u, p.M - m0);
-    if (n0 + 256u <= p.N && (((uintptr_t)p.Y | ((uintptr_t)p.ldy * 4u)) & 15u) == 0u) {
-        // whole 1 KB rows, 16 bytes per lane: a wave clears a row per store
-        float4* y = (float4*)(p.Y + (size_t)m0 * p.ldy + n0) + (threadIdx.x & 63u);
-        for (uint32_t r = threadIdx.x >> 6; r < rows; r += 4u) y[(size_t)r * (p.ldy / 4u)] = float4{0.0f, 0.0f, 0.0f, 0.0f};
-    } else {
-        const uint32_t n = n0 + threadIdx.x;
-        if (n < p.N)
-            for (uint32_t r = 0; r < rows; ++r) p.Y[(size_t)(m0 + r) * p.ldy + n] = 0.0f;
+    const uint32_t tile = cut / nk_all, tile_u = tile * nk_all;
+    if (blockIdx.x * share > tile_u) return;   // an earlier cut point lies inside the same tile
+    const uint32_t b_first = blockIdx.x, b_last = min((tile_u + nk_all - 1u) / share, (p.units - 1u) / share);
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, g = blockIdx.y;
+    f32x4 sum[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) sum[r] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t b = b_first; b <= b_last; ++b) {
+        const uint32_t slot = 2u * b + (b * share < tile_u ? 1u : 0u);
+        const f32x4* src = (const f32x4*)(p.partial + (size_t)slot * 65536u) + wave * 2048u + g * 256u + lane;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sum[r] += src[r * 64];
     }
+    // register 4r+e of block (i, j) of wave (wm, wn): token row 8r + 4*(lane/32) + e, weight row lane%32
+    const uint32_t m0 = (tile / p.tiles_n) * 256u + (wave >> 2) * 128u + (g >> 1) * 32u + 4u * (lane >> 5);
+    const uint32_t n = (tile % p.tiles_n) * 256u + (wave & 3u) * 64u + (g & 1u) * 32u + (lane & 31u);
+    if (n >= p.N) return;
+    const float bias = p.bias ? p.bias[n] : 0.0f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t m = m0 + 8u * r + e;
+            if (m < p.M) p.Y[(size_t)m * p.ldy + n] = sum[r][e] + bias;
+        }
 }
 
 bool gemm_bf16_supported(const MatmulArgs& a)
@@ -632,7 +664,7 @@ static hipError_t launch_gemm(const GemmParams& p, hipStream_t s)
 // 256-tile kernel.  share = k steps per workgroup: nk for one tile per workgroup, otherwise the walk over all
 // (tile, k step) units is cut into runs of that length.
 template <int TYPE>
-static hipError_t launch_gemm_persistent(GemmParams p, uint32_t share, hipStream_t s)
+static hipError_t launch_gemm_persistent(GemmParams p, uint32_t share, const SplitScratch& sc, hipStream_t s)
 {
     constexpr size_t shmem = 2 * (size_t)(256 + 256) * GEMM_LD;
     auto kern = gemm_bf16_sk_kernel<TYPE>;
@@ -646,15 +678,18 @@ static hipError_t launch_gemm_persistent(GemmParams p, uint32_t share, hipStream
     p.tiles_n = (p.N + 255u) / 256u;
     const uint32_t tiles = ((p.M + 255u) / 256u) * p.tiles_n;
     p.units = tiles * nk;
+    // cut tiles need two workspace slots per workgroup: without them, whole tiles
+    if ((size_t)2u * ((p.units + share - 1u) / share) * 65536u > sc.capacity_floats) share = nk;
     p.units_per_wg = share;
+    p.partial = sc.partial;
     const uint32_t wgs = (p.units + p.units_per_wg - 1u) / p.units_per_wg;
-    if (wgs > 1u && p.units_per_wg % nk != 0u)
-        hipLaunchKernelGGL(gemm_clear_split_tiles_kernel, dim3(wgs - 1u), dim3(256), 0, s, p);
     hipLaunchKernelGGL(kern, dim3(wgs), dim3(512), shmem, s, p);
+    if (wgs > 1u && p.units_per_wg % nk != 0u)
+        hipLaunchKernelGGL(gemm_sum_cut_tiles_kernel, dim3(wgs - 1u, 8), dim3(512), 0, s, p);
     return hipGetLastError();
 }
 
-hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, hipStream_t s)
+hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const SplitScratch& sc, hipStream_t s)
 {
     GemmParams p{};
     p.X = (const uint16_t*)a.X;
@@ -669,29 +704,28 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, hipStream_
     // Q5_K runs on the 128-tile kernel whatever the shape (the persistent kernel's dequantiser is written
     // for the other two types)
     if (a.type == KQ_TYPE_Q5_K) return launch_gemm<KQ_TYPE_Q5_K, 128, 128, 4>(p, s);
-    // Measured on M = 2048: 256-tiles win once they occupy more than half the CUs.  Below that, a long K is
-    // worth cutting (the epilogue of a cut tile costs about 15 k steps), a short one runs on 128-tiles, two
-    // workgroups per CU.  With many tiles per CU, equal shares also remove the ragged last round.
+    // Three ways to run a shape, priced in microseconds with figures measured on the Llama-3-8B matrices at
+    // M = 256 .. 2048: (a) 256-tiles, one workgroup per tile, in rounds over the CUs; (b) the walk over all
+    // (tile, k step) units of the 256-tiles cut into equal shares, one per CU, where every run over part of a
+    // tile costs a workspace slot (256 KB written, read back by the sum kernel); (c) 128-tiles, two workgroups
+    // per CU.  A k step of a 256-tile takes tk, of a 128-tile tk128; a tile's epilogue te.
     const uint32_t cus = device_cu_count(), nk = a.K / GEMM_BK;
     const uint64_t big = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 255u) / 256u);
-    // A cut tile is summed with atomics, which is order-independent for two addends only: the automatic
-    // choices never cut a tile into more than two runs.
+    const uint64_t small = (uint64_t)((a.M + 127u) / 128u) * ((a.N + 127u) / 128u);
+    const float tk = q4 ? 1.7f : 2.7f, tk128 = q4 ? 1.4f : 2.0f, te = 12.0f, t_slot = 0.1f, t_sum = 5.0f;
     const uint32_t one_per_cu = (uint32_t)((big * nk + cus - 1u) / cus);   // equal shares over all CUs
-    bool use_big;
-    uint32_t share = nk;
-    if (big * 2u > cus) {
-        use_big = true;
-        if (big >= 8ull * cus) share = one_per_cu;   // >= 8 tiles each: at most one cut per tile
-    } else {
-        use_big = nk >= 128u && big * nk >= 16ull * cus;
-        share = nk / 2u;                             // every tile in two halves (nk is a multiple of 4)
-    }
+    const uint64_t runs = (big * nk + one_per_cu - 1u) / one_per_cu;
+    const float t_whole = (float)((big + cus - 1u) / cus) * ((float)nk * tk + te);
+    const float t_shares = (float)one_per_cu * tk + te * (1.0f + (float)one_per_cu / (float)nk)
+                           + t_slot * (float)(one_per_cu < nk ? runs : 2u * (runs - 1u)) + t_sum;
+    const float t_small = (float)((small + 2u * cus - 1u) / (2u * cus)) * ((float)nk * tk128 + 0.25f * te);
+    bool use_big = t_small > (t_whole < t_shares ? t_whole : t_shares);
+    uint32_t share = t_shares < t_whole ? one_per_cu : nk;
     if (tile == 256) use_big = true;
     if (tile == 128) use_big = false;
     if (split == 1) share = nk;
     if (split == 2) share = one_per_cu;              // forced: any number of runs per tile
-    (void)cus;
-    if (use_big) return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, share, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, share, s);
+    if (use_big) return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, share, sc, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, share, sc, s);
     return q4 ? launch_gemm<KQ_TYPE_Q4_K, 128, 128, 4>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 128, 128, 4>(p, s);
 }
 

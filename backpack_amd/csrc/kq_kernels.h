@@ -123,7 +123,7 @@ hipError_t launch_moe_combine(const float* down, const float* wt, float* out, ui
 // 128 or 256 (square workgroup tile); split (256-tile only) = 0 (automatic),
 // 1 (one tile per workgroup) or 2 (the walk cut into equal shares per CU).
 bool gemm_bf16_supported(const MatmulArgs& a);
-hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, hipStream_t s);
+hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const SplitScratch& gemm_scratch, hipStream_t s);
 
 // Compute units of the current device (cached per device id).
 inline uint32_t device_cu_count()

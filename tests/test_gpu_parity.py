@@ -412,25 +412,40 @@ def _bf16_bits(x32):
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
-@pytest.mark.parametrize("type_,M,N,K", [(Q6_K, 1024, 2048, 8192),    # 32 big tiles, long K: every tile cut in two halves
-                                          (Q4_K, 2048, 5120, 512)])    # 160 tiles: one tile per workgroup
-def test_gemm_bf16_repeatable(gpu, type_, M, N, K):
-    """The automatic work split never sums more than two partial tiles per element, so a call repeated on the
-    same inputs gives the same bits (fp32 atomics on cleared memory commute for two addends)."""
+@pytest.mark.parametrize("type_,M,N,K,split", [
+    (Q6_K, 1024, 2048, 8192, 0),    # 32 big tiles, long K: the automatic choice cuts every tile
+    (Q4_K, 2048, 5120, 512, 0),     # 160 tiles
+    (Q6_K, 256, 512, 8192, 2),      # 2 tiles x 128 k steps over all CUs: a tile is the sum of up to 128 runs
+    (Q4_K, 512, 1536, 4096, 2),     # 12 tiles x 64 k steps: shares of 3, cut points wander through the tiles
+])
+def test_gemm_bf16_repeatable(gpu, type_, M, N, K, split):
+    """Runs over part of a tile leave their sums in a workspace and a second kernel adds them in the order
+    of the walk, so a call repeated on the same inputs gives the same bits however many runs a tile has."""
     import torch
     from backpack_amd import capi, kquant
     raw, packed, w = gpu.make_weight(type_, N, K, seed=7)
     rng = np.random.default_rng(11)
     bits = _bf16_bits(rng.standard_normal((M, K)).astype(np.float32))
     xd = torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
-    _say("gemm repeat", type_, M, N, K)
+    _say("gemm repeat", type_, M, N, K, split)
+    if split:
+        capi.set_option("gemm_tile", 256)
+        capi.set_option("gemm_split", split)
+    try:
+        _gemm_repeat_body(capi, kquant, xd, w, split)
+    finally:
+        capi.set_option("gemm_tile", 0)
+        capi.set_option("gemm_split", 0)
+
+
+def _gemm_repeat_body(capi, kquant, xd, w, split):
     first = kquant.matmul(xd, w).cpu().numpy()
     assert capi.last_kernel() == "gemm_bf16"
-    capi.set_option("gemm_split", 1)    # the same tiles, each walked by one workgroup: no atomics
+    capi.set_option("gemm_split", 1)    # whole tiles, each walked by one workgroup
     try:
         whole = kquant.matmul(xd, w).cpu().numpy()
     finally:
-        capi.set_option("gemm_split", 0)
+        capi.set_option("gemm_split", split)
     assert np.allclose(first, whole, rtol=0, atol=1e-4 * float(np.abs(whole).max()))
     for _ in range(3):
         again = kquant.matmul(xd, w).cpu().numpy()
