@@ -516,13 +516,14 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
     };
     // piece v of tile t: X copy and 8 dequantised weights into LDS buffer t&1, then the registers of the
     // piece are refilled from tile t+1 (a full step before they are converted)
-    auto convert_piece = [&](uint32_t t, int v) {
+    // refill = false: tile t+1 is made of the same quant bytes as tile t (see the k loop), nothing to fetch
+    auto convert_piece = [&](uint32_t t, int v, bool refill = true) {
         const uint32_t buf = t & 1u;
         *(u32x4*)(As + buf * A_BYTES + x_dst + v * XROWS * GEMM_LD) = xr[v];
         *(u32x4*)(Bs + buf * B_BYTES + w_dst + v * 16) = il_expand(w, tile_at(t), whf, v, s0, s1, nb);
         load_x(t + 1u, v);
-        if (v == 1) il_load_q(wsrc, tile_at(t + 1u), whf, 0, w);
-        if (v == 3) il_load_q(wsrc, tile_at(t + 1u), whf, 1, w);
+        if (v == 1 && refill) il_load_q(wsrc, tile_at(t + 1u), whf, 0, w);
+        if (v == 3 && refill) il_load_q(wsrc, tile_at(t + 1u), whf, 1, w);
     };
     // the matrix instructions of a slice take turns with the conversion arithmetic; LDS reads go first
     auto slice_schedule = [&]() {
@@ -553,14 +554,15 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
 
     bf16x8 af[2][TM], bfr[2][TN];
     read_ops(0, 0, af[0], bfr[0]);
-    for (uint32_t kt = 0; kt < nk; ++kt) {
+    // one k step; refill = whether the quant registers freed by tile kt+1 are loaded with tile kt+2
+    auto k_step = [&](uint32_t kt, bool refill) {
         const uint32_t buf = kt & 1u;
         // slices 0..2 of tile kt; pieces 1..3 of tile kt+1 go to the other buffer
 #pragma unroll
         for (int s = 0; s < 3; ++s) {
             read_ops(buf, s + 1, af[(s + 1) & 1], bfr[(s + 1) & 1]);
             mfma_ops(af[s & 1], bfr[s & 1]);
-            convert_piece(kt + 1u, s + 1);
+            convert_piece(kt + 1u, s + 1, refill);
             slice_schedule();
         }
         // every wave has now read all of tile kt and written its part of tile kt+1
@@ -573,6 +575,18 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
         il_load_head(wsrc, tile_at(kt + 3u), whf, w);
         convert_piece(kt + 2u, 0);
         slice_schedule();
+    };
+    if constexpr (TYPE == KQ_TYPE_Q6_K) {
+        // Q6_K: k steps 2j and 2j+1 of a row take the low and the high nibbles of the same 32 bytes of ql and
+        // different bit pairs of the same 32 bytes of qh, so the registers loaded for an even tile serve the
+        // odd tile after it.  Runs start on even k steps and have even lengths (the launcher sees to it):
+        // tile kt+2 is odd exactly when kt is.
+        for (uint32_t kt = 0; kt < nk; kt += 2u) {
+            k_step(kt, true);
+            k_step(kt + 1u, false);
+        }
+    } else {
+        for (uint32_t kt = 0; kt < nk; ++kt) k_step(kt, true);
     }
 
     // A tile walked in one piece is stored.  A run over part of a tile leaves its sums in the workspace, in
@@ -680,6 +694,7 @@ static hipError_t launch_gemm_persistent(GemmParams p, uint32_t share, const Spl
     p.units = tiles * nk;
     // cut tiles need two workspace slots per workgroup: without them, whole tiles
     if ((size_t)2u * ((p.units + share - 1u) / share) * 65536u > sc.capacity_floats) share = nk;
+    if (TYPE == KQ_TYPE_Q6_K) share += share & 1u;   // the Q6_K k loop takes its steps in pairs (nk is a multiple of 4)
     p.units_per_wg = share;
     p.partial = sc.partial;
     const uint32_t wgs = (p.units + p.units_per_wg - 1u) / p.units_per_wg;
