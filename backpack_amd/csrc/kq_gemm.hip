@@ -354,9 +354,9 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm_bf16_kernel(GemmParams p)
 struct RawQ4 { u32x4 h, q0, q1; };
 struct RawQ6 { u32x4 a0, a1, b0, b1; uint32_t sc2, d16; };
 
-__device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, uint32_t, RawQ4& r)
+__device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, uint32_t, RawQ4& r, bool new_block = true)
 {
-    r.h = *(const u32x4*)(row + (size_t)(kc >> 2) * KQ_Q4K_BYTES);
+    if (new_block) r.h = *(const u32x4*)(row + (size_t)(kc >> 2) * KQ_Q4K_BYTES);
 }
 __device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint32_t, int half, RawQ4& r)
 {
@@ -393,15 +393,18 @@ __device__ __forceinline__ u32x4 il_expand(const RawQ4& r, uint32_t, uint32_t hf
     return out;
 }
 
-__device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, uint32_t hf, RawQ6& r)
+// new_block = false: the step lies in the same superblock as the one before it (d is already there)
+__device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, uint32_t hf, RawQ6& r, bool new_block = true)
 {
     const uint32_t c = kc & 3u, h = c >> 1, t = (c & 1u) * 2u + hf;
     const uint8_t* blk = row + (size_t)(kc >> 2) * KQ_Q6K_BYTES;
     uint16_t s2, d2;
     __builtin_memcpy(&s2, blk + 192u + 8u * h + 2u * t, 2);
-    __builtin_memcpy(&d2, blk + 208u, 2);
     r.sc2 = s2;
-    r.d16 = d2;
+    if (new_block) {
+        __builtin_memcpy(&d2, blk + 208u, 2);
+        r.d16 = d2;
+    }
 }
 __device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint32_t hf, int half, RawQ6& r)
 {
@@ -554,8 +557,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
 
     bf16x8 af[2][TM], bfr[2][TN];
     read_ops(0, 0, af[0], bfr[0]);
-    // one k step; refill = whether the quant registers freed by tile kt+1 are loaded with tile kt+2
-    auto k_step = [&](uint32_t kt, bool refill) {
+    // one k step; refill = whether the quant registers freed by tile kt+1 are loaded with tile kt+2,
+    // new_block = whether tile kt+3 opens a superblock (else its header is the one already in registers)
+    auto k_step = [&](uint32_t kt, bool refill, bool new_block) {
         const uint32_t buf = kt & 1u;
         // slices 0..2 of tile kt; pieces 1..3 of tile kt+1 go to the other buffer
 #pragma unroll
@@ -572,21 +576,22 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
         read_ops(buf ^ 1u, 0, af[0], bfr[0]);
         mfma_ops(af[1], bfr[1]);
         il_scales(w, tile_at(kt + 2u), whf, s0, s1, nb);
-        il_load_head(wsrc, tile_at(kt + 3u), whf, w);
+        il_load_head(wsrc, tile_at(kt + 3u), whf, w, new_block);
         convert_piece(kt + 2u, 0);
         slice_schedule();
     };
-    if constexpr (TYPE == KQ_TYPE_Q6_K) {
-        // Q6_K: k steps 2j and 2j+1 of a row take the low and the high nibbles of the same 32 bytes of ql and
-        // different bit pairs of the same 32 bytes of qh, so the registers loaded for an even tile serve the
-        // odd tile after it.  Runs start on even k steps and have even lengths (the launcher sees to it):
-        // tile kt+2 is odd exactly when kt is.
-        for (uint32_t kt = 0; kt < nk; kt += 2u) {
-            k_step(kt, true);
-            k_step(kt + 1u, false);
-        }
-    } else {
-        for (uint32_t kt = 0; kt < nk; ++kt) k_step(kt, true);
+    // Runs start on a superblock (k step 4j) and cover whole superblocks (the launcher sees to it), so the four
+    // steps of a superblock are told apart at compile time.  The header of tile kt+3 has to be fetched when
+    // kt+3 is a multiple of 4 (the tile beyond the run is the clamped last one: same superblock, no fetch is
+    // lost).  Q6_K: k steps 2j and 2j+1 of a row take the low and the high nibbles of the same 32 bytes of ql
+    // and different bit pairs of the same 32 bytes of qh, so the registers loaded for an even tile serve the
+    // odd tile after it.
+    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
+    for (uint32_t kt = 0; kt < nk; kt += 4u) {
+        k_step(kt, true, false);
+        k_step(kt + 1u, !Q6, true);
+        k_step(kt + 2u, true, false);
+        k_step(kt + 3u, !Q6, false);
     }
 
     // A tile walked in one piece is stored.  A run over part of a tile leaves its sums in the workspace, in
@@ -694,7 +699,7 @@ static hipError_t launch_gemm_persistent(GemmParams p, uint32_t share, const Spl
     p.units = tiles * nk;
     // cut tiles need two workspace slots per workgroup: without them, whole tiles
     if ((size_t)2u * ((p.units + share - 1u) / share) * 65536u > sc.capacity_floats) share = nk;
-    if (TYPE == KQ_TYPE_Q6_K) share += share & 1u;   // the Q6_K k loop takes its steps in pairs (nk is a multiple of 4)
+    share = (share + 3u) & ~3u;   // the k loop takes whole superblocks (nk is a multiple of 4)
     p.units_per_wg = share;
     p.partial = sc.partial;
     const uint32_t wgs = (p.units + p.units_per_wg - 1u) / p.units_per_wg;
@@ -727,7 +732,7 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const Spli
     const uint32_t cus = device_cu_count(), nk = a.K / GEMM_BK;
     const uint64_t big = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 255u) / 256u);
     const uint64_t small = (uint64_t)((a.M + 127u) / 128u) * ((a.N + 127u) / 128u);
-    const float tk = q4 ? 1.7f : 2.7f, tk128 = q4 ? 1.4f : 2.0f, te = 12.0f, t_slot = 0.1f, t_sum = 5.0f;
+    const float tk = q4 ? 1.7f : 2.2f, tk128 = q4 ? 1.4f : 2.0f, te = 12.0f, t_slot = 0.1f, t_sum = 5.0f;
     const uint32_t one_per_cu = (uint32_t)((big * nk + cus - 1u) / cus);   // equal shares over all CUs
     const uint64_t runs = (big * nk + one_per_cu - 1u) / one_per_cu;
     const float t_whole = (float)((big + cus - 1u) / cus) * ((float)nk * tk + te);
