@@ -100,8 +100,6 @@ int ensure_device(int device, DeviceState** out)
         if (e == hipSuccess) e = hipMalloc((void**)&st.split.counters, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMemset(st.split.counters, 0, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMalloc((void**)&st.gemm_split.partial, kGemmPartialFloats * sizeof(float));
-        if (e == hipSuccess) e = hipMalloc((void**)&st.gemm_split.counters, kCounters * sizeof(uint32_t));
-        if (e == hipSuccess) e = hipMemset(st.gemm_split.counters, 0, kCounters * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMalloc((void**)&st.moe_tiles, kMoeWords * sizeof(uint32_t));
         constexpr size_t kArgmaxWords = (size_t)kq::ARGMAX_MAX_ROWS * (2u * kq::ARGMAX_PARTS + 1u);
         if (e == hipSuccess) e = hipMalloc((void**)&st.argmax_scratch, kArgmaxWords * sizeof(uint32_t));
@@ -112,7 +110,7 @@ int ensure_device(int device, DeviceState** out)
         st.split.capacity_floats = kPartialFloats;
         st.split.n_counters = kCounters;
         st.gemm_split.capacity_floats = kGemmPartialFloats;
-        st.gemm_split.n_counters = kCounters;
+        st.gemm_split.n_counters = 0;   // the sum kernel needs no arrival counters
         st.ready = true;
     }
     if (out) *out = &st;

@@ -372,8 +372,9 @@ BPK_API int bpk_force_kernel(int family);
  * keeps in flight (1, 2 or 4); "gemm_tile": square workgroup tile of the bf16
  * GEMM (128 or 256); "gemm_split": how the 256-tile GEMM hands out work
  * (1 = one tile per workgroup, 2 = the walk over tiles and k steps cut into
- * equal shares per compute unit, tiles cut between workgroups are summed with
- * fp32 atomics); "fused_separate": 1 makes bpk_kq_matmul_fused run its prologue,
+ * equal shares per compute unit; the runs of a tile cut between workgroups go
+ * through a per-device workspace and are added in the order of the walk, so
+ * results repeat bit for bit); "fused_separate": 1 makes bpk_kq_matmul_fused run its prologue,
  * matmul and add as separate launches for every shape (needs the workspace).
  * 0 = automatic. */
 BPK_API int bpk_set_option(const char *name, int value);
