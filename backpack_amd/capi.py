@@ -84,6 +84,8 @@ _SIGS = {
                                       C.POINTER(Fusion), C.c_void_p, C.c_size_t, C.c_void_p]),
     "bpk_kq_matmul_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
                                      C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p]),
+    "bpk_prefill_rows_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_uint32, C.c_uint32,
+                                        C.c_void_p, C.c_void_p]),
     "bpk_kq_dequant_rows": (C.c_int, [C.c_int, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_uint32,
                                       C.c_void_p, C.c_void_p]),
     "bpk_kq_moe_matmul": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,

@@ -533,6 +533,21 @@ int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bi
     return BPK_OK;
 }
 
+int bpk_prefill_rows_bf16(int prologue, const float* X, const float* norm_w, float eps, uint32_t M, uint32_t K,
+                          uint16_t* out, void* stream)
+{
+    if (prologue < BPK_PRO_NONE || prologue > BPK_PRO_GELU_MUL) return fail(BPK_ERR_SHAPE, "unknown prologue");
+    if (!X || !out) return fail(BPK_ERR_NULL, "X and out are required");
+    if (prologue == BPK_PRO_RMS_NORM && !norm_w) return fail(BPK_ERR_NULL, "BPK_PRO_RMS_NORM needs norm_w");
+    if (K == 0) return fail(BPK_ERR_SHAPE, "K must be positive");
+    if (M > 65535u && prologue != BPK_PRO_RMS_NORM) return fail(BPK_ERR_SHAPE, "at most 65535 rows per call");
+    if (M == 0) return BPK_OK;
+    if (int rc = current_state(nullptr)) return rc;
+    t_kernel = "prefill_rows_bf16";
+    const hipError_t e = kq::launch_prologue_rows_bf16(prologue, X, norm_w, eps, M, K, out, (hipStream_t)stream);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
 int bpk_kq_matmul_bf16(int type, const uint16_t* X, const void* W, const float* bias, float* Y, uint32_t M,
                        uint32_t N, uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, void* stream)
 {

@@ -12,9 +12,17 @@
 
 namespace kq {
 
+// An output element as fp32, or as bf16 (round to nearest even: the activation rows of the prefill GEMM).
+__device__ __forceinline__ void put_out(float* out, size_t at, float v) { out[at] = v; }
+__device__ __forceinline__ void put_out(uint16_t* out, size_t at, float v)
+{
+    out[at] = __builtin_bit_cast(uint16_t, (__bf16)v);
+}
+
 // One workgroup of 256 lanes per row.
+template <typename OUT>
 __global__ __launch_bounds__(256) void rms_norm_rows_kernel(const float* X, const float* w, float eps, uint32_t K,
-                                                            float* out)
+                                                            OUT* out)
 {
     __shared__ float part[4];
     const float* x = X + (size_t)blockIdx.x * K;
@@ -25,13 +33,22 @@ __global__ __launch_bounds__(256) void rms_norm_rows_kernel(const float* X, cons
     if ((threadIdx.x & 63u) == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
     const float rstd = 1.0f / sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)K + eps);
-    float* o = out + (size_t)blockIdx.x * K;
-    for (uint32_t k = threadIdx.x; k < K; k += 256u) o[k] = x[k] * rstd * w[k];
+    const size_t o = (size_t)blockIdx.x * K;
+    for (uint32_t k = threadIdx.x; k < K; k += 256u) put_out(out, o + k, x[k] * rstd * w[k]);
+}
+
+// out[m, k] = X[m, k] converted (blockIdx.y = row)
+__global__ __launch_bounds__(256) void cast_rows_bf16_kernel(const float* X, uint32_t K, uint16_t* out)
+{
+    const uint32_t k = blockIdx.x * 256u + threadIdx.x;
+    if (k >= K) return;
+    const size_t at = (size_t)blockIdx.y * K + k;
+    put_out(out, at, X[at]);
 }
 
 // GU rows are gate | up (2K floats); out rows are K floats.
-template <bool GELU>
-__global__ __launch_bounds__(256) void act_mul_rows_kernel(const float* GU, uint32_t K, float* out)
+template <bool GELU, typename OUT>
+__global__ __launch_bounds__(256) void act_mul_rows_kernel(const float* GU, uint32_t K, OUT* out)
 {
     const float* g = GU + (size_t)blockIdx.y * 2u * K;
     const uint32_t k = blockIdx.x * 256u + threadIdx.x;
@@ -44,7 +61,7 @@ __global__ __launch_bounds__(256) void act_mul_rows_kernel(const float* GU, uint
     } else {
         a = gv / (expf(-gv) + 1.0f);
     }
-    out[(size_t)blockIdx.y * K + k] = a * uv;
+    put_out(out, (size_t)blockIdx.y * K + k, a * uv);
 }
 
 // Y[m, y_offset + n] = T[m, n] + R[m, y_offset + n]   (R may be Y)
@@ -57,12 +74,28 @@ __global__ __launch_bounds__(256) void add_residual_kernel(const float* T, const
     Y[at] = T[(size_t)blockIdx.y * N + n] + R[at];
 }
 
+template <typename OUT>
+static hipError_t launch_prologue_rows_as(int pro, const float* X, const float* norm_w, float eps, uint32_t M, uint32_t K,
+                                          OUT* out, hipStream_t s)
+{
+    if (pro == 1) hipLaunchKernelGGL(rms_norm_rows_kernel<OUT>, dim3(M), dim3(256), 0, s, X, norm_w, eps, K, out);
+    else if (pro == 2) hipLaunchKernelGGL((act_mul_rows_kernel<false, OUT>), dim3((K + 255u) / 256u, M), dim3(256), 0, s, X, K, out);
+    else hipLaunchKernelGGL((act_mul_rows_kernel<true, OUT>), dim3((K + 255u) / 256u, M), dim3(256), 0, s, X, K, out);
+    return hipGetLastError();
+}
+
 hipError_t launch_prologue_rows(int pro, const float* X, const float* norm_w, float eps, uint32_t M, uint32_t K,
                                 float* out, hipStream_t s)
 {
-    if (pro == 1) hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(M), dim3(256), 0, s, X, norm_w, eps, K, out);
-    else if (pro == 2) hipLaunchKernelGGL(act_mul_rows_kernel<false>, dim3((K + 255u) / 256u, M), dim3(256), 0, s, X, K, out);
-    else hipLaunchKernelGGL(act_mul_rows_kernel<true>, dim3((K + 255u) / 256u, M), dim3(256), 0, s, X, K, out);
+    return launch_prologue_rows_as(pro, X, norm_w, eps, M, K, out, s);
+}
+
+// pro 0: the rows as they are
+hipError_t launch_prologue_rows_bf16(int pro, const float* X, const float* norm_w, float eps, uint32_t M, uint32_t K,
+                                     uint16_t* out, hipStream_t s)
+{
+    if (pro != 0) return launch_prologue_rows_as(pro, X, norm_w, eps, M, K, out, s);
+    hipLaunchKernelGGL(cast_rows_bf16_kernel, dim3((K + 255u) / 256u, M), dim3(256), 0, s, X, K, out);
     return hipGetLastError();
 }
 

@@ -55,6 +55,9 @@ hipError_t launch_dequant_rows(int type, const uint8_t* W, uint32_t row_stride_b
 // Y[m, y_offset + n] = T[m, n] + R[m, y_offset + n].
 hipError_t launch_prologue_rows(int pro, const float* X, const float* norm_w, float eps, uint32_t M, uint32_t K,
                                 float* out, hipStream_t s);
+// The same prologues with bf16 rows as their output (pro 0: plain conversion): X of the prefill GEMM.
+hipError_t launch_prologue_rows_bf16(int pro, const float* X, const float* norm_w, float eps, uint32_t M, uint32_t K,
+                                     uint16_t* out, hipStream_t s);
 hipError_t launch_add_residual(const float* T, const float* R, float* Y, uint32_t M, uint32_t N, uint32_t ldy,
                                uint32_t y_offset, hipStream_t s);
 

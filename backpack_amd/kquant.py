@@ -128,6 +128,19 @@ def matmul(x: torch.Tensor, w: KQuantPacked, bias: torch.Tensor | None = None,
     return out
 
 
+def prefill_rows_bf16(x: torch.Tensor, K: int, prologue: int = capi.PRO_NONE, norm_w: torch.Tensor | None = None,
+                      eps: float = 0.0) -> torch.Tensor:
+    """fp32 rows -> the bf16 activation rows of the prefill GEMM, [M, K]: x as it is, its RMSNorm, or
+    act(gate) * up of gate|up rows of 2K floats, evaluated in fp32 and rounded to nearest even."""
+    assert x.is_cuda and x.is_contiguous() and x.dtype == torch.float32
+    row = 2 * K if prologue in (capi.PRO_SILU_MUL, capi.PRO_GELU_MUL) else K
+    assert x.shape[-1] == row
+    M = x.numel() // row
+    out = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
+    capi.check(capi.lib().bpk_prefill_rows_bf16(prologue, _ptr(x), _ptr(norm_w), eps, M, K, _ptr(out), _stream()))
+    return out
+
+
 def matmul_fused(x: torch.Tensor, w: KQuantPacked, prologue: int = capi.PRO_NONE, norm_w: torch.Tensor | None = None,
                  eps: float = 0.0, residual: torch.Tensor | None = None, bias: torch.Tensor | None = None,
                  out: torch.Tensor | None = None, workspace: torch.Tensor | None = None,

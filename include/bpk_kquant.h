@@ -284,6 +284,19 @@ BPK_API int bpk_kq_matmul_bf16(int type, const uint16_t *X, const void *W,
                                uint32_t N, uint32_t K, uint32_t n_blocks,
                                uint32_t row_stride_words, void *stream);
 
+/* Activation rows for bpk_kq_matmul_bf16 from the engine's fp32 buffers:
+ *   out[m*K + k] = bf16(x[m,k]), round to nearest even, with x the prologue
+ * forms of bpk_kq_matmul_fused (BPK_PRO_NONE: X as it is; BPK_PRO_RMS_NORM:
+ * norm/rms_norm.wgsl:15-20; BPK_PRO_SILU_MUL / BPK_PRO_GELU_MUL: X rows are
+ * gate | up, 2K floats, fused/silu_mul_fused.wgsl:39-49 and
+ * fused/gelu_mul_fused.wgsl:22-32), evaluated in fp32.  The reference keeps
+ * activations in fp32 and has no bf16 path; this is the one pass its norm and
+ * act*mul dispatches become in front of a prefill GEMM.  X f32 (device),
+ * out bf16 [M,K] (device, 2-byte aligned); K any positive size. */
+BPK_API int bpk_prefill_rows_bf16(int prologue, const float *X,
+                                  const float *norm_w, float eps, uint32_t M,
+                                  uint32_t K, uint16_t *out, void *stream);
+
 /* ---- dequantised rows: replaces q6k_gather / q6k_gather_batched -------------
  * runtime/kernels/quant_kq/q6k_gather.wgsl:15-44, q6k_gather_batched.wgsl:9-21.
  * out[m*K + k] = dequant(W)[max(rows[m],0), k], bit-identical to

@@ -199,3 +199,60 @@ def test_fused_epilogue_argument_checks(gpu):
     assert call(capi.Fusion(capi.PRO_NONE, None, 0.0, None, 1)) == -2                  # unknown epilogue
     assert call(capi.Fusion(capi.PRO_NONE, None, 0.0, y.data_ptr(), capi.EPI_SILU_MUL)) == -2   # residual with epilogue
     assert call(capi.Fusion(capi.PRO_NONE, None, 0.0, None, capi.EPI_SILU_MUL)) == 0
+
+
+def _bf16_rne(x32):
+    u = np.ascontiguousarray(x32, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+@pytest.mark.parametrize("M,K,pro", [(1, 256, NONE), (37, 4096, NONE), (300, 1000, NONE),
+                                      (5, 4096, NORM), (257, 768, NORM), (3, 300, NORM),
+                                      (4, 14336, SILU), (130, 768, SILU), (2, 1000, SILU),
+                                      (6, 2048, GELU), (129, 512, GELU)])
+def test_prefill_rows_bf16(gpu, kqo, M, K, pro):
+    """Activation rows of the prefill GEMM: plain conversion is the round-to-nearest-even bit pattern;
+    the prologue forms are the oracle's fp32 prologue rounded the same way, to within one bf16 step where
+    the device's exp / tanh / rsqrt differ from the oracle's libm in the last place."""
+    from backpack_amd import kquant
+    rng = np.random.default_rng(M * 7 + K + pro)
+    X = (rng.standard_normal((M, K if pro in (NONE, NORM) else 2 * K)) * 1.5).astype(np.float32)
+    if pro == NONE:   # ties, subnormals, signed zero, the largest finite value
+        X.flat[:6] = np.array([1.00390625, 1.01171875, 1e-40, -0.0, 3.3895313e38, -1.00390625], dtype=np.float32)[:min(6, X.size)]
+    norm_w = (1 + 0.1 * rng.standard_normal(K)).astype(np.float32) if pro == NORM else None
+    got = kquant.prefill_rows_bf16(gpu.dev(X), K, prologue=pro, norm_w=gpu.dev(norm_w) if norm_w is not None else None,
+                                   eps=1e-5)
+    assert tuple(got.shape) == (M, K)
+    got = got.view(__import__("torch").int16).cpu().numpy().view(np.uint16)
+    ref32 = X if pro == NONE else kqo.prologue(pro, X, K, norm_w=norm_w, eps=1e-5)
+    want = _bf16_rne(ref32).reshape(M, K)
+    if pro == NONE:
+        assert np.array_equal(got, want)
+        return
+    step = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    assert step.max() <= 1, f"{int((step > 1).sum())} elements more than one bf16 step away"
+    assert (step > 0).mean() < 0.02, f"{(step > 0).mean():.3%} of the elements differ"
+
+
+def test_prefill_rows_bf16_feeds_the_gemm_and_checks_arguments(gpu, kqo):
+    """norm -> bf16 rows -> dequant-GEMM equals the oracle matmul of the rounded rows; argument errors."""
+    from backpack_amd import capi, kquant
+    M, N, K = 300, 520, 1024
+    rng = np.random.default_rng(5)
+    raw, packed, w = gpu.make_weight(Q4_K, N, K, seed=9)
+    X = rng.standard_normal((M, K)).astype(np.float32)
+    norm_w = (1 + 0.1 * rng.standard_normal(K)).astype(np.float32)
+    xb = kquant.prefill_rows_bf16(gpu.dev(X), K, prologue=NORM, norm_w=gpu.dev(norm_w), eps=1e-5)
+    got = kquant.matmul(xb, w).cpu().numpy()
+    assert capi.last_kernel() == "gemm_bf16"
+    bits = xb.view(__import__("torch").int16).cpu().numpy().view(np.uint16)
+    Xw = (bits.astype(np.uint32) << 16).view(np.float32)
+    cpu = kqo.matmul(Q4_K, Xw, packed, N, K)
+    assert np.abs(got - cpu).max() <= 1e-2 * float(np.abs(cpu).max())
+    L = capi.lib()
+    x = gpu.dev(X)
+    assert L.bpk_prefill_rows_bf16(7, x.data_ptr(), None, 0.0, M, K, xb.data_ptr(), None) == -2
+    assert L.bpk_prefill_rows_bf16(NORM, x.data_ptr(), None, 1e-5, M, K, xb.data_ptr(), None) == -3
+    assert L.bpk_prefill_rows_bf16(NONE, None, None, 0.0, M, K, xb.data_ptr(), None) == -3
+    assert L.bpk_prefill_rows_bf16(NONE, x.data_ptr(), None, 0.0, M, 0, xb.data_ptr(), None) == -2
+    assert L.bpk_prefill_rows_bf16(NONE, x.data_ptr(), None, 0.0, 0, K, xb.data_ptr(), None) == 0
