@@ -353,12 +353,13 @@ __global__ __launch_bounds__(64 * NWAVES) void gemm_bf16_kernel(GemmParams p)
 // 16-byte pieces of the X tile per step; their raw bytes live in registers one step ahead of their use.
 struct RawQ4 { u32x4 h, q0, q1; };
 struct RawQ6 { u32x4 a0, a1, b0, b1; uint32_t sc2, d16; };
+struct RawQ5 { u32x4 h, q0, q1, b0, b1; };   // header, the run's 32 quant bytes, the block's 32 bytes of fifth bits
 
 __device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, uint32_t, RawQ4& r, bool new_block = true)
 {
     if (new_block) r.h = *(const u32x4*)(row + (size_t)(kc >> 2) * KQ_Q4K_BYTES);
 }
-__device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint32_t, int half, RawQ4& r)
+__device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint32_t, int half, RawQ4& r, bool = true)
 {
     const u32x4* q = (const u32x4*)(row + (size_t)(kc >> 2) * KQ_Q4K_BYTES + 16 + (kc & 3u) * 32u);
     if (half == 0) r.q0 = q[0]; else r.q1 = q[1];
@@ -394,6 +395,49 @@ __device__ __forceinline__ u32x4 il_expand(const RawQ4& r, uint32_t, uint32_t hf
 }
 
 // new_block = false: the step lies in the same superblock as the one before it (d is already there)
+// Q5_K: the Q4_K walk with the quants 32 bytes further on; the fifth bits of a run's 32 elements are bit
+// 2c + hf of the block's 32 bytes of qh (the same bytes for the four k steps c of a superblock: extra = false
+// leaves them in their registers).  Both nibbles come down to bits 0..3 so that the fifth bit joins at bit 4.
+__device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, uint32_t, RawQ5& r, bool new_block = true)
+{
+    if (new_block) r.h = *(const u32x4*)(row + (size_t)(kc >> 2) * KQ_Q5K_BYTES);
+}
+__device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint32_t, int half, RawQ5& r, bool extra = true)
+{
+    const uint8_t* blk = row + (size_t)(kc >> 2) * KQ_Q5K_BYTES;
+    const u32x4* q = (const u32x4*)(blk + 48 + (kc & 3u) * 32u);
+    const u32x4* b = (const u32x4*)(blk + 16);
+    if (half == 0) { r.q0 = q[0]; if (extra) r.b0 = b[0]; }
+    else { r.q1 = q[1]; if (extra) r.b1 = b[1]; }
+}
+__device__ __forceinline__ void il_scales(const RawQ5& r, uint32_t kc, uint32_t hf, float& s0, float& s1, float& nb)
+{
+    const float d = half_bits_to_float(r.h.x & 0xFFFFu);
+    const float dmin = half_bits_to_float(r.h.x >> 16);
+    uint32_t sc, mn;
+    q4k_scale_min(r.h.y, r.h.z, r.h.w, (int)((kc & 3u) * 2u + hf), sc, mn);
+    s0 = d * (float)sc;
+    s1 = s0;
+    nb = -(dmin * (float)mn);
+}
+__device__ __forceinline__ u32x4 il_expand(const RawQ5& r, uint32_t kc, uint32_t hf, int v, float s0, float, float nb)
+{
+    const u32x4 src = v < 2 ? r.q0 : r.q1, bits = v < 2 ? r.b0 : r.b1;
+    const uint32_t sh = hf * 4u, sb = (kc & 3u) * 2u + hf;
+    u32x4 out;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t w = ((src[(v & 1) * 2 + j] >> sh) & 0x0F0F0F0Fu) | (((bits[(v & 1) * 2 + j] >> sb) & 0x01010101u) << 4);
+        const float f0 = fmaf(s0, (float)(w & 255u), nb);
+        const float f1 = fmaf(s0, (float)((w >> 8) & 255u), nb);
+        const float f2 = fmaf(s0, (float)((w >> 16) & 255u), nb);
+        const float f3 = fmaf(s0, (float)(w >> 24), nb);
+        out[j * 2] = pack_bf16(f0, f1);
+        out[j * 2 + 1] = pack_bf16(f2, f3);
+    }
+    return out;
+}
+
 __device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, uint32_t hf, RawQ6& r, bool new_block = true)
 {
     const uint32_t c = kc & 3u, h = c >> 1, t = (c & 1u) * 2u + hf;
@@ -406,7 +450,7 @@ __device__ __forceinline__ void il_load_head(const uint8_t* row, uint32_t kc, ui
         r.d16 = d2;
     }
 }
-__device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint32_t hf, int half, RawQ6& r)
+__device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint32_t hf, int half, RawQ6& r, bool = true)
 {
     const uint32_t c = kc & 3u, h = c >> 1, t = (c & 1u) * 2u + hf;
     const uint8_t* blk = row + (size_t)(kc >> 2) * KQ_Q6K_BYTES;
@@ -456,7 +500,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
     constexpr int BM = 256, BN = 256, WAVES_N = 4, WM = 128, WN = 64, TM = 4, TN = 2;
     constexpr int A_BYTES = BM * GEMM_LD, B_BYTES = BN * GEMM_LD;
     constexpr int XROWS = 64;   // X rows per piece: 8 threads x 16 bytes per row, 4 pieces
-    using Raw = typename std::conditional<TYPE == KQ_TYPE_Q4_K, RawQ4, RawQ6>::type;
+    using Raw = typename std::conditional<TYPE == KQ_TYPE_Q4_K, RawQ4,
+                                          typename std::conditional<TYPE == KQ_TYPE_Q5_K, RawQ5, RawQ6>::type>::type;
     uint8_t* As = smem;
     uint8_t* Bs = smem + 2 * A_BYTES;
 
@@ -519,14 +564,15 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
     };
     // piece v of tile t: X copy and 8 dequantised weights into LDS buffer t&1, then the registers of the
     // piece are refilled from tile t+1 (a full step before they are converted)
-    // refill = false: tile t+1 is made of the same quant bytes as tile t (see the k loop), nothing to fetch
-    auto convert_piece = [&](uint32_t t, int v, bool refill = true) {
+    // refill = false: tile t+1 is made of the same quant bytes as tile t (see the k loop), nothing to fetch;
+    // extra = false: tile t+1 lies in the superblock of tile t (Q5_K keeps its fifth bits)
+    auto convert_piece = [&](uint32_t t, int v, bool refill = true, bool extra = true) {
         const uint32_t buf = t & 1u;
         *(u32x4*)(As + buf * A_BYTES + x_dst + v * XROWS * GEMM_LD) = xr[v];
         *(u32x4*)(Bs + buf * B_BYTES + w_dst + v * 16) = il_expand(w, tile_at(t), whf, v, s0, s1, nb);
         load_x(t + 1u, v);
-        if (v == 1 && refill) il_load_q(wsrc, tile_at(t + 1u), whf, 0, w);
-        if (v == 3 && refill) il_load_q(wsrc, tile_at(t + 1u), whf, 1, w);
+        if (v == 1 && refill) il_load_q(wsrc, tile_at(t + 1u), whf, 0, w, extra);
+        if (v == 3 && refill) il_load_q(wsrc, tile_at(t + 1u), whf, 1, w, extra);
     };
     // the matrix instructions of a slice take turns with the conversion arithmetic; LDS reads go first
     auto slice_schedule = [&]() {
@@ -559,14 +605,15 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
     read_ops(0, 0, af[0], bfr[0]);
     // one k step; refill = whether the quant registers freed by tile kt+1 are loaded with tile kt+2,
     // new_block = whether tile kt+3 opens a superblock (else its header is the one already in registers)
-    auto k_step = [&](uint32_t kt, bool refill, bool new_block) {
+    // (opens = whether tile kt+2 opens a superblock)
+    auto k_step = [&](uint32_t kt, bool refill, bool new_block, bool opens) {
         const uint32_t buf = kt & 1u;
         // slices 0..2 of tile kt; pieces 1..3 of tile kt+1 go to the other buffer
 #pragma unroll
         for (int s = 0; s < 3; ++s) {
             read_ops(buf, s + 1, af[(s + 1) & 1], bfr[(s + 1) & 1]);
             mfma_ops(af[s & 1], bfr[s & 1]);
-            convert_piece(kt + 1u, s + 1, refill);
+            convert_piece(kt + 1u, s + 1, refill, opens);
             slice_schedule();
         }
         // every wave has now read all of tile kt and written its part of tile kt+1
@@ -588,10 +635,10 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
     // odd tile after it.
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
     for (uint32_t kt = 0; kt < nk; kt += 4u) {
-        k_step(kt, true, false);
-        k_step(kt + 1u, !Q6, true);
-        k_step(kt + 2u, true, false);
-        k_step(kt + 3u, !Q6, false);
+        k_step(kt, true, false, false);
+        k_step(kt + 1u, !Q6, true, false);
+        k_step(kt + 2u, true, false, true);
+        k_step(kt + 3u, !Q6, false, false);
     }
 
     // A tile walked in one piece is stored.  A run over part of a tile leaves its sums in the workspace, in
@@ -720,10 +767,7 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const Spli
     p.n_blocks = a.n_blocks;
     p.row_stride_bytes = a.row_stride_bytes;
     p.ldy = a.ldy;
-    const bool q4 = a.type == KQ_TYPE_Q4_K;
-    // Q5_K runs on the 128-tile kernel whatever the shape (the persistent kernel's dequantiser is written
-    // for the other two types)
-    if (a.type == KQ_TYPE_Q5_K) return launch_gemm<KQ_TYPE_Q5_K, 128, 128, 4>(p, s);
+    const bool q4 = a.type == KQ_TYPE_Q4_K, q5 = a.type == KQ_TYPE_Q5_K;
     // Three ways to run a shape, priced in microseconds with figures measured on the Llama-3-8B matrices at
     // M = 256 .. 2048: (a) 256-tiles, one workgroup per tile, in rounds over the CUs; (b) the walk over all
     // (tile, k step) units of the 256-tiles cut into equal shares, one per CU, where every run over part of a
@@ -732,7 +776,7 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const Spli
     const uint32_t cus = device_cu_count(), nk = a.K / GEMM_BK;
     const uint64_t big = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 255u) / 256u);
     const uint64_t small = (uint64_t)((a.M + 127u) / 128u) * ((a.N + 127u) / 128u);
-    const float tk = q4 ? 1.7f : 2.2f, tk128 = q4 ? 1.4f : 2.0f, te = 12.0f, t_slot = 0.1f, t_sum = 5.0f;
+    const float tk = q4 ? 1.7f : q5 ? 1.9f : 2.2f, tk128 = q4 ? 1.4f : q5 ? 1.6f : 2.0f, te = 12.0f, t_slot = 0.1f, t_sum = 5.0f;
     const uint32_t one_per_cu = (uint32_t)((big * nk + cus - 1u) / cus);   // equal shares over all CUs
     const uint64_t runs = (big * nk + one_per_cu - 1u) / one_per_cu;
     const float t_whole = (float)((big + cus - 1u) / cus) * ((float)nk * tk + te);
@@ -745,8 +789,11 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const Spli
     if (tile == 128) use_big = false;
     if (split == 1) share = nk;
     if (split == 2) share = one_per_cu;              // forced: any number of runs per tile
-    if (use_big) return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, share, sc, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, share, sc, s);
-    return q4 ? launch_gemm<KQ_TYPE_Q4_K, 128, 128, 4>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 128, 128, 4>(p, s);
+    if (use_big)
+        return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, share, sc, s)
+                  : q5 ? launch_gemm_persistent<KQ_TYPE_Q5_K>(p, share, sc, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, share, sc, s);
+    return q4 ? launch_gemm<KQ_TYPE_Q4_K, 128, 128, 4>(p, s)
+              : q5 ? launch_gemm<KQ_TYPE_Q5_K, 128, 128, 4>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 128, 128, 4>(p, s);
 }
 
 }  // namespace kq

@@ -387,11 +387,15 @@ GEMM_SHAPES = [
     (Q6_K, 256, 256, 768, 256),      # odd block count: rows only 8-byte aligned
     (Q6_K, 190, 260, 1024, 128),
     (Q6_K, 512, 512, 4096, 0),
-    # Q5_K: the 128-tile kernel whatever is asked for
-    (Q5_K, 128, 128, 256, 0),
+    # Q5_K: both tiles, the automatic choice, whole tiles and equal shares
+    (Q5_K, 128, 128, 256, 128),
     (Q5_K, 200, 300, 1024, 0),
     (Q5_K, 512, 1024, 4096, 0),
     (Q5_K, 300, 520, 768, 256),
+    (Q5_K, 256, 256, 512, 257),
+    (Q5_K, 300, 520, 1024, 257),
+    (Q5_K, 512, 1024, 4096, 258),
+    (Q5_K, 190, 260, 2048, 258),
     # 256-tile with the walk cut into equal shares per CU (tiles summed with atomics)
     (Q4_K, 256, 256, 256, 258),
     (Q4_K, 300, 520, 768, 258),
