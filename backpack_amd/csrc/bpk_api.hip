@@ -81,6 +81,17 @@ struct DeviceState {
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 
+// Frees every device buffer of the state (hipFree(nullptr) is a no-op); the device must be current.
+void free_device_buffers(DeviceState& st)
+{
+    (void)hipFree(st.split.partial);
+    (void)hipFree(st.split.counters);
+    (void)hipFree(st.gemm_split.partial);
+    (void)hipFree(st.moe_tiles);
+    (void)hipFree(st.route_logits);
+    (void)hipFree(st.argmax_scratch);
+}
+
 int ensure_device(int device, DeviceState** out)
 {
     if (device < 0 || device >= kMaxDevices) return fail(BPK_ERR_DEVICE, "device %d out of range", device);
@@ -105,8 +116,13 @@ int ensure_device(int device, DeviceState** out)
         if (e == hipSuccess) e = hipMalloc((void**)&st.argmax_scratch, kArgmaxWords * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMemset(st.argmax_scratch, 0, kArgmaxWords * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMalloc((void**)&st.route_logits, kq::ROUTE_SPREAD_TOKENS * 1024u * sizeof(float));
+        if (e != hipSuccess) {
+            // nothing half-made stays behind: a later call starts from scratch
+            free_device_buffers(st);
+            st = DeviceState{};
+        }
         if (cur != device && cur >= 0) (void)hipSetDevice(cur);
-        if (e != hipSuccess) return hip_fail(e, "allocating split-K scratch");
+        if (e != hipSuccess) return hip_fail(e, "allocating the per-device scratch");
         st.split.capacity_floats = kPartialFloats;
         st.split.n_counters = kCounters;
         st.gemm_split.capacity_floats = kGemmPartialFloats;
@@ -209,11 +225,7 @@ int bpk_shutdown(void)
         DeviceState& st = g_dev[d];
         if (!st.ready) continue;
         (void)hipSetDevice(d);
-        (void)hipFree(st.split.partial);
-        (void)hipFree(st.split.counters);
-        (void)hipFree(st.moe_tiles);
-        (void)hipFree(st.route_logits);
-        (void)hipFree(st.argmax_scratch);
+        free_device_buffers(st);
         for (int b = 0; b < 2; ++b) {
             if (st.up.buf[b]) (void)hipHostFree(st.up.buf[b]);
             if (st.up.sent[b]) (void)hipEventDestroy(st.up.sent[b]);
