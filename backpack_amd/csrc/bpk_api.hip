@@ -23,6 +23,7 @@ constexpr uint32_t kCounters = 1u << 16;
 // bf16 GEMM: two 256 x 256 fp32 slots per workgroup for the runs of cut tiles, a workgroup per CU
 constexpr size_t kGemmPartialFloats = size_t(2) * 256 * 65536;  // 128 MiB
 constexpr size_t kMoeWords = size_t(4) << 20;       // 16 MiB of tile records for bpk_kq_moe_matmul
+static_assert(BPK_ARGMAX_STATIC_MAX_ROWS == kq::ARGMAX_MAX_ROWS, "the header's limit is the scratch array's");
 
 thread_local char t_err[512] = "";
 thread_local const char* t_kernel = "";
@@ -75,6 +76,7 @@ struct DeviceState {
     uint32_t* moe_tiles = nullptr;   // kMoeWords words
     uint32_t* argmax_scratch = nullptr;   // partial values | partial indices | tickets of bpk_argmax_rows
     float* route_logits = nullptr;   // ROUTE_SPREAD_TOKENS x 1024 router logits of a small-T route call
+    uint32_t* argmax_static = nullptr;    // this device's copy of the scratch array in the code object (not allocated)
     UploadStage up{};                // created by the first upload on the device
 };
 
@@ -116,6 +118,7 @@ int ensure_device(int device, DeviceState** out)
         if (e == hipSuccess) e = hipMalloc((void**)&st.argmax_scratch, kArgmaxWords * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMemset(st.argmax_scratch, 0, kArgmaxWords * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMalloc((void**)&st.route_logits, kq::ROUTE_SPREAD_TOKENS * 1024u * sizeof(float));
+        if (e == hipSuccess) e = kq::argmax_static_scratch(&st.argmax_static);   // with `device` current
         if (e != hipSuccess) {
             // nothing half-made stays behind: a later call starts from scratch
             free_device_buffers(st);
@@ -666,6 +669,33 @@ int bpk_argmax_rows(const float* logits, uint32_t M, uint32_t N, uint32_t ld, in
     uint32_t* tickets = pi + (size_t)kq::ARGMAX_MAX_ROWS * kq::ARGMAX_PARTS;
     const hipError_t e = kq::launch_argmax_rows(logits, M, N, ld, out_idx, out_val, pv, pi, tickets, (hipStream_t)stream);
     return e == hipSuccess ? BPK_OK : hip_fail(e, "argmax_rows");
+}
+
+int bpk_argmax_rows_static(const float* logits, uint32_t M, uint32_t N, uint32_t ld, int32_t* out_idx, float* out_val,
+                           void* stream)
+{
+    if (!logits || !out_idx) return fail(BPK_ERR_NULL, "logits and out_idx must be non-null");
+    if (N == 0 || ld < N) return fail(BPK_ERR_SHAPE, "N=%u must be positive and ld=%u at least N", N, ld);
+    if (M > BPK_ARGMAX_STATIC_MAX_ROWS)
+        return fail(BPK_ERR_SHAPE, "M=%u exceeds the %u rows the built-in scratch holds; split the call or use bpk_argmax_rows",
+                    M, (unsigned)BPK_ARGMAX_STATIC_MAX_ROWS);
+    if (M == 0) return BPK_OK;
+    int dev = -1;
+    const hipError_t eg = hipGetDevice(&dev);
+    if (eg != hipSuccess) return hip_fail(eg, "hipGetDevice");
+    uint32_t* base = nullptr;
+    if (dev >= 0 && dev < kMaxDevices) {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (g_dev[dev].ready) base = g_dev[dev].argmax_static;
+    }
+    // (never ensure_device here: that allocates)
+    if (!base)
+        return fail(BPK_ERR_DEVICE, "bpk_init(%d) must have run before bpk_argmax_rows_static: this call allocates nothing", dev);
+    float* pv = (float*)base;
+    uint32_t* pi = base + (size_t)kq::ARGMAX_MAX_ROWS * kq::ARGMAX_PARTS;
+    uint32_t* tickets = pi + (size_t)kq::ARGMAX_MAX_ROWS * kq::ARGMAX_PARTS;
+    const hipError_t e = kq::launch_argmax_rows(logits, M, N, ld, out_idx, out_val, pv, pi, tickets, (hipStream_t)stream);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, "argmax_rows_static");
 }
 
 int bpk_kq_matmul_argmax(int type, const float* X, const void* W, const float* bias, float* logits, uint32_t M,

@@ -71,6 +71,23 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const float* logits, u
     }
 }
 
+// Scratch of the entry point that allocates nothing (bpk_argmax_rows_static): partial values | partial
+// indices | tickets, the layout of the allocated scratch of bpk_argmax_rows, 132 096 bytes that every GPU
+// the library runs on holds until the process ends.  Zero when the code object is loaded; the last
+// workgroup of a row to arrive puts the row's ticket back to zero, so every launch finds its tickets
+// cleared.  In host code this name stands for the array only as a symbol: its device address, one per
+// GPU, comes from hipGetSymbolAddress below and is what launches are given.
+static __device__ __align__(256) __attribute__((used)) uint32_t scratch[ARGMAX_STATIC_WORDS];
+
+hipError_t argmax_static_scratch(uint32_t** out)
+{
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));   // of the current device
+    if (e != hipSuccess) return e;
+    *out = (uint32_t*)ptr;
+    return hipSuccess;
+}
+
 // scratch: ARGMAX_MAX_ROWS * ARGMAX_PARTS floats, as many words, ARGMAX_MAX_ROWS tickets (zero between launches)
 hipError_t launch_argmax_rows(const float* logits, uint32_t M, uint32_t N, uint32_t ld, int32_t* out_idx,
                               float* out_val, float* part_val, uint32_t* part_idx, uint32_t* tickets, hipStream_t s)

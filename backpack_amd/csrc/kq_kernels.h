@@ -76,6 +76,10 @@ hipError_t launch_route(const float* X, const float* router_w, uint32_t T, uint3
 constexpr uint32_t ARGMAX_PARTS = 64, ARGMAX_MAX_ROWS = 256;
 hipError_t launch_argmax_rows(const float* logits, uint32_t M, uint32_t N, uint32_t ld, int32_t* out_idx,
                               float* out_val, float* part_val, uint32_t* part_idx, uint32_t* tickets, hipStream_t s);
+// Device address, on the current device, of a scratch of ARGMAX_STATIC_WORDS words in that layout which
+// lives in the library's code object (no allocation): looked up once per device at set-up.
+constexpr size_t ARGMAX_STATIC_WORDS = (size_t)ARGMAX_MAX_ROWS * (2u * ARGMAX_PARTS + 1u);
+hipError_t argmax_static_scratch(uint32_t** out);
 
 // Any shape with K % 256 == 0, any 4-byte aligned W.  M tiled by 4 inside.
 hipError_t launch_matmul_generic(const MatmulArgs& a, hipStream_t s);

@@ -265,6 +265,24 @@ BPK_API int bpk_argmax_rows(const float *logits, uint32_t M, uint32_t N,
                             uint32_t ld, int32_t *out_idx, float *out_val,
                             void *stream);
 
+/* bpk_argmax_rows for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
+ * has no counterpart in the reference (whose argmax dispatches bind buffers made
+ * at load time, runtime/model_runner.cpp:2441-2453).  Same function and same
+ * kernel as bpk_argmax_rows; the per-row partial maxima and arrival tickets live
+ * in an array inside the library's code object (132 096 bytes per GPU, held
+ * until the process ends) instead of allocated scratch, and the call itself
+ * allocates and frees nothing.  bpk_init(device) must have run on the current
+ * device (that is where the array's address is looked up); otherwise
+ * BPK_ERR_DEVICE.  At most BPK_ARGMAX_STATIC_MAX_ROWS rows per call
+ * (BPK_ERR_SHAPE beyond); any N.  All calls on one GPU share the array: calls
+ * on different streams of one GPU that overlap in time race.  The tickets are
+ * zero when the library is loaded and each launch leaves them zero again. */
+#define BPK_ARGMAX_STATIC_MAX_ROWS 256u
+BPK_API int bpk_argmax_rows_static(const float *logits, uint32_t M, uint32_t N,
+                                   uint32_t ld, int32_t *out_idx,
+                                   float *out_val, void *stream);
+
 /* lm_head and its argmax in one call (runtime/model_runner.cpp:4124-4135 then
  * :2441-2453): bpk_kq_matmul with y_offset 0 into `logits` (f32 [M,N], kept for
  * the caller) followed by bpk_argmax_rows on it. */
