@@ -41,7 +41,9 @@ def _compile(src: str) -> str:
     r = subprocess.run(cmd, capture_output=True, text=True)
     lines = r.stderr.splitlines()
     if guarded:
-        bad = [l for l in lines if re.search(r"(Spill|ScratchSize[^:]*):\s*[1-9]", l)]
+        # (scalar registers spilled into lanes of a reserved vector register are harmless here: no register
+        # with a load in flight moves; vector spills and scratch memory are what must not happen)
+        bad = [l for l in lines if re.search(r"(VGPRs Spill|ScratchSize[^:]*):\s*[1-9]", l)]
         if bad and r.returncode == 0:
             raise RuntimeError(f"{src} must not spill registers (hand-waited loads):\n" + "\n".join(bad[:8]))
         lines = [l for l in lines if "kernel-resource-usage" not in l and not re.match(r"^\s*\d*\s*\|", l)]

@@ -35,6 +35,12 @@ class Fusion(C.Structure):
                 ("epilogue", C.c_int)]
 
 
+class ChainOp(C.Structure):
+    _fields_ = [("type", C.c_int), ("X", C.c_void_p), ("W", C.c_void_p), ("bias", C.c_void_p), ("Y", C.c_void_p),
+                ("N", C.c_uint32), ("K", C.c_uint32), ("n_blocks", C.c_uint32), ("row_stride_words", C.c_uint32),
+                ("y_offset", C.c_uint32), ("fusion", Fusion)]
+
+
 PRO_NONE, PRO_RMS_NORM, PRO_SILU_MUL, PRO_GELU_MUL = range(4)
 EPI_NONE, EPI_SILU_MUL, EPI_GELU_MUL = 0, 2, 3
 
@@ -91,6 +97,11 @@ _SIGS = {
     "bpk_kq_moe_matmul": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
                                     C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32,
                                     C.c_int, C.c_void_p]),
+    "bpk_chain_create": (C.c_int, [C.POINTER(ChainOp), C.c_uint32, C.POINTER(C.c_void_p)]),
+    "bpk_chain_run": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]),
+    "bpk_chain_status": (C.c_int, [C.c_void_p]),
+    "bpk_chain_reset": (C.c_int, [C.c_void_p]),
+    "bpk_chain_destroy": (C.c_int, [C.c_void_p]),
     "bpk_argmax_rows": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "bpk_argmax_rows_static": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p,
                                          C.c_void_p]),

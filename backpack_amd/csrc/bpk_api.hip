@@ -32,6 +32,9 @@ thread_local kq::GemvTuning t_gemv;
 thread_local int t_gemm_tile = 0;
 thread_local int t_gemm_split = 0;
 thread_local int t_fused_separate = 0;
+thread_local int t_chain_spin_us = 0;    // 0 = default
+thread_local int t_chain_ahead = 0;      // 1 + rows touched ahead; 0 = default
+thread_local int t_chain_hold = 0;
 
 int fail(int code, const char* fmt, ...)
 {
@@ -207,6 +210,20 @@ int bpk_set_option(const char* name, int value)
     }
     if (!strcmp(name, "fused_separate")) {
         t_fused_separate = value != 0;
+        return BPK_OK;
+    }
+    if (!strcmp(name, "chain_ahead")) {
+        if (value < 0 || value > 9) return fail(BPK_ERR_SHAPE, "chain_ahead must be 0..9");
+        t_chain_ahead = value;
+        return BPK_OK;
+    }
+    if (!strcmp(name, "chain_spin_us")) {
+        if (value < 0) return fail(BPK_ERR_SHAPE, "chain_spin_us must not be negative");
+        t_chain_spin_us = value;
+        return BPK_OK;
+    }
+    if (!strcmp(name, "chain_hold")) {
+        t_chain_hold = value != 0;
         return BPK_OK;
     }
     if (!strcmp(name, "gemm_split")) {
@@ -654,6 +671,203 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
         e = kq::launch_matmul_generic(a, s);
     }
     return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+struct bpk_chain {
+    int device = 0;
+    uint32_t n_ops = 0;
+    uint32_t max_k = 0;
+    kq::ChainOp* d_ops = nullptr;      // n_ops descriptors
+    uint32_t* d_words = nullptr;       // n_ops parity words, the arrival counter, the error word
+    float* d_mail = nullptr;           // the ops' mailboxes, back to back
+    size_t mail_floats = 0;
+};
+
+namespace {
+
+struct Span {
+    uintptr_t lo, hi;   // [lo, hi)
+    bool overlaps(const Span& o) const { return lo < o.hi && o.lo < hi; }
+    bool inside(const Span& o) const { return lo >= o.lo && hi <= o.hi; }
+};
+
+// Words of a fresh chain: every mailbox entry carries parity 0, so the first run writes parity 1.
+hipError_t chain_arm(bpk_chain* c)
+{
+    std::vector<uint32_t> w(c->n_ops + 2u, 1u);
+    w[c->n_ops] = 0;        // arrivals
+    w[c->n_ops + 1u] = 0;   // error
+    hipError_t e = hipMemcpy(c->d_words, w.data(), w.size() * sizeof(uint32_t), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemset(c->d_mail, 0, c->mail_floats * sizeof(float));
+    return e;
+}
+
+}  // namespace
+
+int bpk_chain_create(const bpk_chain_op* ops, uint32_t n_ops, bpk_chain** out)
+{
+    if (!ops || !out) return fail(BPK_ERR_NULL, "ops and out must be non-null");
+    if (n_ops == 0 || n_ops > kq::CHAIN_MAX_OPS) return fail(BPK_ERR_SHAPE, "n_ops=%u out of range (1..%u)", n_ops, kq::CHAIN_MAX_OPS);
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
+    std::vector<kq::ChainOp> h(n_ops);
+    std::vector<Span> out_span(n_ops), x_span(n_ops), r_span(n_ops);
+    std::vector<size_t> mail_at(n_ops);
+    uint32_t max_k = 0;
+    size_t mail_floats = 0;
+    for (uint32_t i = 0; i < n_ops; ++i) {
+        const bpk_chain_op& o = ops[i];
+        const bpk_kq_fusion& f = o.fusion;
+        if (o.type != BPK_TYPE_Q4_K && o.type != BPK_TYPE_Q6_K)
+            return fail(BPK_ERR_TYPE, "op %u: a chain takes Q4_K and Q6_K (type %d)", i, o.type);
+        if (f.prologue < BPK_PRO_NONE || f.prologue > BPK_PRO_GELU_MUL) return fail(BPK_ERR_SHAPE, "op %u: prologue %d unknown", i, f.prologue);
+        if (f.epilogue != BPK_EPI_NONE && f.epilogue != BPK_EPI_SILU_MUL && f.epilogue != BPK_EPI_GELU_MUL)
+            return fail(BPK_ERR_SHAPE, "op %u: epilogue %d unknown", i, f.epilogue);
+        const bool epi = f.epilogue != BPK_EPI_NONE;
+        if (epi && f.residual) return fail(BPK_ERR_SHAPE, "op %u: an epilogue takes no residual", i);
+        if (epi && o.N > 0x7FFFFFFFu) return fail(BPK_ERR_SHAPE, "op %u: N too large", i);
+        if (f.prologue == BPK_PRO_RMS_NORM && !f.norm_w) return fail(BPK_ERR_NULL, "op %u: norm_w must be non-null for the norm prologue", i);
+        const uint32_t w_rows = epi ? 2u * o.N : o.N;
+        if (int rc = check_matmul(o.type, o.X, o.W, o.Y, 1, w_rows, o.K, o.n_blocks, o.row_stride_words)) return rc;
+        if (((uintptr_t)o.X | (uintptr_t)f.norm_w) & 15u) return fail(BPK_ERR_ALIGN, "op %u: X and norm_w must be 16-byte aligned", i);
+        if (o.type == BPK_TYPE_Q4_K && (((uintptr_t)o.W & 15u) || ((o.row_stride_words * 4u) & 15u)))
+            return fail(BPK_ERR_ALIGN, "op %u: Q4_K rows must be 16-byte aligned", i);
+        const int mode = kq::chain_mode_for(o.type, o.n_blocks, f.epilogue);
+        if (mode < 0)
+            return fail(BPK_ERR_SHAPE, "op %u: a chain has no kernel form for type %d with K=%u%s", i, o.type, o.K,
+                        epi ? " and an epilogue" : "");
+        const size_t x_len = (f.prologue >= BPK_PRO_SILU_MUL ? 2u : 1u) * (size_t)o.K;
+        x_span[i] = Span{(uintptr_t)o.X, (uintptr_t)(o.X + x_len)};
+        out_span[i] = Span{(uintptr_t)(o.Y + o.y_offset), (uintptr_t)(o.Y + o.y_offset + o.N)};
+        r_span[i] = f.residual ? Span{(uintptr_t)(f.residual + o.y_offset), (uintptr_t)(f.residual + o.y_offset + o.N)} : Span{0, 0};
+        kq::ChainOp& d = h[i];
+        d = kq::ChainOp{};
+        d.W = (const uint8_t*)o.W; d.X = o.X; d.bias = o.bias; d.Y = o.Y;
+        d.norm_w = f.prologue == BPK_PRO_RMS_NORM ? f.norm_w : nullptr;
+        d.residual = f.residual;
+        d.x_src = d.res_src = kq::CHAIN_NO_SRC;
+        d.N = w_rows; d.K = o.K; d.n_blocks = o.n_blocks; d.row_stride_bytes = o.row_stride_words * 4u;
+        d.y_offset = o.y_offset;
+        d.pro = (uint32_t)f.prologue; d.epi = (uint32_t)f.epilogue; d.eps = f.eps;
+        d.mode = (uint32_t)mode;
+        if (o.K > max_k) max_k = o.K;
+        mail_at[i] = mail_floats;
+        mail_floats += ((size_t)o.N + 63u) & ~(size_t)63u;
+        // who writes what this op reads: the latest earlier op whose outputs overlap the range
+        for (int pass = 0; pass < 2; ++pass) {
+            const Span& rd = pass == 0 ? x_span[i] : r_span[i];
+            if (rd.lo == rd.hi) continue;
+            for (uint32_t j = i; j-- > 0;) {
+                if (!rd.overlaps(out_span[j])) continue;
+                const size_t delta = (rd.lo - out_span[j].lo) / sizeof(float);
+                if (!rd.inside(out_span[j]) || (pass == 0 && (delta & 1u)))
+                    return fail(BPK_ERR_SHAPE, "op %u reads part of the outputs of op %u: an input must lie inside one earlier "
+                                "op's outputs (at an even element) or outside all of them", i, j);
+                if (pass == 0) { d.x_src = j; d.x_mail = (const float*)0 + mail_at[j] + delta; }
+                else { d.res_src = j; d.res_mail = (const float*)0 + mail_at[j] + delta; }
+                break;
+            }
+        }
+        // What this op overwrites must not be in use by an earlier op that may still be running somewhere.
+        // An op starts once the whole mailbox of the op that writes its X is filled, which every reader and
+        // writer of that op's buffers precedes; so the ops ordered before op i are the chain of its X's
+        // producers, and only those may share a buffer with its output.
+        for (uint32_t k = 0; k < i; ++k) {
+            if (!(out_span[i].overlaps(x_span[k]) || out_span[i].overlaps(out_span[k]) ||
+                  (r_span[k].hi && out_span[i].overlaps(r_span[k]))))
+                continue;
+            bool ordered = false;
+            for (uint32_t j = d.x_src; j != kq::CHAIN_NO_SRC && j >= k; j = h[j].x_src)
+                if (j == k) { ordered = true; break; }
+            if (!ordered)
+                return fail(BPK_ERR_SHAPE, "op %u writes a buffer that op %u reads or writes, and nothing orders the two "
+                            "(an op follows the ops that lead to its X)", i, k);
+        }
+    }
+    if (kq::chain_lds_bytes(max_k) > kq::CHAIN_MAX_LDS) return fail(BPK_ERR_SHAPE, "K=%u exceeds what a workgroup can stage", max_k);
+    bpk_chain* c = new (std::nothrow) bpk_chain;
+    if (!c) return fail(BPK_ERR_SHAPE, "out of host memory");
+    (void)hipGetDevice(&c->device);
+    c->n_ops = n_ops;
+    c->max_k = max_k;
+    c->mail_floats = mail_floats;
+    hipError_t e = hipMalloc((void**)&c->d_ops, n_ops * sizeof(kq::ChainOp));
+    if (e == hipSuccess) e = hipMalloc((void**)&c->d_words, (n_ops + 2u) * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc((void**)&c->d_mail, mail_floats * sizeof(float));
+    if (e == hipSuccess) {
+        for (uint32_t i = 0; i < n_ops; ++i) {
+            h[i].y_mail = c->d_mail + mail_at[i];
+            if (h[i].x_src != kq::CHAIN_NO_SRC) h[i].x_mail = c->d_mail + (h[i].x_mail - (const float*)0);
+            if (h[i].res_src != kq::CHAIN_NO_SRC) h[i].res_mail = c->d_mail + (h[i].res_mail - (const float*)0);
+        }
+        e = hipMemcpy(c->d_ops, h.data(), n_ops * sizeof(kq::ChainOp), hipMemcpyHostToDevice);
+    }
+    if (e == hipSuccess) e = chain_arm(c);
+    if (e != hipSuccess) {
+        (void)hipFree(c->d_ops);
+        (void)hipFree(c->d_words);
+        (void)hipFree(c->d_mail);
+        delete c;
+        return hip_fail(e, "creating a chain");
+    }
+    *out = c;
+    return BPK_OK;
+}
+
+int bpk_chain_run(bpk_chain* c, uint32_t first, uint32_t count, void* stream)
+{
+    if (!c) return fail(BPK_ERR_NULL, "chain must be non-null");
+    if (count == 0) return BPK_OK;
+    if (first >= c->n_ops || count > c->n_ops - first)
+        return fail(BPK_ERR_SHAPE, "ops [%u, %u + %u) outside the chain's %u", first, first, count, c->n_ops);
+    if (count > kq::CHAIN_MAX_PER_LAUNCH) return fail(BPK_ERR_SHAPE, "a launch walks at most %u ops (asked for %u)", kq::CHAIN_MAX_PER_LAUNCH, count);
+    int dev = -1;
+    (void)hipGetDevice(&dev);
+    if (dev != c->device) return fail(BPK_ERR_DEVICE, "the chain was created on device %d, current is %d", c->device, dev);
+    kq::ChainLaunch a{};
+    a.ops = c->d_ops;
+    a.parity = c->d_words;
+    a.arrivals = c->d_words + c->n_ops;
+    a.error = c->d_words + c->n_ops + 1u;
+    a.first = first;
+    a.count = count;
+    a.max_k = c->max_k;
+    a.hold = (uint32_t)t_chain_hold;
+    a.ahead = t_chain_ahead > 0 ? (uint32_t)t_chain_ahead - 1u : 2u;
+    a.spin_ticks = (uint64_t)(t_chain_spin_us > 0 ? t_chain_spin_us : 2000000) * 100u;   // 100 MHz wall clock
+    t_kernel = "chain";
+    const hipError_t e = kq::launch_chain(a, kq::device_cu_count(), (hipStream_t)stream);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+int bpk_chain_status(bpk_chain* c)
+{
+    if (!c) return fail(BPK_ERR_NULL, "chain must be non-null");
+    uint32_t word = 0;
+    const hipError_t e = hipMemcpy(&word, c->d_words + c->n_ops + 1u, sizeof word, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e, "reading the chain's error word");
+    if (word == 0) return BPK_OK;
+    return fail(BPK_ERR_TIMEOUT, "a launch of the chain gave up waiting for the inputs of op %u (the grid was not all "
+                "resident, or the ops that write them were not part of the launch's past); its outputs are incomplete", word >> 8);
+}
+
+int bpk_chain_reset(bpk_chain* c)
+{
+    if (!c) return fail(BPK_ERR_NULL, "chain must be non-null");
+    hipError_t e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = chain_arm(c);
+    return e == hipSuccess ? BPK_OK : hip_fail(e, "resetting a chain");
+}
+
+int bpk_chain_destroy(bpk_chain* c)
+{
+    if (!c) return BPK_OK;
+    hipError_t e = hipFree(c->d_ops);
+    const hipError_t e2 = hipFree(c->d_words), e3 = hipFree(c->d_mail);
+    delete c;
+    if (e == hipSuccess) e = e2;
+    if (e == hipSuccess) e = e3;
+    return e == hipSuccess ? BPK_OK : hip_fail(e, "hipFree(chain)");
 }
 
 int bpk_argmax_rows(const float* logits, uint32_t M, uint32_t N, uint32_t ld, int32_t* out_idx, float* out_val,

@@ -132,6 +132,53 @@ hipError_t launch_moe_combine(const float* down, const float* wt, float* out, ui
 bool gemm_bf16_supported(const MatmulArgs& a);
 hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const SplitScratch& gemm_scratch, hipStream_t s);
 
+// A chain of decode matvecs (M = 1) in one launch: a persistent grid walks ops[first .. first + count).
+struct ChainOp {                 // device-resident, written once when the chain is created
+    const uint8_t* W;            // packed rows
+    const float* X;              // f32 [K]; [2K] (gate | up) for the act prologues
+    const float* bias;           // [N] or nullptr
+    float* Y;
+    const float* norm_w;         // [K], pro == 1
+    const float* residual;       // indexed like Y, or nullptr
+    // Mailboxes (owned by the chain): a copy of an op's outputs, written through to memory, whose lowest
+    // mantissa bit carries the parity of the run.  y_mail: this op's; x_mail / res_mail: where, in the mailbox
+    // of op x_src / res_src, this op's X row / its residual elements start (used when that op belongs to
+    // the same launch; otherwise X / residual are read from the caller's buffers).
+    float* y_mail;
+    const float* x_mail;
+    const float* res_mail;
+    uint32_t x_src, res_src;     // op indices, or CHAIN_NO_SRC
+    uint32_t N;                  // rows of W (twice the outputs with an epilogue)
+    uint32_t K, n_blocks, row_stride_bytes, y_offset;
+    uint32_t pro, epi;           // as MatmulArgs
+    float eps;
+    uint32_t mode;               // CHAIN_MODE_* bits, from chain_mode_for
+};
+constexpr uint32_t CHAIN_NO_SRC = 0xFFFFFFFFu;
+constexpr uint32_t CHAIN_MODE_P2 = 1u;     // two passes of eight superblocks per wave (else one)
+constexpr uint32_t CHAIN_MODE_SLICED = 2u; // the waves of a workgroup share rows, a K slice each (else a wave per row)
+constexpr uint32_t CHAIN_MODE_Q6 = 4u;     // Q6_K (else Q4_K)
+constexpr int CHAIN_WAVES = 8;
+constexpr uint32_t CHAIN_MAX_OPS = 1024;
+constexpr uint32_t CHAIN_MAX_PER_LAUNCH = 64;   // ops one launch walks (their descriptors sit in LDS)
+constexpr size_t CHAIN_MAX_LDS = (size_t)156 << 10;   // dynamic LDS a chain launch may ask for
+constexpr uint32_t CHAIN_ERR_TIMEOUT = 1u; // low byte of the error word; the op index sits above it
+struct ChainLaunch {
+    const ChainOp* ops;
+    uint32_t* parity;            // per op: the bit this run's mailbox entries carry (flipped when a launch ends)
+    uint32_t* arrivals;          // workgroups that have finished the launch; zero between launches
+    uint32_t* error;             // 0, or CHAIN_ERR_* | op << 8 once a thread gave up waiting
+    uint32_t first, count;
+    uint32_t max_k;              // floats of x the LDS holds
+    uint32_t hold;               // testing: 1 keeps the ops from filling their mailboxes, so every wait runs out
+    uint32_t ahead;              // rows per wave touched into L2 behind the staged first rows of the next op
+    uint64_t spin_ticks;         // bound of a wait, in ticks of the 100 MHz wall clock
+};
+// CHAIN_MODE_* bits for a matrix, or -1 where the chain kernel has no form for it.
+int chain_mode_for(int type, uint32_t n_blocks, int epi);
+size_t chain_lds_bytes(uint32_t max_k);
+hipError_t launch_chain(const ChainLaunch& a, uint32_t workgroups, hipStream_t s);
+
 // Compute units of the current device (cached per device id).
 inline uint32_t device_cu_count()
 {

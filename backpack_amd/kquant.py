@@ -168,6 +168,55 @@ def matmul_fused(x: torch.Tensor, w: KQuantPacked, prologue: int = capi.PRO_NONE
     return out
 
 
+class Chain:
+    """A recorded list of decode matvecs (M = 1) with their fused forms; run(first, count) issues a stretch
+    of it as one launch (bpk_chain_*).  Ops are added with the arguments of matmul_fused; an op whose x or
+    residual is the output buffer of an earlier op follows that op."""
+
+    def __init__(self):
+        self._ops, self._keep, self._h = [], [], None
+
+    def add(self, x, w: KQuantPacked, out, prologue=capi.PRO_NONE, norm_w=None, eps=0.0, residual=None, bias=None,
+            epilogue=capi.EPI_NONE, y_offset=0) -> int:
+        assert self._h is None, "the chain is already built"
+        n_out = w.N // 2 if epilogue else w.N
+        op = capi.ChainOp(w.type, _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out), n_out, w.K, w.n_blocks,
+                          w.row_stride_words, y_offset,
+                          capi.Fusion(prologue, _ptr(norm_w), eps, _ptr(residual), epilogue))
+        self._ops.append(op)
+        self._keep.append((x, w, out, norm_w, residual, bias))      # the buffers live as long as the chain
+        return len(self._ops) - 1
+
+    def build(self) -> "Chain":
+        import ctypes as C
+        arr = (capi.ChainOp * len(self._ops))(*self._ops)
+        h = C.c_void_p()
+        capi.check(capi.lib().bpk_chain_create(arr, len(self._ops), C.byref(h)))
+        self._h = h
+        return self
+
+    def __len__(self):
+        return len(self._ops)
+
+    def run(self, first: int = 0, count: int | None = None) -> None:
+        count = len(self._ops) - first if count is None else count
+        capi.check(capi.lib().bpk_chain_run(self._h, first, count, _stream()))
+
+    def status(self) -> None:
+        capi.check(capi.lib().bpk_chain_status(self._h))
+
+    def reset(self) -> None:
+        capi.check(capi.lib().bpk_chain_reset(self._h))
+
+    def __del__(self):
+        try:
+            if self._h:
+                capi.lib().bpk_chain_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
 def argmax_rows(logits: torch.Tensor):
     """(index int32 [M], value f32 [M]) of the largest element of each row; lowest index on ties."""
     assert logits.is_cuda and logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1

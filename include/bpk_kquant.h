@@ -49,7 +49,8 @@ enum {
     BPK_ERR_WORKSPACE = -7, /* workspace missing or too small                 */
     BPK_ERR_IO = -8,        /* a file could not be opened or mapped           */
     BPK_ERR_FORMAT = -9,    /* not a GGUF file, or truncated / inconsistent   */
-    BPK_ERR_NOT_FOUND = -10 /* no tensor / metadata element of that name      */
+    BPK_ERR_NOT_FOUND = -10,/* no tensor / metadata element of that name      */
+    BPK_ERR_TIMEOUT = -11   /* a chain launch gave up a wait between its ops  */
 };
 
 /* Library version, major*10000 + minor*100 + patch. */
@@ -253,6 +254,62 @@ BPK_API int bpk_kq_matmul_fused(int type, const float *X, const void *W,
                                 const bpk_kq_fusion *fusion, void *workspace,
                                 size_t workspace_bytes, void *stream);
 
+/* ---- chains of decode matvecs: replaces a recorded stretch of the dispatch list ----
+ * The reference records one token's dispatches once (buildDecodePipeline) and
+ * replays the list per token (runtime/model_runner.cpp:5725-5759).  Between two
+ * attention blocks that list is k-quant matvecs and the elementwise dispatches
+ * around them: o + add_inplace (runtime/model_runner.cpp:3324-3330), rms_norm,
+ * gate|up, act_mul, down + add_inplace (:3711-3793), rms_norm and q|k|v of the
+ * next layer (:3206-3243).  A chain holds such a list as bpk_kq_matmul_fused
+ * calls with M = 1 and runs any stretch of it, ops [first, first + count), as
+ * ONE launch: a persistent grid walks the ops in order without draining between
+ * them; an op whose X (or residual) is the output of an earlier op of the launch
+ * starts as soon as those outputs have arrived, and the next op's weights are
+ * already being fetched while it waits.  Which op feeds which is found from the
+ * pointers: an input that lies inside an earlier op's output range comes from
+ * that op.  Results are those of the same bpk_kq_matmul_fused calls issued one
+ * after the other, except that an input handed from op to op inside a launch
+ * has its lowest mantissa bit cleared (a relative 2^-24; Y itself is exact).
+ *
+ * Each op: the arguments of bpk_kq_matmul_fused with M = 1 (N counts outputs; W
+ * has 2N rows with an epilogue).  Served: Q4_K and Q6_K, K <= 32768, X and norm_w
+ * 16-byte aligned, Q4_K rows 16-byte aligned; the act(gate)*up epilogue for Q4_K
+ * with K <= 4096.  An input must lie wholly inside one earlier op's outputs or
+ * outside all of them, and an op may overwrite a buffer an earlier op uses only
+ * if it follows that op through its X (as x += down(...) follows o).
+ * bpk_chain_create refuses anything else with BPK_ERR_SHAPE / BPK_ERR_TYPE /
+ * BPK_ERR_ALIGN (issue such ops as separate calls).  Pointers are captured at
+ * creation, like the reference's bind groups; the buffers must stay valid while
+ * the chain lives.
+ *
+ * bpk_chain_run is asynchronous on `stream`, allocates nothing and may be
+ * captured into a HIP graph.  Launches of one chain must not overlap in time,
+ * and nothing else should occupy the GPU's compute units while one runs: an op
+ * waits for the workgroups that produce its input, every wait is bounded (about
+ * two seconds), and a launch whose workgroups were not all resident gives up,
+ * leaves outputs unwritten and records the fact.  bpk_chain_status
+ * (synchronises with the device) returns BPK_ERR_TIMEOUT once that has
+ * happened, and launches do nothing until bpk_chain_reset. */
+typedef struct bpk_chain bpk_chain;
+
+typedef struct bpk_chain_op {
+    int type;                  /* BPK_TYPE_Q4_K or BPK_TYPE_Q6_K              */
+    const float *X;            /* f32 [K], or [2K] for the act prologues      */
+    const void *W;
+    const float *bias;         /* f32 [rows of W] or NULL                     */
+    float *Y;
+    uint32_t N, K, n_blocks, row_stride_words, y_offset;
+    bpk_kq_fusion fusion;      /* prologue, norm_w, eps, residual, epilogue   */
+} bpk_chain_op;
+
+BPK_API int bpk_chain_create(const bpk_chain_op *ops, uint32_t n_ops,
+                             bpk_chain **out);
+BPK_API int bpk_chain_run(bpk_chain *c, uint32_t first, uint32_t count,
+                          void *stream);
+BPK_API int bpk_chain_status(bpk_chain *c);
+BPK_API int bpk_chain_reset(bpk_chain *c);
+BPK_API int bpk_chain_destroy(bpk_chain *c);
+
 /* ---- greedy sampling tail: replaces argmax + argmax_reduce -----------------
  * The two dispatches after the lm_head matvec (kernels argmax.wgsl /
  * argmax_reduce.wgsl, wired in runtime/model_runner.cpp:2441-2453), as one
@@ -406,8 +463,12 @@ BPK_API int bpk_force_kernel(int family);
  * equal shares per compute unit; the runs of a tile cut between workgroups go
  * through a per-device workspace and are added in the order of the walk, so
  * results repeat bit for bit); "fused_separate": 1 makes bpk_kq_matmul_fused run its prologue,
- * matmul and add as separate launches for every shape (needs the workspace).
- * 0 = automatic. */
+ * matmul and add as separate launches for every shape (needs the workspace);
+ * "chain_spin_us": bound of a wait between the ops of a chain in microseconds;
+ * "chain_hold": 1 keeps the ops of a chain from handing their outputs on, so
+ * that every wait for them runs out (the way the tests reach the give-up path
+ * with every workgroup exiting normally); "chain_ahead": 1 + the rows per wave
+ * of the next op touched into L2 while an op finishes.  0 = automatic. */
 BPK_API int bpk_set_option(const char *name, int value);
 
 #ifdef __cplusplus
