@@ -102,6 +102,7 @@ _SIGS = {
     "bpk_chain_status": (C.c_int, [C.c_void_p]),
     "bpk_chain_reset": (C.c_int, [C.c_void_p]),
     "bpk_chain_destroy": (C.c_int, [C.c_void_p]),
+    "bpk_chain_trace": (C.c_int, [C.c_void_p]),
     "bpk_argmax_rows": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "bpk_argmax_rows_static": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p,
                                          C.c_void_p]),

@@ -34,6 +34,7 @@ thread_local int t_gemm_split = 0;
 thread_local int t_fused_separate = 0;
 thread_local int t_chain_spin_us = 0;    // 0 = default
 thread_local int t_chain_ahead = 0;      // 1 + rows touched ahead; 0 = default
+thread_local void* t_chain_trace = nullptr;   // device buffer for the chain kernel's time stamps (diagnostics)
 thread_local int t_chain_hold = 0;
 
 int fail(int code, const char* fmt, ...)
@@ -833,11 +834,18 @@ int bpk_chain_run(bpk_chain* c, uint32_t first, uint32_t count, void* stream)
     a.count = count;
     a.max_k = c->max_k;
     a.hold = (uint32_t)t_chain_hold;
-    a.ahead = t_chain_ahead > 0 ? (uint32_t)t_chain_ahead - 1u : 2u;
+    a.ahead = t_chain_ahead > 0 ? (uint32_t)t_chain_ahead - 1u : 0u;   // (measured: touching ahead gains nothing)
+    a.trace = (uint64_t*)t_chain_trace;
     a.spin_ticks = (uint64_t)(t_chain_spin_us > 0 ? t_chain_spin_us : 2000000) * 100u;   // 100 MHz wall clock
     t_kernel = "chain";
     const hipError_t e = kq::launch_chain(a, kq::device_cu_count(), (hipStream_t)stream);
     return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+int bpk_chain_trace(void* stamps)
+{
+    t_chain_trace = stamps;
+    return BPK_OK;
 }
 
 int bpk_chain_status(bpk_chain* c)

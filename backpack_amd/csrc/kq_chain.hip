@@ -102,79 +102,113 @@ __device__ __forceinline__ float block_sum(float v, float* red, uint32_t wave, u
     return t;
 }
 
-// Two consecutive activations of the op's input: from the caller's buffer, or from the mailbox of the op
-// of this launch that writes them (polled until both carry the run's parity).
-__device__ __forceinline__ float2 chain_x2(const float* plain, const float* mail, bool from_chain, uint32_t par, const Patience& pt,
-                                           int& bad)
+// A thread's share of the op's input: XB pairs of activations (pair tid + 512 u), 64-bit loads that are all
+// in flight together: one memory round trip, not one per pair.  No branch around a load (with one the
+// compiler waits for each load before it issues the next): a pair past the end re-reads the last one and is
+// zeroed afterwards.  From the caller's buffer, or from the mailbox of the op of this launch that writes
+// them: then the loads are repeated until every pair carries the run's parity.
+template <int XB>
+__device__ __forceinline__ void chain_x_load(float2 (&v)[XB], const float* plain, const float* mail, bool from_chain, uint32_t par,
+                                             uint32_t half, const Patience& pt, int& bad)
 {
+    const uint32_t tid = threadIdx.x;
+    uint32_t at[XB];
+#pragma unroll
+    for (int u = 0; u < XB; ++u) at[u] = 2u * min(tid + u * CHAIN_THREADS, half - 1u);
     if (!mail) {
-        // written by an op of the chain in an earlier launch: the same value as through the mailbox, so that
-        // results do not depend on where a chain is cut into launches
-        float2 v = *(const float2*)plain;
-        if (from_chain) { v.x = tag(v.x, 0u); v.y = tag(v.y, 0u); }
-        return v;
+#pragma unroll
+        for (int u = 0; u < XB; ++u) v[u] = *(const float2*)(plain + at[u]);
+    } else {
+        uint64_t t0 = 0;
+        uint32_t tries = 0;
+        // While the producers are still at work, a workgroup polls a sample (one pair per thread, 4 KB instead
+        // of the whole x): every compute unit reading all of x from memory again and again takes the
+        // bandwidth the producers' last rows need.  Once the sample is there nearly everything is.
+        for (;;) {
+            const float2 probe = ld_agent2(mail + at[0]);
+            if (tagged(probe.x, par) && tagged(probe.y, par)) break;
+            if (give_up(pt, t0, tries)) { bad = 1; break; }
+        }
+        uint32_t pending = bad ? 0u : 1u;
+        while (pending) {
+            // (all of them again: the ones that had arrived are still there, and no load waits for another)
+#pragma unroll
+            for (int u = 0; u < XB; ++u) v[u] = ld_agent2(mail + at[u]);
+            pending = 0;
+#pragma unroll
+            for (int u = 0; u < XB; ++u)
+                if (!(tagged(v[u].x, par) && tagged(v[u].y, par))) pending |= 1u << u;
+            if (pending && give_up(pt, t0, tries)) { bad = 1; break; }
+        }
     }
-    uint64_t t0 = 0;
-    uint32_t tries = 0;
-    float2 v = ld_agent2(mail);
-    while (!(tagged(v.x, par) && tagged(v.y, par))) {
-        if (give_up(pt, t0, tries)) { bad = 1; break; }
-        v = ld_agent2(mail);
+#pragma unroll
+    for (int u = 0; u < XB; ++u) {
+        if (tid + u * CHAIN_THREADS >= half) v[u] = float2{0.0f, 0.0f};
+        // the flag bit is cleared whatever the run's parity (the same x from run to run), also where the
+        // values come from an op of the chain in an earlier launch (the same x wherever a chain is cut)
+        else if (from_chain) { v[u].x = tag(v[u].x, 0u); v[u].y = tag(v[u].y, 0u); }
     }
-    // (the flag bit is cleared, whatever the run's parity: the same x from run to run)
-    v.x = tag(v.x, 0u);
-    v.y = tag(v.y, 0u);
-    return v;
 }
 
 // x of the op -> xs[0..K), prologue applied (runtime/kernels/norm/rms_norm.wgsl:15-20,
-// fused/silu_mul_fused.wgsl:39-49, fused/gelu_mul_fused.wgsl:22-32).  Returns false (for the whole
-// workgroup) when a wait was given up.  Ends with a barrier.
-__device__ __forceinline__ bool chain_stage_x(const ChainOp& p, const float* mail, uint32_t par, const Patience& pt, float* xs,
-                                              float* red, volatile uint32_t* gave_up, uint32_t wave, uint32_t lane)
+// fused/silu_mul_fused.wgsl:39-49, fused/gelu_mul_fused.wgsl:22-32), for K <= 1024 XB.  Returns false (for
+// the whole workgroup) when a wait was given up.  Ends with a barrier.
+template <int XB>
+__device__ __forceinline__ bool chain_stage_x_n(const ChainOp& p, const float* mail, uint32_t par, const Patience& pt, float* xs,
+                                                float* red, volatile uint32_t* gave_up, uint32_t wave, uint32_t lane)
 {
     const uint32_t tid = threadIdx.x;
     const uint32_t half = p.K >> 1;   // K is a multiple of 256
     const bool fc = p.x_src != CHAIN_NO_SRC;
     int bad = 0;
+    float2 v[XB];
+    chain_x_load<XB>(v, p.X, mail, fc, par, half, pt, bad);
     if (p.pro == STREAM_PRO_SILU || p.pro == STREAM_PRO_GELU) {
-        for (uint32_t i = tid; i < half; i += CHAIN_THREADS) {
-            const float2 g = chain_x2(p.X + 2u * i, mail ? mail + 2u * i : nullptr, fc, par, pt, bad);
-            const float2 u = chain_x2(p.X + p.K + 2u * i, mail ? mail + p.K + 2u * i : nullptr, fc, par, pt, bad);
-            float2 r;
+        float2 up[XB];
+        chain_x_load<XB>(up, p.X + p.K, mail ? mail + p.K : nullptr, fc, par, half, pt, bad);
+#pragma unroll
+        for (int u = 0; u < XB; ++u) {
             if (p.pro == STREAM_PRO_SILU) {
-                r.x = stream_act<STREAM_PRO_SILU, true>(g.x, u.x);
-                r.y = stream_act<STREAM_PRO_SILU, true>(g.y, u.y);
+                v[u].x = stream_act<STREAM_PRO_SILU, true>(v[u].x, up[u].x);
+                v[u].y = stream_act<STREAM_PRO_SILU, true>(v[u].y, up[u].y);
             } else {
-                r.x = stream_act<STREAM_PRO_GELU, true>(g.x, u.x);
-                r.y = stream_act<STREAM_PRO_GELU, true>(g.y, u.y);
+                v[u].x = stream_act<STREAM_PRO_GELU, true>(v[u].x, up[u].x);
+                v[u].y = stream_act<STREAM_PRO_GELU, true>(v[u].y, up[u].y);
             }
-            *(float2*)(xs + 2u * i) = r;
         }
-        if (bad) *gave_up = 1u;
-        __syncthreads();
-        return *gave_up == 0u;
-    }
-    float ss = 0.0f;
-    for (uint32_t i = tid; i < half; i += CHAIN_THREADS) {
-        const float2 v = chain_x2(p.X + 2u * i, mail ? mail + 2u * i : nullptr, fc, par, pt, bad);
-        ss = __builtin_fmaf(v.x, v.x, __builtin_fmaf(v.y, v.y, ss));
-        *(float2*)(xs + 2u * i) = v;
-    }
-    if (p.pro == STREAM_PRO_NORM) {
+    } else if (p.pro == STREAM_PRO_NORM) {
+        // the norm's weights travel while the sum of squares is formed
+        float2 nw[XB];
+#pragma unroll
+        for (int u = 0; u < XB; ++u) nw[u] = *(const float2*)(p.norm_w + 2u * min(tid + u * CHAIN_THREADS, half - 1u));
+        float ss = 0.0f;
+#pragma unroll
+        for (int u = 0; u < XB; ++u) ss = __builtin_fmaf(v[u].x, v[u].x, __builtin_fmaf(v[u].y, v[u].y, ss));   // (pairs past the end are zero)
         const float tot = block_sum(ss, red, wave, lane);
         const float rstd = 1.0f / sqrtf(tot / (float)p.K + p.eps);
-        for (uint32_t i = tid; i < half; i += CHAIN_THREADS) {   // each thread rescales what it wrote
-            const float2 v = *(const float2*)(xs + 2u * i), w = *(const float2*)(p.norm_w + 2u * i);
-            float2 r;
-            r.x = v.x * rstd * w.x;
-            r.y = v.y * rstd * w.y;
-            *(float2*)(xs + 2u * i) = r;
+#pragma unroll
+        for (int u = 0; u < XB; ++u) {
+            v[u].x = v[u].x * rstd * nw[u].x;
+            v[u].y = v[u].y * rstd * nw[u].y;
         }
+    }
+#pragma unroll
+    for (int u = 0; u < XB; ++u) {
+        const uint32_t i = tid + u * CHAIN_THREADS;
+        if (i < half) *(float2*)(xs + 2u * i) = v[u];
     }
     if (bad) *gave_up = 1u;
     __syncthreads();
     return *gave_up == 0u;
+}
+
+// (three sizes, so that a short x is not loaded as a long one's worth of repeated pairs)
+__device__ __forceinline__ bool chain_stage_x(const ChainOp& p, const float* mail, uint32_t par, const Patience& pt, float* xs,
+                                              float* red, volatile uint32_t* gave_up, uint32_t wave, uint32_t lane)
+{
+    if (p.K <= 4096u) return chain_stage_x_n<4>(p, mail, par, pt, xs, red, gave_up, wave, lane);
+    if (p.K <= 9216u) return chain_stage_x_n<9>(p, mail, par, pt, xs, red, gave_up, wave, lane);
+    return chain_stage_x_n<18>(p, mail, par, pt, xs, red, gave_up, wave, lane);
 }
 
 // Which rows of an op a wave walks.
@@ -539,6 +573,12 @@ __device__ __forceinline__ void chain_q6(const ChainOp& p, const Geo& g, const C
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// Diagnostics: thread 0 of every workgroup leaves the wall clock at a few points of every op.
+__device__ __forceinline__ void chain_stamp(uint64_t* trace, uint32_t count, uint32_t op, uint32_t point)
+{
+    if (trace && threadIdx.x == 0) trace[((size_t)blockIdx.x * count + op) * CHAIN_TRACE_POINTS + point] = wall_clock64();
+}
+
 // A descriptor out of the launch's LDS copy, as wave-uniform values.
 constexpr uint32_t CHAIN_OP_WORDS = sizeof(ChainOp) / 4u;
 static_assert(sizeof(ChainOp) % 4u == 0, "descriptors are copied word by word");
@@ -569,6 +609,7 @@ __global__ __launch_bounds__(CHAIN_THREADS) void chain_kernel(ChainLaunch a)
     uint8_t* stage = (uint8_t*)(lds_ops + CHAIN_MAX_PER_LAUNCH * CHAIN_OP_WORDS) + wave * CHAIN_WAVE_STAGE;
     const uint32_t wg = blockIdx.x, G = gridDim.x;
 
+    chain_stamp(a.trace, a.count, 0, 3);
     // Everything the launch needs to know, in one round trip: descriptors, parities, the error word.
     {
         const uint32_t* src = (const uint32_t*)(a.ops + a.first);
@@ -608,10 +649,12 @@ __global__ __launch_bounds__(CHAIN_THREADS) void chain_kernel(ChainLaunch a)
         uint32_t lane_i = lane;
         asm volatile("" : "+v"(lane_i));
         c.lane = lane_i;
+        chain_stamp(a.trace, a.count, i, 0);
         if (!chain_stage_x(p, x_here ? p.x_mail : nullptr, x_par, c.pt, xs, red, flags, wave, lane)) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no load may outlive the wave
             return;
         }
+        chain_stamp(a.trace, a.count, i, 1);
         switch (p.mode) {
         case 0: chain_q4<1, false>(p, g, c, bad); break;
         case CHAIN_MODE_P2: chain_q4<2, false>(p, g, c, bad); break;
@@ -622,6 +665,7 @@ __global__ __launch_bounds__(CHAIN_THREADS) void chain_kernel(ChainLaunch a)
         case CHAIN_MODE_Q6 | CHAIN_MODE_SLICED: chain_q6<1, true>(p, g, c, bad); break;
         default: chain_q6<2, true>(p, g, c, bad); break;
         }
+        chain_stamp(a.trace, a.count, i, 2);
         if (i + 1u < a.count) {
             // the next op's first rows start moving before anybody waits for its x
             p = chain_op_at(lds_ops, i + 1u);
@@ -631,6 +675,7 @@ __global__ __launch_bounds__(CHAIN_THREADS) void chain_kernel(ChainLaunch a)
     }
     // (a lane that gave up waiting for a residual has set the error word; the launch still ends normally)
     __syncthreads();
+    chain_stamp(a.trace, a.count, 0, 4);
     if (threadIdx.x == 0)
         flags[1] = __hip_atomic_fetch_add(a.arrivals, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();

@@ -160,6 +160,7 @@ constexpr uint32_t CHAIN_MODE_SLICED = 2u; // the waves of a workgroup share row
 constexpr uint32_t CHAIN_MODE_Q6 = 4u;     // Q6_K (else Q4_K)
 constexpr int CHAIN_WAVES = 8;
 constexpr uint32_t CHAIN_MAX_OPS = 1024;
+constexpr uint32_t CHAIN_TRACE_POINTS = 8;
 constexpr uint32_t CHAIN_MAX_PER_LAUNCH = 64;   // ops one launch walks (their descriptors sit in LDS)
 constexpr size_t CHAIN_MAX_LDS = (size_t)156 << 10;   // dynamic LDS a chain launch may ask for
 constexpr uint32_t CHAIN_ERR_TIMEOUT = 1u; // low byte of the error word; the op index sits above it
@@ -173,6 +174,7 @@ struct ChainLaunch {
     uint32_t hold;               // testing: 1 keeps the ops from filling their mailboxes, so every wait runs out
     uint32_t ahead;              // rows per wave touched into L2 behind the staged first rows of the next op
     uint64_t spin_ticks;         // bound of a wait, in ticks of the 100 MHz wall clock
+    uint64_t* trace;             // diagnostics: [workgroup][op][CHAIN_TRACE_POINTS] wall-clock stamps, or nullptr
 };
 // CHAIN_MODE_* bits for a matrix, or -1 where the chain kernel has no form for it.
 int chain_mode_for(int type, uint32_t n_blocks, int epi);

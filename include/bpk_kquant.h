@@ -309,6 +309,13 @@ BPK_API int bpk_chain_run(bpk_chain *c, uint32_t first, uint32_t count,
 BPK_API int bpk_chain_status(bpk_chain *c);
 BPK_API int bpk_chain_reset(bpk_chain *c);
 BPK_API int bpk_chain_destroy(bpk_chain *c);
+/* Diagnostics: the next bpk_chain_run calls on this thread make every workgroup
+ * leave wall-clock stamps (100 MHz ticks) in `stamps`, device memory for
+ * [workgroups (one per compute unit)][ops of the launch][8] uint64: [0] the op
+ * begins, [1] its x is staged, [2] its rows are done; for the launch's first op
+ * also [3] the workgroup starts and [4] it has finished its last op.  NULL
+ * switches it off. */
+BPK_API int bpk_chain_trace(void *stamps);
 
 /* ---- greedy sampling tail: replaces argmax + argmax_reduce -----------------
  * The two dispatches after the lm_head matvec (kernels argmax.wgsl /

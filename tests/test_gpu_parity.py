@@ -299,6 +299,33 @@ def test_gemv_stream_shapes(gpu, kqo, type_, N, K, depth, rows_per_wave, M):
                      label=f"stream {type_} {N}x{K} d{depth} r{rows_per_wave}")
 
 
+@pytest.mark.parametrize("N,K", [(1000, 4096), (70, 3072), (16500, 2304), (9, 4096)])
+def test_gemv_stream_eight_wave_form(gpu, kqo, N, K):
+    """The lanes-along-K kernel as eight waves per workgroup, two rows in flight each (what matrices of
+    16384 rows and more get by default), forced on small and ragged shapes; with a y offset and bias."""
+    import torch
+    from backpack_amd import capi, kquant
+    raw, packed, w = gpu.make_weight(Q4_K, N, K, seed=N + 1)
+    rng = np.random.default_rng(N)
+    X = rng.standard_normal((1, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    out = torch.full((1, N + 5), 4.5, device="cuda")
+    capi.set_option("gemv_waves", 8)
+    capi.force_kernel(5)
+    try:
+        _say("stream eight waves", N, K)
+        xd, bd = gpu.dev(X), gpu.dev(bias)
+        capi.check(capi.lib().bpk_kq_matmul(Q4_K, xd.data_ptr(), w.data.data_ptr(), bd.data_ptr(), out.data_ptr(), 1, N, K,
+                                            w.n_blocks, w.row_stride_words, 5, None))
+        assert capi.last_kernel() == "gemv_stream"
+    finally:
+        capi.force_kernel(0)
+        capi.set_option("gemv_waves", 0)
+    got = out.cpu().numpy()
+    assert np.all(got[:, :5] == 4.5)
+    gpu.check_matmul(kqo, Q4_K, got[:, 5:], X, packed, N, K, bias=bias, label=f"stream 8 waves {N}x{K}")
+
+
 @pytest.mark.parametrize("type_,M,N,K", [(Q6_K, 5, 4096, 14336), (Q4_K, 16, 6144, 4096)])
 def test_tile_kernel_k_split_repeatable_and_counters_rearmed(gpu, type_, M, N, K):
     """Matrices of few rows: K is cut over workgroups and the last one to arrive adds the partial tiles in
