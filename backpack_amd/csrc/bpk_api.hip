@@ -682,6 +682,10 @@ struct bpk_chain {
     uint32_t* d_words = nullptr;       // n_ops parity words, the arrival counter, the error word
     float* d_mail = nullptr;           // the ops' mailboxes, back to back
     size_t mail_floats = 0;
+    // host copies for the check a launch makes of its range of ops
+    std::vector<uintptr_t> span;       // per op: x, output and residual ranges, [lo, hi) each (6 words)
+    std::vector<uint32_t> x_src;
+    std::vector<uint64_t> checked;     // (first << 32 | count) of ranges already found sound
 };
 
 namespace {
@@ -769,21 +773,6 @@ int bpk_chain_create(const bpk_chain_op* ops, uint32_t n_ops, bpk_chain** out)
                 break;
             }
         }
-        // What this op overwrites must not be in use by an earlier op that may still be running somewhere.
-        // An op starts once the whole mailbox of the op that writes its X is filled, which every reader and
-        // writer of that op's buffers precedes; so the ops ordered before op i are the chain of its X's
-        // producers, and only those may share a buffer with its output.
-        for (uint32_t k = 0; k < i; ++k) {
-            if (!(out_span[i].overlaps(x_span[k]) || out_span[i].overlaps(out_span[k]) ||
-                  (r_span[k].hi && out_span[i].overlaps(r_span[k]))))
-                continue;
-            bool ordered = false;
-            for (uint32_t j = d.x_src; j != kq::CHAIN_NO_SRC && j >= k; j = h[j].x_src)
-                if (j == k) { ordered = true; break; }
-            if (!ordered)
-                return fail(BPK_ERR_SHAPE, "op %u writes a buffer that op %u reads or writes, and nothing orders the two "
-                            "(an op follows the ops that lead to its X)", i, k);
-        }
     }
     if (kq::chain_lds_bytes(max_k) > kq::CHAIN_MAX_LDS) return fail(BPK_ERR_SHAPE, "K=%u exceeds what a workgroup can stage", max_k);
     bpk_chain* c = new (std::nothrow) bpk_chain;
@@ -792,6 +781,13 @@ int bpk_chain_create(const bpk_chain_op* ops, uint32_t n_ops, bpk_chain** out)
     c->n_ops = n_ops;
     c->max_k = max_k;
     c->mail_floats = mail_floats;
+    c->span.resize((size_t)n_ops * 6u);
+    c->x_src.resize(n_ops);
+    for (uint32_t i = 0; i < n_ops; ++i) {
+        uintptr_t* w = &c->span[(size_t)i * 6u];
+        w[0] = x_span[i].lo; w[1] = x_span[i].hi; w[2] = out_span[i].lo; w[3] = out_span[i].hi; w[4] = r_span[i].lo; w[5] = r_span[i].hi;
+        c->x_src[i] = h[i].x_src;
+    }
     hipError_t e = hipMalloc((void**)&c->d_ops, n_ops * sizeof(kq::ChainOp));
     if (e == hipSuccess) e = hipMalloc((void**)&c->d_words, (n_ops + 2u) * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMalloc((void**)&c->d_mail, mail_floats * sizeof(float));
@@ -825,6 +821,30 @@ int bpk_chain_run(bpk_chain* c, uint32_t first, uint32_t count, void* stream)
     int dev = -1;
     (void)hipGetDevice(&dev);
     if (dev != c->device) return fail(BPK_ERR_DEVICE, "the chain was created on device %d, current is %d", c->device, dev);
+    // What an op overwrites must not be in use by an earlier op of the same launch that may still be running
+    // somewhere.  An op starts once the whole mailbox of the op that writes its X is filled, which every
+    // reader and writer of that op's buffers precedes; so the ops ordered before op i are the chain of its
+    // X's producers inside the launch, and only those may share a buffer with its output.
+    const uint64_t key = ((uint64_t)first << 32) | count;
+    bool known = false;
+    for (uint64_t k : c->checked) known = known || k == key;
+    if (!known) {
+        auto overlap = [](const uintptr_t* a, const uintptr_t* b) { return a[0] < b[1] && b[0] < a[1]; };
+        for (uint32_t i = first + 1u; i < first + count; ++i) {
+            const uintptr_t* wi = &c->span[(size_t)i * 6u];
+            for (uint32_t k = first; k < i; ++k) {
+                const uintptr_t* wk = &c->span[(size_t)k * 6u];
+                if (!(overlap(wi + 2, wk) || overlap(wi + 2, wk + 2) || (wk[5] && overlap(wi + 2, wk + 4)))) continue;
+                bool ordered = false;
+                for (uint32_t j = c->x_src[i]; j != kq::CHAIN_NO_SRC && j >= k && j >= first; j = c->x_src[j])
+                    if (j == k) { ordered = true; break; }
+                if (!ordered)
+                    return fail(BPK_ERR_SHAPE, "op %u writes a buffer that op %u of the same launch reads or writes, and nothing "
+                                "orders the two (an op follows the ops that lead to its X): launch them separately", i, k);
+            }
+        }
+        if (c->checked.size() < 4096u) c->checked.push_back(key);
+    }
     kq::ChainLaunch a{};
     a.ops = c->d_ops;
     a.parity = c->d_words;

@@ -29,31 +29,34 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+COPY_RATE_GBS = 6350.0          # what a plain streaming read reaches on this pool's MI355X (6.0-6.7 TB/s measured)
 METRIC = "Q4_K M=1 matvec HBM GB/s (% of peak); M=2048 dequant-GEMM TFLOPS (% MFMA)"
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE (profiles/decode_gemv_hbm_traffic_pmc.txt): FETCH_SIZE 32386.8
-# x 2.000 KiB + WRITE_SIZE 224.0 x 1.000 KiB, the factors being what the same
-# counters read for a 256 MiB copy kernel.
+# HBM bytes per launch of the dominant kernel.  NOT measured in this run: copied from the rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE summary named below (FETCH_SIZE x 2.000 KiB + WRITE_SIZE x 1.000 KiB, the factors
+# being what the same counters read for a 256 MiB copy kernel); regenerate that file when the kernel changes.
+TRAFFIC_PROFILE = "profiles/decode_gemv_hbm_traffic_pmc.txt"
 MEASURED_TRAFFIC_BYTES = 66557583
 
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--layers", type=int, default=32, help="layers in the set (32 = the named workload)")
     ap.add_argument("--prefill", action="store_true",
                     help="(kept for old command lines: the M=2048 / M=512 prefill GEMM leg now runs by default)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM leg")
-    ap.add_argument("--verify", action="store_true",
-                    help="also time the layer set at M = 2, 4, 8, 16 (speculative-decode verify batches)")
-    ap.add_argument("--moe", action="store_true",
-                    help="also time the Qwen3-30B-A3B-shaped routed-expert FFN at T = 1 and T = 256")
-    ap.add_argument("--all", action="store_true", help="--prefill --verify --moe")
+    ap.add_argument("--verify", action="store_true", help="(kept for old command lines: the verify leg runs by default)")
+    ap.add_argument("--moe", action="store_true", help="(kept for old command lines: the MoE leg runs by default)")
+    ap.add_argument("--no-verify", action="store_true",
+                    help="skip the layer set at M = 2, 4, 8, 16 (speculative-decode verify batches)")
+    ap.add_argument("--no-moe", action="store_true",
+                    help="skip the Qwen3-30B-A3B-shaped routed-expert FFN at T = 1 and T = 256")
+    ap.add_argument("--all", action="store_true", help="also the single-matvec leg (config 0), --fused")
     ap.add_argument("--fused", action="store_true",
                     help="also time the layer set with RMSNorm folded into qkv and act*mul + residual into down")
     ap.add_argument("--load", action="store_true",
@@ -104,8 +107,9 @@ def algorithmic_bytes(mats, M=1):
     return wb, act
 
 
-def run_region(mats, steps, warmup, use_graph):
-    """Times `steps` passes over mats with HIP events on the current stream."""
+def run_region(mats, steps, warmup, use_graph, per_step=None):
+    """Times `steps` passes over mats with HIP events on the launch stream.  per_step: a list that receives
+    the duration of every pass of a second, separately timed round of `steps` passes (an event pair each)."""
     import torch
     from backpack_amd import kquant
 
@@ -138,6 +142,14 @@ def run_region(mats, steps, warmup, use_graph):
         stream.synchronize()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
+        if per_step is not None:
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+            evs[0].record(stream)
+            for i in range(steps):
+                step()
+                evs[i + 1].record(stream)
+            stream.synchronize()
+            per_step.extend(evs[i].elapsed_time(evs[i + 1]) * 1e-3 for i in range(steps))
     return e0.elapsed_time(e1) * 1e-3, wall
 
 
@@ -157,7 +169,23 @@ def cpu_baseline():
     sample = list(spec["layer"]) * n_layers + [spec["lm_head"]]
     rng = np.random.default_rng(0)
     total_bytes, t_deq, t_dot = 0, 0.0, 0.0
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    # every core this job may use: the scheduler affinity, cut down to the control group's CPU quota where
+    # one is set (threads beyond it would only take turns); the host's own count is reported beside it
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count() or 1
+    quota = None
+    try:
+        with open("/sys/fs/cgroup/cpu.max") as f:
+            q, period = f.read().split()[:2]
+            if q != "max":
+                quota = max(1, int(int(q) / int(period)))
+    except (OSError, ValueError):
+        pass
+    if quota:
+        cores = min(cores, quota)
+    cores = max(1, min(cores, 256))
     t_par = 0.0
     for i, (name, type_, N, K) in enumerate(sample):
         # the CPU leg only needs bytes of the right shape: uniform random
@@ -189,7 +217,9 @@ def cpu_baseline():
         "sample": f"{n_layers} of the 32 layers (qkv, o, gate_up, down) + lm_head of the same workload, "
                   f"{total_bytes} weight bytes; dequant {t_deq:.2f} s + dot {t_dot:.2f} s",
         "dequant_s": round(t_deq, 3), "dot_s": round(t_dot, 3),
-        "all_cores": {"value": round(total_bytes / t_par / 1e9, 4), "unit": "GB/s", "cores": cores},
+        "all_cores": {"value": round(total_bytes / t_par / 1e9, 4), "unit": "GB/s", "cores": cores,
+                      "nproc": os.cpu_count(), "cgroup_cpu_quota": quota,
+                      "note": "threads = the cores this job may use (affinity, cut to the cgroup quota)"},
     }
 
 
@@ -226,30 +256,41 @@ def main():
     wb, act = algorithmic_bytes(mats)
     use_graph = not args.no_graph
 
-    sec, wall = run_region(mats, args.steps, args.warmup, use_graph)
+    step_s = []
+    sec, wall = run_region(mats, args.steps, args.warmup, use_graph, per_step=step_s)
+    step_s.sort()
     ms_per_step = sec / args.steps * 1e3
     gbs = (wb + act) / (sec / args.steps) / 1e9
 
     # dominant kernel: the Q4_K GEMV on gate|up, every layer's own matrix
     dom = [m for m in mats if m[0] == "gate_up"]
-    dsec, _ = run_region(dom, max(args.steps, 10), args.warmup, use_graph)
-    launches = len(dom) * max(args.steps, 10)
+    dom_steps = min(max(args.steps, 10), 50)
+    dom_pass = []
+    dsec, _ = run_region(dom, dom_steps, min(args.warmup, 5), use_graph, per_step=dom_pass)
+    dom_pass.sort()
+    launches = len(dom) * dom_steps
     dom_w = dom[0][1]
     dom_bytes = synth.weight_bytes(dom_w.type, dom_w.N, dom_w.K) + (dom_w.K + dom_w.N) * 4
     dom_gbs = dom_bytes / (dsec / launches) / 1e9
     roofline = {
-        "kernel": f"kq::q4k_stream_kernel<2, 4, 4, 1, kq::StreamDense, false> ({capi.last_kernel()}; gate|up 28672x4096 Q4_K, M=1)",
+        "kernel": f"kq::q4k_stream_kernel<2, 8, 2, 1, kq::StreamDense, false> ({capi.last_kernel()}; gate|up 28672x4096 Q4_K, M=1)",
         "bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
         "bytes_per_launch": dom_bytes, "us_per_launch": round(dsec / launches * 1e6, 3),
+        # per launch, from passes of 32 launches each timed by an event pair
+        "us_per_launch_min": round(dom_pass[0] / len(dom) * 1e6, 3),
+        "us_per_launch_median": round(dom_pass[len(dom_pass) // 2] / len(dom) * 1e6, 3),
+        "launches_timed": launches,
         "traffic": MEASURED_TRAFFIC_BYTES,
+        "traffic_source": f"not measured in this run: rocprofv3 --pmc summary {TRAFFIC_PROFILE}",
+        "frac_of_measured_copy_rate": round(dom_gbs / COPY_RATE_GBS, 4),
     }
 
     # per-shape breakdown (extra information, same protocol)
     shapes = {}
     for name in ("qkv", "o", "down", "lm_head"):
         sel = [m for m in mats if m[0] == name]
-        reps = max(args.steps, 10) * (8 if name == "lm_head" else 1)
+        reps = 20 * (8 if name == "lm_head" else 1)
         s, _ = run_region(sel, reps, 2, use_graph)
         w = sel[0][1]
         b = synth.weight_bytes(w.type, w.N, w.K) + (w.K + w.N) * 4
@@ -268,6 +309,8 @@ def main():
                    "accumulation": "f32", "launches_per_step": len(mats), "weight_bytes": wb, "activation_bytes": act,
                    "graph_replay": use_graph},
         "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 2),
+        "pct_of_measured_copy_rate": round(gbs / COPY_RATE_GBS * 100, 2),
+        "ms_per_step_min": round(step_s[0] * 1e3, 4), "ms_per_step_median": round(step_s[len(step_s) // 2] * 1e3, 4),
         "tokens_per_s_equiv": round(args.steps / sec, 1),
         "host_wall_ms_per_step": round(wall / args.steps * 1e3, 4),
         "roofline": roofline,
@@ -275,9 +318,9 @@ def main():
     }
     if args.all:
         out["config0"] = config0_leg()
-    if args.verify or args.all:
+    if not args.no_verify:
         out["verify"] = verify_leg(mats, wb, use_graph)
-    if args.moe or args.all:
+    if not args.no_moe:
         out["moe"] = moe_leg()
     if args.fused or args.all:
         out["fused"] = fused_leg(mats, use_graph)
@@ -359,6 +402,37 @@ def fused_leg(mats, use_graph):
         res["separate_ms"] = round(timed(fused_pass), 4)
     finally:
         capi.set_option("fused_separate", 0)
+    # The same fused function as chains: one launch per stretch between two attention blocks
+    # (o, gate|up, down and the next layer's q|k|v, the last stretch ending in lm_head), 1 + n_layers launches.
+    # Every op reads what the op before it wrote (x += o(attn); act; x += down(act); qkv = W n(x)), handed on
+    # inside the launch.
+    attn = torch.randn(1, hidden, device="cuda") * 0.05
+    xres = torch.randn(1, hidden, device="cuda")
+    x0 = xres.clone()
+    order = [m for m in mats]
+    ch = kquant.Chain()
+    cuts = []
+    for name, w, x, y in order:
+        if name in ("qkv", "lm_head"):
+            ch.add(xres, w, y, prologue=capi.PRO_RMS_NORM, norm_w=norm_w, eps=1e-5)
+            cuts.append(len(ch))            # a launch ends behind every q|k|v (attention follows) and behind lm_head
+        elif name == "o":
+            ch.add(attn, w, xres, residual=xres)
+        elif name == "gate_up":
+            ch.add(xres, w, act, prologue=capi.PRO_RMS_NORM, norm_w=norm_w, eps=1e-5, epilogue=capi.EPI_SILU_MUL)
+        else:
+            ch.add(act, w, xres, residual=xres)
+    ch.build()
+
+    def chain_pass():
+        xres.copy_(x0)                      # (the residual stream would grow without bound over replays otherwise)
+        a = 0
+        for b in cuts:
+            ch.run(a, b - a)
+            a = b
+    res["chain_ms"] = round(timed(chain_pass), 4)
+    ch.status()
+    res["chain_launches"] = len(cuts)
     # the greedy pick behind lm_head: one launch over the 128256 logits, timed in a graph of 50
     logits = next(y for n_, _, _, y in mats if n_ == "lm_head")
     idx = torch.empty(1, dtype=torch.int32, device="cuda")
@@ -578,7 +652,9 @@ def prefill_leg(M=2048):
         del data, w, x, y
     tf = flops_total / sec_total / 1e12
     res["layer_set"] = {"TFLOPs": round(tf, 1), "pct_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS * 100, 2),
-                        "M": M, "ms_extrapolated": round(sec_total * 1e3, 2)}
+                        "M": M, "ms_extrapolated": round(sec_total * 1e3, 2),
+                        "how": "one layer's four matrices x 32 + lm_head, extrapolated: each matrix timed as 20 launches "
+                               "back to back on the same weights (cache-warm; the kernel is bound by the matrix cores)"}
     return res
 
 

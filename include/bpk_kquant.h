@@ -275,10 +275,12 @@ BPK_API int bpk_kq_matmul_fused(int type, const float *X, const void *W,
  * has 2N rows with an epilogue).  Served: Q4_K and Q6_K, K <= 32768, X and norm_w
  * 16-byte aligned, Q4_K rows 16-byte aligned; the act(gate)*up epilogue for Q4_K
  * with K <= 4096.  An input must lie wholly inside one earlier op's outputs or
- * outside all of them, and an op may overwrite a buffer an earlier op uses only
- * if it follows that op through its X (as x += down(...) follows o).
- * bpk_chain_create refuses anything else with BPK_ERR_SHAPE / BPK_ERR_TYPE /
- * BPK_ERR_ALIGN (issue such ops as separate calls).  Pointers are captured at
+ * outside all of them; bpk_chain_create refuses anything else with
+ * BPK_ERR_SHAPE / BPK_ERR_TYPE / BPK_ERR_ALIGN (issue such ops as separate
+ * calls).  Inside one launch an op may overwrite a buffer an earlier op of that
+ * launch uses only if it follows that op through its X (as x += down(...)
+ * follows o); bpk_chain_run refuses a range where that is not so with
+ * BPK_ERR_SHAPE (cut the launch there).  Pointers are captured at
  * creation, like the reference's bind groups; the buffers must stay valid while
  * the chain lives.
  *

@@ -251,10 +251,15 @@ def test_chain_create_refusals(gpu):
     with pytest.raises(capi.BpkError) as e:
         build(((x, w4, y), {}), ((y[:, 32:544], w4, torch.zeros(1, 64, device="cuda")), {}))
     assert e.value.code == -2 and "part of the outputs" in str(e.value)
-    # two ops that write the same buffer with nothing ordering them
+    # two ops that write the same buffer with nothing ordering them: fine as two launches, refused as one
+    ch = build(((x, w4, y), {}), ((x, w6, y), {}))
+    ch.run(0, 1)
+    ch.run(1, 1)
     with pytest.raises(capi.BpkError) as e:
-        build(((x, w4, y), {}), ((x, w6, y), {}))
+        ch.run(0, 2)
     assert e.value.code == -2 and "orders" in str(e.value)
+    torch.cuda.synchronize()
+    ch.status()
     # misaligned x
     xx = torch.zeros(1, 516, device="cuda")
     with pytest.raises(capi.BpkError) as e:
