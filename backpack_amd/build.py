@@ -26,17 +26,93 @@ FLAGS = [
 
 # A source that carries this marker issues global loads from inline asm and waits
 # for them by hand; that is only sound while the loaded registers stay where they
-# are, so such a file must compile without any register spill or scratch use.
+# are, so such a file must compile without any register spill or scratch use, and
+# its generated code is read: see check_ring_registers.
 NO_SPILL_MARKER = "KQ_REQUIRES_NO_SPILL"
+
+# The compiler the hand-waited kernels were validated with on the GPU (first line of `hipcc --version`, up to
+# the build number).  Another compiler may place registers differently; the checks below still run, but the
+# GPU parity tests (tests/test_gpu_parity.py::test_matmul_vs_oracle and test_gemv_stream_shapes, which between
+# them reach every instantiation of the lanes-along-K kernels) have not been run against its code.
+VALIDATED_HIPCC = "HIP version: 7.2.26015"
+
+
+def hipcc_version() -> str:
+    try:
+        r = subprocess.run([HIPCC, "--version"], capture_output=True, text=True)
+        return r.stdout.splitlines()[0].strip() if r.stdout else ""
+    except OSError:
+        return ""
+
+
+def check_compiler() -> None:
+    """Refuses a compiler other than the validated one unless BPK_ALLOW_UNVALIDATED_HIPCC=1 (then it warns);
+    BPK_TRACKED_LOADS=1 builds the hand-waited kernels with ordinary compiler-tracked loads instead."""
+    v = hipcc_version()
+    if v.startswith(VALIDATED_HIPCC) or os.environ.get("BPK_TRACKED_LOADS") == "1":
+        return
+    msg = (f"hipcc reports '{v}', the hand-waited decode kernels were validated with '{VALIDATED_HIPCC}*'. "
+           "Run the GPU parity tests after building; set BPK_ALLOW_UNVALIDATED_HIPCC=1 to build anyway, or "
+           "BPK_TRACKED_LOADS=1 to build those kernels with compiler-tracked loads (slower, no such dependence).")
+    if os.environ.get("BPK_ALLOW_UNVALIDATED_HIPCC") == "1":
+        sys.stderr.write("warning: " + msg + "\n")
+    else:
+        raise RuntimeError(msg)
+
+
+_REG = re.compile(r"v\[(\d+):(\d+)\]|v(\d+)")
+
+
+def _regs(text: str) -> set[int]:
+    out: set[int] = set()
+    for a, b, c in _REG.findall(text):
+        if c:
+            out.add(int(c))
+        else:
+            out.update(range(int(a), int(b) + 1))
+    return out
+
+
+def check_ring_registers(asm_path: str) -> list[str]:
+    """In every function of the generated code, the vector registers written by the marked ring loads must be
+    exactly those the marked ring waits pass through: a register that was copied between its load and its
+    wait (a split live range, a copy on a back edge) leaves a load whose register no wait names, or a wait
+    on a register no load writes."""
+    problems = []
+    func, loads, waits = None, set(), set()
+
+    def close():
+        if func and (loads or waits) and loads != waits:
+            problems.append(f"{func}: ring loads write v{sorted(loads - waits)} that no ring wait covers, "
+                            f"ring waits name v{sorted(waits - loads)} that no ring load writes")
+    with open(asm_path) as f:
+        for line in f:
+            m = re.match(r"^([A-Za-z_][\w.$]*):\s*(;.*)?$", line)
+            if m and not m.group(1).startswith(".L"):
+                close()
+                func, loads, waits = m.group(1), set(), set()
+                continue
+            if "; ringld" in line:
+                # global_load_dwordx4 v[a:b], v[c:d], off ; ringld  -> the first operand is the destination
+                dest = line.split(",")[0]
+                loads |= _regs(dest.split(None, 1)[1] if len(dest.split(None, 1)) > 1 else "")
+            elif "; ringwait" in line:
+                waits |= _regs(line.split("; ringwait", 1)[1])
+    close()
+    return problems
 
 
 def _compile(src: str) -> str:
-    obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", ".o"))
+    base = os.path.basename(src).replace(".hip", "")
+    obj = os.path.join(OBJ, base + ".o")
     extra = os.environ.get("BPK_EXTRA_FLAGS", "").split()   # experiments only
     with open(src) as f:
         guarded = NO_SPILL_MARKER in f.read()
+    tracked = os.environ.get("BPK_TRACKED_LOADS") == "1"
     if guarded:
         extra.append("-Rpass-analysis=kernel-resource-usage")
+        if tracked:
+            extra.append("-DKQ_TRACKED_LOADS")
     cmd = [HIPCC, *FLAGS, *extra, "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     lines = r.stderr.splitlines()
@@ -44,7 +120,7 @@ def _compile(src: str) -> str:
         # (scalar registers spilled into lanes of a reserved vector register are harmless here: no register
         # with a load in flight moves; vector spills and scratch memory are what must not happen)
         bad = [l for l in lines if re.search(r"(VGPRs Spill|ScratchSize[^:]*):\s*[1-9]", l)]
-        if bad and r.returncode == 0:
+        if bad and r.returncode == 0 and not tracked:
             raise RuntimeError(f"{src} must not spill registers (hand-waited loads):\n" + "\n".join(bad[:8]))
         lines = [l for l in lines if "kernel-resource-usage" not in l and not re.match(r"^\s*\d*\s*\|", l)]
     err = "\n".join(l for l in lines if "packed-fp32-ops" not in l)
@@ -52,11 +128,23 @@ def _compile(src: str) -> str:
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
     if err.strip():
         sys.stderr.write(err + "\n")
+    if guarded and not tracked:
+        # the device code as text, for the register check
+        asm = os.path.join(OBJ, base + ".s")
+        ra = subprocess.run([HIPCC, *FLAGS, *[e for e in extra if not e.startswith("-Rpass")], "-S", "--cuda-device-only",
+                             src, "-o", asm], capture_output=True, text=True)
+        if ra.returncode:
+            raise RuntimeError(f"hipcc -S failed on {src}:\n{ra.stderr}")
+        problems = check_ring_registers(asm)
+        if problems:
+            raise RuntimeError(f"{src}: registers of hand-waited loads were moved between load and wait:\n" +
+                               "\n".join(problems[:8]))
     return obj
 
 
 def build_library(jobs: int = 8) -> str:
     os.makedirs(OBJ, exist_ok=True)
+    check_compiler()
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(_compile, srcs))

@@ -16,6 +16,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <new>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -159,7 +160,7 @@ bool read_value(Cursor& c, uint32_t t, MetaValue& v, int depth)
     v.len = c.get<uint64_t>();
     if (!c.ok) return false;
     if (v.elem_type == META_STRING) {
-        if (v.len > c.size) return false;   // each string costs at least its 8-byte length
+        if (v.len > (c.size - c.pos) / 8u) return false;   // each string costs at least its 8-byte length
         v.strs.reserve((size_t)v.len);
         for (uint64_t i = 0; i < v.len; ++i) {
             const char* s; uint64_t n;
@@ -219,10 +220,24 @@ void fill_info(const bpk_gguf* g, const Tensor& t, bpk_gguf_tensor* out)
 
 extern "C" {
 
+static int gguf_open_body(const char* path, bpk_gguf** out);
+
+// (no exception crosses the C boundary: a file that makes the parser run out of memory is a bad file)
 int bpk_gguf_open(const char* path, bpk_gguf** out)
 {
     if (!path || !out) return fail(BPK_ERR_NULL, "path and out must be non-null");
     *out = nullptr;
+    try {
+        return gguf_open_body(path, out);
+    } catch (const std::bad_alloc&) {
+        return fail(BPK_ERR_FORMAT, "%s: metadata too large to hold in memory", path);
+    } catch (...) {
+        return fail(BPK_ERR_IO, "%s: unexpected failure while reading", path);
+    }
+}
+
+static int gguf_open_body(const char* path, bpk_gguf** out)
+{
     const int fd = open(path, O_RDONLY | O_CLOEXEC);
     if (fd < 0) return fail(BPK_ERR_IO, "cannot open %s", path);
     struct stat st;
@@ -233,11 +248,18 @@ int bpk_gguf_open(const char* path, bpk_gguf** out)
     bpk_gguf* g = new bpk_gguf;
     g->map = (const uint8_t*)m;
     g->size = (uint64_t)st.st_size;
-    auto bail = [&](int code, const char* what) {
-        munmap((void*)g->map, (size_t)g->size);
-        delete g;
-        return fail(code, "%s: %s", path, what);
-    };
+    // whatever way this function is left other than by success (an error return, an exception from a
+    // container), the mapping and the object go with it
+    struct Guard {
+        bpk_gguf* g;
+        ~Guard()
+        {
+            if (!g) return;
+            munmap((void*)g->map, (size_t)g->size);
+            delete g;
+        }
+    } guard{g};
+    auto bail = [&](int code, const char* what) { return fail(code, "%s: %s", path, what); };
     Cursor c{g->map, g->size};
     if (c.get<uint32_t>() != 0x46554747u) return bail(BPK_ERR_FORMAT, "not a GGUF file (magic)");
     g->version = c.get<uint32_t>();
@@ -275,7 +297,10 @@ int bpk_gguf_open(const char* path, bpk_gguf** out)
     for (Tensor& t : g->tensors) {
         uint32_t be, bb;
         type_block(t.type, be, bb);
-        if (be == 0) continue;   // size unknown: the caller gets the pointer only
+        if (be == 0) {           // size unknown here: the caller gets the pointer only, and it lies inside the file
+            if (t.offset > g->size - g->data_offset) return bail(BPK_ERR_FORMAT, "tensor data lies outside the file");
+            continue;
+        }
         uint64_t n = 1;
         for (uint32_t d = 0; d < t.n_dims; ++d) {
             if (t.dims[d] != 0 && n > UINT64_MAX / t.dims[d]) return bail(BPK_ERR_FORMAT, "tensor element count overflows");
@@ -286,6 +311,7 @@ int bpk_gguf_open(const char* path, bpk_gguf** out)
         if (t.offset > g->size - g->data_offset || t.bytes > g->size - g->data_offset - t.offset)
             return bail(BPK_ERR_FORMAT, "tensor data lies outside the file");
     }
+    guard.g = nullptr;
     *out = g;
     return BPK_OK;
 }
@@ -345,7 +371,9 @@ int bpk_gguf_get_u32(const bpk_gguf* g, const char* key, uint32_t def, uint32_t*
         case META_UINT8: case META_UINT16: case META_UINT32: case META_UINT64: *out = (uint32_t)v->u; break;
         case META_INT8: case META_INT16: case META_INT32: case META_INT64: *out = (uint32_t)v->i; break;
         case META_ARRAY:
-            if ((v->elem_type == META_INT32 || v->elem_type == META_UINT32) && v->len) {
+            // (the reference keeps both kinds as int32 and compares them so; elements of a uint32 array are
+            // compared as what they are, which differs only from 2^31 on)
+            if (v->elem_type == META_INT32 && v->len) {
                 int32_t m;
                 memcpy(&m, v->arr, 4);
                 for (uint64_t i = 1; i < v->len; ++i) {
@@ -354,6 +382,15 @@ int bpk_gguf_get_u32(const bpk_gguf* g, const char* key, uint32_t def, uint32_t*
                     if (x > m) m = x;
                 }
                 *out = (uint32_t)m;
+            } else if (v->elem_type == META_UINT32 && v->len) {
+                uint32_t m;
+                memcpy(&m, v->arr, 4);
+                for (uint64_t i = 1; i < v->len; ++i) {
+                    uint32_t x;
+                    memcpy(&x, v->arr + 4 * i, 4);
+                    if (x > m) m = x;
+                }
+                *out = m;
             }
             break;
         default: break;
@@ -439,7 +476,20 @@ int bpk_gguf_array_string(const bpk_gguf* g, const char* key, uint64_t index, ch
 
 // Named Q4_K / Q5_K / Q6_K matrices (GGUF shape {K, N}) -> one device weight, rows stacked in the order given
 // (q|k|v, gate|up).  All parts must share the type and K.
+static int gguf_weight_create_body(const bpk_gguf* g, const char* const* names, uint32_t n_names, bpk_weight** out);
+
 int bpk_gguf_weight_create(const bpk_gguf* g, const char* const* names, uint32_t n_names, bpk_weight** out)
+{
+    try {
+        return gguf_weight_create_body(g, names, n_names, out);
+    } catch (const std::bad_alloc&) {
+        return fail(BPK_ERR_IO, "out of host memory while creating a weight");
+    } catch (...) {
+        return fail(BPK_ERR_IO, "unexpected failure while creating a weight");
+    }
+}
+
+static int gguf_weight_create_body(const bpk_gguf* g, const char* const* names, uint32_t n_names, bpk_weight** out)
 {
     if (!g || !names || !out) return fail(BPK_ERR_NULL, "null argument");
     if (n_names == 0 || n_names > 64) return fail(BPK_ERR_SHAPE, "1..64 tensors per weight");

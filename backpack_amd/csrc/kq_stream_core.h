@@ -76,19 +76,40 @@ __device__ __forceinline__ float wave_sum(float v)
 // be overwritten by the late data.
 typedef uint32_t s_u32x2 __attribute__((ext_vector_type(2)));
 
+// Every such load and wait carries a marker in its assembly text (a comment that names the registers), and
+// the build reads the generated code: in each kernel the registers the marked loads write must be exactly
+// the registers the marked waits pass through.  A register copied between its load and its wait (a split
+// live range, a copy on a loop's back edge) would show up as a load whose register no wait names.
+// With KQ_TRACKED_LOADS defined the same kernels are built with ordinary loads that the compiler waits for
+// itself (slower: it drains the queue at every refill): the fallback for a compiler the check rejects.
+typedef uint32_t s_u32x4_u __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint32_t s_u32x2_u __attribute__((ext_vector_type(2), aligned(2)));
+
 __device__ __forceinline__ void ring_load16(s_u32x4& v, const uint8_t* ptr)
 {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(v) : "v"(ptr));
+#ifdef KQ_TRACKED_LOADS
+    v = *(const s_u32x4_u*)ptr;
+#else
+    asm volatile("global_load_dwordx4 %0, %1, off ; ringld" : "+v"(v) : "v"(ptr));
+#endif
 }
 
 __device__ __forceinline__ void ring_load8(s_u32x2& v, const uint8_t* ptr)
 {
-    asm volatile("global_load_dwordx2 %0, %1, off" : "+v"(v) : "v"(ptr));
+#ifdef KQ_TRACKED_LOADS
+    v = *(const s_u32x2_u*)ptr;
+#else
+    asm volatile("global_load_dwordx2 %0, %1, off ; ringld" : "+v"(v) : "v"(ptr));
+#endif
 }
 
 __device__ __forceinline__ void ring_load2(uint32_t& v, const uint8_t* ptr)
 {
-    asm volatile("global_load_ushort %0, %1, off" : "+v"(v) : "v"(ptr));
+#ifdef KQ_TRACKED_LOADS
+    v = *(const uint16_t*)ptr;
+#else
+    asm volatile("global_load_ushort %0, %1, off ; ringld" : "+v"(v) : "v"(ptr));
+#endif
 }
 
 // One lane's share of one pass of a Q4_K row, for MT tokens (the unpack is shared).
@@ -178,15 +199,15 @@ struct Q4Slot {
     __device__ __forceinline__ void wait()
     {
         if constexpr (Q5 && P == 1)
-            asm volatile("s_waitcnt vmcnt(%3)" : "+v"(hdr[0]), "+v"(q[0]), "+v"(qh[0]) : "n"(N));
+            asm volatile("s_waitcnt vmcnt(%3) ; ringwait %0 %1 %2" : "+v"(hdr[0]), "+v"(q[0]), "+v"(qh[0]) : "n"(N));
         else if constexpr (Q5)
-            asm volatile("s_waitcnt vmcnt(%6)"
+            asm volatile("s_waitcnt vmcnt(%6) ; ringwait %0 %1 %2 %3 %4 %5"
                          : "+v"(hdr[0]), "+v"(q[0]), "+v"(qh[0]), "+v"(hdr[1]), "+v"(q[1]), "+v"(qh[1])
                          : "n"(N));
         else if constexpr (P == 1)
-            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(hdr[0]), "+v"(q[0]) : "n"(N));
+            asm volatile("s_waitcnt vmcnt(%2) ; ringwait %0 %1" : "+v"(hdr[0]), "+v"(q[0]) : "n"(N));
         else
-            asm volatile("s_waitcnt vmcnt(%4)" : "+v"(hdr[0]), "+v"(q[0]), "+v"(hdr[1]), "+v"(q[1]) : "n"(N));
+            asm volatile("s_waitcnt vmcnt(%4) ; ringwait %0 %1 %2 %3" : "+v"(hdr[0]), "+v"(q[0]), "+v"(hdr[1]), "+v"(q[1]) : "n"(N));
     }
 };
 
@@ -215,11 +236,11 @@ struct Q6Slot {
     __device__ __forceinline__ void wait()
     {
         if constexpr (P == 1)
-            asm volatile("s_waitcnt vmcnt(%5)"
+            asm volatile("s_waitcnt vmcnt(%5) ; ringwait %0 %1 %2 %3 %4"
                          : "+v"(v[0].a), "+v"(v[0].b), "+v"(v[0].h), "+v"(v[0].sc), "+v"(v[0].d)
                          : "n"(N));
         else
-            asm volatile("s_waitcnt vmcnt(%10)"
+            asm volatile("s_waitcnt vmcnt(%10) ; ringwait %0 %1 %2 %3 %4 %5 %6 %7 %8 %9"
                          : "+v"(v[0].a), "+v"(v[0].b), "+v"(v[0].h), "+v"(v[0].sc), "+v"(v[0].d), "+v"(v[1].a),
                            "+v"(v[1].b), "+v"(v[1].h), "+v"(v[1].sc), "+v"(v[1].d)
                          : "n"(N));

@@ -271,6 +271,54 @@ def test_truncated_and_corrupt_files_are_refused(tmp_path):
     L.bpk_gguf_close(h)
 
 
+def test_hostile_counts_offsets_and_unsigned_arrays(tmp_path):
+    """Files assembled by hand: a string array that claims more strings than the rest of the file could hold
+    (refused before anything is reserved for them), a tensor of a type the reader does not know whose data
+    would start past the end of the file (refused: the pointer handed out always lies inside the mapping),
+    and a uint32 array with an element beyond 2^31 (the largest element, compared as unsigned)."""
+    L = capi.lib()
+    h = C.c_void_p()
+
+    def s(b):
+        return struct.pack("<Q", len(b)) + b
+    path = str(tmp_path / "hostile.gguf")
+    # 1. one key: array of strings, count = one more than eight bytes apiece would allow
+    tail = b"\0" * 4096
+    head = struct.pack("<IIQQ", 0x46554747, 3, 0, 1) + s(b"tok") + struct.pack("<II", 9, 8)
+    count = (len(tail)) // 8 + 1
+    open(path, "wb").write(head + struct.pack("<Q", count) + tail)
+    assert L.bpk_gguf_open(path.encode(), C.byref(h)) == -9 and not h.value
+    open(path, "wb").write(head + struct.pack("<Q", 1 << 40) + tail)
+    assert L.bpk_gguf_open(path.encode(), C.byref(h)) == -9 and not h.value
+    # ... while as many empty strings as do fit are read
+    open(path, "wb").write(head + struct.pack("<Q", 512) + tail)
+    assert L.bpk_gguf_open(path.encode(), C.byref(h)) == 0
+    n, et = C.c_uint64(), C.c_uint32()
+    assert L.bpk_gguf_array_len(h, b"tok", C.byref(n), C.byref(et)) == 0 and (n.value, et.value) == (512, 8)
+    L.bpk_gguf_close(h)
+    # 2. a tensor of an unknown type (IQ2_XXS = 16) at an offset past the end of the file
+    for offset, want in ((0, 0), (64, 0), (1 << 20, -9), (1 << 62, -9)):
+        blob = struct.pack("<IIQQ", 0x46554747, 3, 1, 0) + s(b"odd") + struct.pack("<IQQIQ", 2, 32, 2, 16, offset)
+        blob += b"\0" * ((-len(blob)) % 32) + b"\x11" * 96
+        open(path, "wb").write(blob)
+        h = C.c_void_p()
+        assert L.bpk_gguf_open(path.encode(), C.byref(h)) == want, offset
+        if want == 0:
+            t = capi.GgufTensor()
+            assert L.bpk_gguf_find_tensor(h, b"odd", C.byref(t)) == 0 and t.bytes == 0 and t.offset == offset
+            L.bpk_gguf_close(h)
+    # 3. uint32 elements are compared as unsigned, int32 elements as signed
+    kv = s(b"u") + struct.pack("<IIQ", 9, 4, 3) + struct.pack("<III", 7, 0x90000000, 12)
+    kv += s(b"i") + struct.pack("<IIQ", 9, 5, 3) + struct.pack("<iii", 7, -5, 12)
+    open(path, "wb").write(struct.pack("<IIQQ", 0x46554747, 3, 0, 2) + kv)
+    h = C.c_void_p()
+    assert L.bpk_gguf_open(path.encode(), C.byref(h)) == 0
+    out = C.c_uint32()
+    assert L.bpk_gguf_get_u32(h, b"u", 1, C.byref(out)) == 0 and out.value == 0x90000000
+    assert L.bpk_gguf_get_u32(h, b"i", 1, C.byref(out)) == 0 and out.value == 12
+    L.bpk_gguf_close(h)
+
+
 def test_weight_create_argument_checks(tmp_path):
     """The checks that precede any device call (type, shape, names)."""
     path, *_ = _model_file(tmp_path)
