@@ -149,9 +149,6 @@ int current_state(DeviceState** out)
 }
 
 bool known_type(int type) { return type == BPK_TYPE_Q4_K || type == BPK_TYPE_Q5_K || type == BPK_TYPE_Q6_K; }
-// Q5_K is served by the packers, the row dequantiser, the fp32 matmul and the 128-tile bf16 GEMM; the MoE
-// entry points take the two types their kernels are written for.
-bool fast_type(int type) { return type == BPK_TYPE_Q4_K || type == BPK_TYPE_Q6_K; }
 
 int check_matmul(int type, const void* X, const void* W, const void* Y, uint32_t M, uint32_t N, uint32_t K,
                  uint32_t n_blocks, uint32_t row_stride_words)
@@ -440,30 +437,12 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     // weight load and its unpack).  Measured at M = 4: Q4_K 4096x4096 10.0 against 10.8 us on the tile
     // kernel, 6144x4096 a tie, 28672x4096 34.5 against 23.0; Q6_K 4096x14336 23.6 against 27.1.
     const uint64_t weights = (uint64_t)N * K;
-    // (Q5_K has no tile kernel to fall back on: it takes this path whatever the size)
     const bool stream_four = stream_ok && M >= 3 && M <= 4 && N <= 32768u &&
-                             (type == BPK_TYPE_Q5_K || weights <= (type == BPK_TYPE_Q6_K ? (64ull << 20) : (20ull << 20)));
+                             weights <= (type == BPK_TYPE_Q6_K ? (64ull << 20) : (20ull << 20));
     if (t_family == 6 || (t_family == 0 && mtile_ok && M >= 3 && M <= 255 && !stream_four)) {
         t_kernel = "mtile";
         e = kq::launch_mtile(a, st->split, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
-    }
-    // Q5_K beyond four tokens: groups of four on the lanes-along-K kernel (the tile kernel does not take the
-    // type; re-reading the weights per group is still many times faster than the generic kernel)
-    if (t_family == 0 && type == BPK_TYPE_Q5_K && M > 4u && M <= 64u && N <= 32768u) {
-        kq::MatmulArgs g = a;
-        g.M = 4;
-        if (kq::gemv_stream_supported(g)) {
-            t_kernel = "gemv_stream";
-            for (uint32_t m0 = 0; m0 < M; m0 += 4u) {
-                g.M = M - m0 < 4u ? M - m0 : 4u;
-                g.X = X + (size_t)m0 * K;
-                g.Y = Y + (size_t)m0 * N;
-                e = kq::launch_gemv_stream(g, t_gemv, s);
-                if (e != hipSuccess) return hip_fail(e, t_kernel);
-            }
-            return BPK_OK;
-        }
     }
     if (t_family == 5 && !stream_ok) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");
     if (t_family == 4) return fail(BPK_ERR_SHAPE, "kernel family %d is not available for fp32 X", t_family);
@@ -620,7 +599,6 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
                       uint32_t k, uint32_t n_experts, uint32_t N, uint32_t K, uint32_t n_blocks,
                       uint32_t row_stride_words, int x_per_slot, void* stream)
 {
-    if (type == BPK_TYPE_Q5_K) return fail(BPK_ERR_TYPE, "the MoE entry points take Q4_K and Q6_K");
     if (int rc = check_matmul(type, X, W, Y, T, N, K, n_blocks, row_stride_words)) return rc;
     if (!expert_idx) return fail(BPK_ERR_NULL, "expert_idx must be non-null");
     if (k == 0 || n_experts == 0) return fail(BPK_ERR_SHAPE, "k and n_experts must be positive");
@@ -641,13 +619,15 @@ int bpk_kq_moe_matmul(int type, const float* X, const void* W, const uint32_t* e
     const int sets = kq::moe_sets_for(T * k, n_experts);
     hipError_t e;
     // two or more pairs per expert on average: records of 8 pairs on the 16x16 tile kernel
-    const bool tile_path = (t_family == 0 || t_family == 6) && kq::mtile_supported(a) && N >= 128u &&
-                           (uint64_t)T * k >= 2ull * n_experts && n_experts <= 8192u &&
-                           kq::moe_tiles_bound(T * k, n_experts, 4) <= 65535u &&
-                           kq::moe_tiles_words(T * k, n_experts, 4) <= kMoeWords;
+    const bool dense = (uint64_t)T * k >= 2ull * n_experts;
+    const bool tile_ok = (t_family == 0 || t_family == 6) && kq::mtile_supported(a) && N >= 128u && n_experts <= 8192u &&
+                         kq::moe_tiles_bound(T * k, n_experts, 4) <= 65535u &&
+                         kq::moe_tiles_words(T * k, n_experts, 4) <= kMoeWords;
     // a handful of pairs (decode): one lanes-along-K matvec per pair, no grouping pass
-    const bool stream_path = (t_family == 0 || t_family == 5) && !tile_path && (uint64_t)T * k <= 64u &&
+    const bool stream_path = (t_family == 0 || t_family == 5) && !(tile_ok && dense) && (uint64_t)T * k <= 64u &&
                              kq::gemv_stream_supported(a);
+    // (Q5_K has no matrix-core row kernel: its thinly spread pairs take the tile kernel too)
+    const bool tile_path = tile_ok && !stream_path && (dense || !kq::mrow_supported(a));
     if (stream_path) {
         t_kernel = "stream_grouped";
         e = kq::launch_gemv_stream(a, t_gemv, s);
@@ -999,7 +979,7 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
                    uint32_t n_experts, uint32_t hidden, uint32_t inter, void* scratch, size_t scratch_bytes,
                    void* stream)
 {
-    if (!fast_type(type_gu) || !fast_type(type_dn)) return fail(BPK_ERR_TYPE, "the MoE entry points take Q4_K and Q6_K");
+    if (!known_type(type_gu) || !known_type(type_dn)) return fail(BPK_ERR_TYPE, "unsupported GGUF type (Q4_K=12, Q5_K=13, Q6_K=14)");
     if (!X || !gate || !up || !down || !expert_idx || !expert_wt || !out)
         return fail(BPK_ERR_NULL, "X, gate, up, down, expert_idx, expert_wt and out must be non-null");
     if (k == 0 || n_experts == 0) return fail(BPK_ERR_SHAPE, "k and n_experts must be positive");
@@ -1037,11 +1017,13 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
                       kq::mrow_supported(d);
     hipError_t e = hipSuccess;
     const uint32_t bound8 = kq::moe_tiles_bound(P, n_experts, 4);
-    const bool tile_path = (t_family == 0 || t_family == 6) && n_experts <= 8192u && bound8 <= 65535u &&
-                           (uint64_t)P >= 2ull * n_experts && inter >= 128u && hidden >= 128u &&
-                           kq::mtile_supported(a) && kq::mtile_supported(d);
-    const bool stream_path = (t_family == 0 || t_family == 5) && !tile_path && P <= 64u &&
+    const bool dense = (uint64_t)P >= 2ull * n_experts;
+    const bool tile_ok = (t_family == 0 || t_family == 6) && n_experts <= 8192u && bound8 <= 65535u && inter >= 128u &&
+                         hidden >= 128u && kq::mtile_supported(a) && kq::mtile_supported(d);
+    const bool stream_path = (t_family == 0 || t_family == 5) && !(tile_ok && dense) && P <= 64u &&
                              kq::gemv_stream_supported(a) && kq::gemv_stream_supported(d);
+    // (Q5_K has no matrix-core row kernel: its thinly spread pairs take the tile kernel too)
+    const bool tile_path = tile_ok && !stream_path && (dense || !fast);
     if (stream_path) {
         // a handful of pairs (decode): one lanes-along-K matvec per pair, no grouping pass
         // gate and up in one launch (they read the same x), the activation folded into down's load of x

@@ -237,7 +237,23 @@ __device__ __forceinline__ MtileA mtile_read_a(const uint8_t* xa_b, int sb, uint
 // The minima ride on the matrix cores as well: sum over sub-blocks of mn[row][sb] * xsum[token][sb] is one more
 // product with k = sub-block (8 of the 32 k used): A = the staged sums (xv_b), B = the eight 6-bit minima of
 // the lane's row as subnormals.  B's lanes of k >= 8 hold the same finite values; A is zero there.
-__device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2 (&w)[4], const uint8_t* xa_b,
+// Q5: qhw holds the eight bytes of fifth bits of the lane's eight positions (bit sb of a byte belongs to
+// sub-block sb); the bit joins its nibble in the fp16 mantissa (bit 4 beside a low nibble, bit 8 beside a high
+// one: a five-bit value is still a subnormal), four more bit-ops per operand.
+template <bool Q5>
+__device__ __forceinline__ void q5_join(t_u32x4& blo, t_u32x4& bhi, const t_u32x2 qhw, uint32_t sbit)
+{
+    if constexpr (Q5) {
+        const uint32_t h0 = qhw.x >> sbit, h1 = qhw.y >> sbit;   // bit 0 of each byte: sub-block sbit, bit 1: sbit + 1
+        blo.x |= (h0 << 4) & 0x00100010u; blo.y |= (h0 >> 4) & 0x00100010u;
+        blo.z |= (h1 << 4) & 0x00100010u; blo.w |= (h1 >> 4) & 0x00100010u;
+        bhi.x |= (h0 << 7) & 0x01000100u; bhi.y |= (h0 >> 1) & 0x01000100u;
+        bhi.z |= (h1 << 7) & 0x01000100u; bhi.w |= (h1 >> 1) & 0x01000100u;
+    }
+}
+
+template <bool Q5>
+__device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2 (&w)[4], const t_u32x2 qhw, const uint8_t* xa_b,
                                                 const uint8_t* xv_b, const float* xinv_b, uint32_t lane,
                                                 t_f32x4& tot)
 {
@@ -268,6 +284,7 @@ __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2
             const uint32_t e0 = d0 >> 8, e1 = d1 >> 8;
             blo = t_u32x4{d0 & 0x000F000Fu, e0 & 0x000F000Fu, d1 & 0x000F000Fu, e1 & 0x000F000Fu};
             bhi = t_u32x4{d0 & 0x00F000F0u, e0 & 0x00F000F0u, d1 & 0x00F000F0u, e1 & 0x00F000F0u};
+            q5_join<Q5>(blo, bhi, qhw, (uint32_t)sb);
         }
         const t_half8 bq = __builtin_bit_cast(t_half8, (sb & 1) ? bhi : blo);
         t_f32x4 D = {0, 0, 0, 0};
@@ -297,9 +314,10 @@ __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2
 
 // The same arithmetic with every operand read where it is used: fewer registers (the grouped kernel is held
 // to 128 so that two of its workgroups share a CU).
-__device__ __forceinline__ void q4k_mtile_block_compact(const t_u32x4 hdr, const t_u32x2 (&w)[4], const uint8_t* xa_b,
-                                                const float* xs_b, const float* xinv_b, uint32_t lane,
-                                                t_f32x4& tot)
+template <bool Q5>
+__device__ __forceinline__ void q4k_mtile_block_compact(const t_u32x4 hdr, const t_u32x2 (&w)[4], const t_u32x2 qhw,
+                                                        const uint8_t* xa_b, const float* xs_b, const float* xinv_b, uint32_t lane,
+                                                        t_f32x4& tot)
 {
     const float d = half_bits_to_float(hdr.x & 0xFFFFu);
     const float dmin = half_bits_to_float(hdr.x >> 16);
@@ -313,8 +331,9 @@ __device__ __forceinline__ void q4k_mtile_block_compact(const t_u32x4 hdr, const
     for (int g = 0; g < 4; ++g) {
         const uint32_t d0 = w[g].x, d1 = w[g].y;
         const uint32_t e0 = d0 >> 8, e1 = d1 >> 8;
-        const t_u32x4 blo = {d0 & 0x000F000Fu, e0 & 0x000F000Fu, d1 & 0x000F000Fu, e1 & 0x000F000Fu};
-        const t_u32x4 bhi = {d0 & 0x00F000F0u, e0 & 0x00F000F0u, d1 & 0x00F000F0u, e1 & 0x00F000F0u};
+        t_u32x4 blo = {d0 & 0x000F000Fu, e0 & 0x000F000Fu, d1 & 0x000F000Fu, e1 & 0x000F000Fu};
+        t_u32x4 bhi = {d0 & 0x00F000F0u, e0 & 0x00F000F0u, d1 & 0x00F000F0u, e1 & 0x00F000F0u};
+        q5_join<Q5>(blo, bhi, qhw, 2u * (uint32_t)g);
 #pragma unroll
         for (int hn = 0; hn < 2; ++hn) {
             const int sb = 2 * g + hn;
@@ -466,6 +485,8 @@ struct MtileWStage {
 // (the grouped Q4_K kernel is held to 128 registers so that two of its workgroups share a CU)
 template <int TYPE, int NW, int R, bool STAGED, int TOK>
 __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1) void mtile_kernel(MtileParams p)
+// (Q5_K: the Q4_K code with blocks of 176 bytes — header, 32 bytes of fifth bits, quants — and one more
+// 8-byte piece per lane and superblock)
 {
     static_assert(R == NW || R == 1, "a wave owns a tile, or all waves share one");
     extern __shared__ __align__(16) uint8_t smem[];
@@ -497,13 +518,14 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     const uint32_t row = has_tile ? tile * 16u + (lane & 15u) : p.N;
     const uint32_t kq = lane >> 4;
 
-    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
-    constexpr uint32_t BB = Q6 ? KQ_Q6K_BYTES : KQ_Q4K_BYTES;
+    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K, Q5 = TYPE == KQ_TYPE_Q5_K;
+    constexpr uint32_t BB = Q6 ? KQ_Q6K_BYTES : Q5 ? KQ_Q5K_BYTES : KQ_Q4K_BYTES;
+    constexpr uint32_t QOFF = Q5 ? 48u : 16u;   // where the quants start inside a block
     // A wave with a tile of its own stages two superblocks of its 16 rows at a time (two passes per chunk);
     // waves that share a tile stage the one superblock of the chunk that is theirs.
     constexpr int HB = R == 1 ? 1 : 2;                        // superblocks per staging pass
     constexpr int SPAN = HB * BB;
-    constexpr int PITCH = Q6 ? (HB == 1 ? 240 : 464) : (HB == 1 ? 160 : 304);
+    constexpr int PITCH = Q6 ? (HB == 1 ? 240 : 464) : Q5 ? (HB == 1 ? 176 : 368) : (HB == 1 ? 160 : 304);
     constexpr int PASSES = R == 1 ? 1 : MT_KC / HB;
     using WStage = MtileWStage<SPAN, PITCH>;
     static_assert(PITCH >= WStage::UPR * 16 && PITCH % 16 == 0, "window row holds the staged units");
@@ -580,10 +602,11 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                         q6k_mtile_block(w6, xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
                     } else {
                         const t_u32x4 hdr = *(const t_u32x4*)blk;
-                        t_u32x2 w[4];
+                        t_u32x2 w[4], qhw = {0, 0};
 #pragma unroll
-                        for (int g = 0; g < 4; ++g) w[g] = *(const t_u32x2*)(blk + 16u + 32u * g + 8u * kq);
-                        q4k_mtile_block(hdr, w, xa + (size_t)bb * (8 * 2 * 1024), xv + (size_t)bb * 2048, xinv + bb * 16, lane, tot);
+                        for (int g = 0; g < 4; ++g) w[g] = *(const t_u32x2*)(blk + QOFF + 32u * g + 8u * kq);
+                        if constexpr (Q5) qhw = *(const t_u32x2*)(blk + 16u + 8u * kq);
+                        q4k_mtile_block<Q5>(hdr, w, qhw, xa + (size_t)bb * (8 * 2 * 1024), xv + (size_t)bb * 2048, xinv + bb * 16, lane, tot);
                     }
                 }
             }
@@ -606,7 +629,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     for (uint32_t c0 = c_begin; c0 < c_end; c0 += MT_KC) {
         // the chunk's weights are requested first, so that their latency runs under the conversion of X
         t_u32x4 hdr[BPC];
-        t_u32x2 w[BPC][4];
+        t_u32x2 w[BPC][4], qhw[BPC];
         Q6TileW w6[BPC];
 #pragma unroll
         for (int i = 0; i < BPC; ++i) {
@@ -618,7 +641,9 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
             } else {
                 hdr[i] = *(const t_u32x4*)blk;
 #pragma unroll
-                for (int g = 0; g < 4; ++g) w[i][g] = *(const t_u32x2*)(blk + 16u + 32u * g + 8u * kq);
+                for (int g = 0; g < 4; ++g) w[i][g] = *(const t_u32x2*)(blk + QOFF + 32u * g + 8u * kq);
+                qhw[i] = t_u32x2{0, 0};
+                if constexpr (Q5) qhw[i] = *(const t_u32x2*)(blk + 16u + 8u * kq);
             }
         }
         if (it == 0u) {
@@ -634,7 +659,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                     if constexpr (Q6)
                         q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
                     else
-                        q4k_mtile_block_compact(hdr[i], w[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                        q4k_mtile_block_compact<Q5>(hdr[i], w[i], qhw[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
                 }
             }
         }
@@ -704,7 +729,7 @@ bool mtile_supported(const MatmulArgs& a)
     // meant for the few dozen tokens between a verify batch and a prefill, not for prefill itself
     if (!a.expert_idx && (a.M < 1 || a.M > 255)) return false;   // grouped calls bring their tokens in records
     if (((uintptr_t)a.X & 15u)) return false;
-    if (a.type == KQ_TYPE_Q4_K) return !(((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u));
+    if (a.type == KQ_TYPE_Q4_K || a.type == KQ_TYPE_Q5_K) return !(((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u));
     if (a.type == KQ_TYPE_Q6_K) return !(((uintptr_t)a.W & 1u) || (a.row_stride_bytes & 1u));
     return false;
 }
@@ -712,8 +737,8 @@ bool mtile_supported(const MatmulArgs& a)
 template <int TYPE, int NW, int R, bool STAGED = true, int TOK = 16>
 static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s, uint32_t wgs_z = 1)
 {
-    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
-    constexpr int PITCH = Q6 ? (R == 1 ? 240 : 464) : (R == 1 ? 160 : 304);   // as in the kernel
+    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K, Q5 = TYPE == KQ_TYPE_Q5_K;
+    constexpr int PITCH = Q6 ? (R == 1 ? 240 : 464) : Q5 ? (R == 1 ? 176 : 368) : (R == 1 ? 160 : 304);   // as in the kernel
     constexpr size_t shmem = MT_STAGE_BYTES + (STAGED ? (size_t)NW * 16 * PITCH : 0);
     auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK>;
     static bool raised = false;   // per instantiation
@@ -765,6 +790,7 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
     }
     const uint32_t wgs = (row_tiles + tpw * p.tile_iters - 1u) / (tpw * p.tile_iters);
     if (a.type == KQ_TYPE_Q6_K) return launch_mtile_one<KQ_TYPE_Q6_K, 4, 4, false>(p, wgs, tiles_bound, s, slices);
+    if (a.type == KQ_TYPE_Q5_K) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, false>(p, wgs, tiles_bound, s, slices);
     return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, false>(p, wgs, tiles_bound, s, slices);
 }
 
@@ -816,8 +842,10 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
         p.tiles = nullptr; p.n_tiles = nullptr; p.tile_stride = 0; p.tile_iters = 1; p.k_slots = 1; p.x_per_slot = 0;
         p.n_splits = 1; p.chunks_per_split = n_chunks; p.partial = sc.partial; p.counters = sc.counters;
         hipError_t e;
+        const bool q5 = a.type == KQ_TYPE_Q5_K;
         if (shared_tile) {
-            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 4, 1>(p, tiles, 1, s) : launch_mtile_one<KQ_TYPE_Q4_K, 4, 1>(p, tiles, 1, s);
+            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 4, 1>(p, tiles, 1, s)
+                : q5 ? launch_mtile_one<KQ_TYPE_Q5_K, 4, 1>(p, tiles, 1, s) : launch_mtile_one<KQ_TYPE_Q4_K, 4, 1>(p, tiles, 1, s);
         } else {
             p.tiles_per_wg = best_tpw;
             p.n_splits = best_splits;
@@ -827,10 +855,12 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
             // that all waves take part (measured +2-3 %; with 4 tokens or fewer the wider exchange costs more)
             if (p.M > 4u && p.M <= 8u)
                 e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits)
-                       : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits);
+                    : q5 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits)
+                         : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits);
             else
                 e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits)
-                       : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits);
+                    : q5 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits)
+                         : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits);
         }
         if (e != hipSuccess) return e;
     }

@@ -531,7 +531,6 @@ bool gemv_stream_supported(const MatmulArgs& a)
     if (((uintptr_t)a.X & 15u)) return false;
     if (a.n_blocks < 1) return false;
     if (a.type == KQ_TYPE_Q4_K || a.type == KQ_TYPE_Q5_K) {
-        if (a.type == KQ_TYPE_Q5_K && a.expert_idx) return false;
         // longer rows are cut into K slices: dense and fused calls only, and the two-token kernel for
         // the longest rows has no registers for Q5_K's third load or the fused forms
         if (a.n_blocks > 16 && a.expert_idx) return false;
@@ -562,13 +561,11 @@ static void launch_q6k_one(dim3 grid, hipStream_t s, const PT& p)
     if constexpr (!absent) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, D, MT, PT>), grid, dim3(64 * KW), 0, s, p);
 }
 
-// (Q5_K: no grouped launches, the MoE entry points do not take the type; at most two rows in flight, the
-// third load per pass leaves no registers for four.)
+// (Q5_K: at most two rows in flight, the third load per pass leaves no registers for four.)
 template <int P, int NW, int D, int MT, typename PT, bool Q5>
 static void launch_q4k_one(dim3 grid, hipStream_t s, const PT& p)
 {
-    constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && (D == 1 || (D == 4 && MT == 2))) ||
-                            (Q5 && (PT::kGrouped || D > 2));
+    constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && (D == 1 || (D == 4 && MT == 2))) || (Q5 && D > 2);
     if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT, Q5>), grid, dim3(64 * NW), 0, s, p);
 }
 

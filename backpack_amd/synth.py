@@ -206,8 +206,8 @@ def make_packed_device(type_: int, N: int, K: int, seed: int = 0, device="cuda")
         v = (torch.randn((N, nb, cnt), device=device, generator=g) * SIGMA).abs().to(torch.float16)
         return v.view(torch.uint8).reshape(N, nb, 2 * cnt)
 
-    if type_ == Q4_K:
-        blk[:, :, 0:4] = half_scales(2)          # 12 scale bytes and the quants stay uniform
+    if type_ in (Q4_K, Q5_K):
+        blk[:, :, 0:4] = half_scales(2)          # 12 scale bytes, the quants (and Q5_K's fifth bits) stay uniform
     elif type_ == Q6_K:
         sc = torch.randint(-64, 64, (N, nb, 16), dtype=torch.int8, device=device, generator=g)
         blk[:, :, 192:208] = sc.view(torch.uint8)

@@ -34,8 +34,7 @@ extern "C" {
 
 /* GGUF tensor type codes (runtime/gguf_loader.h:29-30). */
 #define BPK_TYPE_Q4_K 12
-#define BPK_TYPE_Q5_K 13 /* every entry point but the MoE calls, which return
-                            BPK_ERR_TYPE for it */
+#define BPK_TYPE_Q5_K 13
 #define BPK_TYPE_Q6_K 14
 
 enum {

@@ -1,6 +1,7 @@
 """GPU parity at the sizes the benchmark times: the five matrices of the Llama-3-8B layer set at their
 real shapes (q|k|v 6144x4096, o 4096x4096, gate|up 28672x4096 in Q4_K; down 4096x14336 and lm_head
-128256x4096 in Q6_K) with the library's own kernel, tile and work-split choices.
+128256x4096 in Q6_K; q|k|v, gate|up and down again in Q5_K) with the library's own kernel, tile and
+work-split choices.
 
 The HIP path runs on the whole matrix; the CPU oracle (the reference's dequantise-then-dot path,
 runtime/gguf_loader.cpp:455-573 + runtime/tests/kernel_test.cpp:1682) runs on a sample of the output
@@ -16,13 +17,17 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-Q4_K, Q6_K = 12, 14
+Q4_K, Q5_K, Q6_K = 12, 13, 14
 LAYER_SET = {
     "qkv": (Q4_K, 6144, 4096),
     "o": (Q4_K, 4096, 4096),
     "gate_up": (Q4_K, 28672, 4096),
     "down": (Q6_K, 4096, 14336),
     "lm_head": (Q6_K, 128256, 4096),
+    # the same projections as a Q5_K file holds them
+    "qkv_q5": (Q5_K, 6144, 4096),
+    "gate_up_q5": (Q5_K, 28672, 4096),
+    "down_q5": (Q5_K, 4096, 14336),
 }
 SLACK = {"mrow": 1e-5, "mtile": 2e-5}
 

@@ -96,7 +96,7 @@ def test_reference_recipe(gpu, kqo, name, family):
     (Q4_K, 3, 130, 2048), (Q4_K, 4, 300, 4096), (Q4_K, 3, 200, 8192), (Q4_K, 4, 100, 14336), (Q4_K, 4, 4096, 4096),
     (Q4_K, 3, 77, 6400),                       # 25 superblocks: the fourth K slice is partial
     (Q6_K, 4, 33, 768), (Q6_K, 3, 150, 4096), (Q6_K, 4, 120, 8192), (Q6_K, 3, 4096, 14336), (Q6_K, 4, 64, 2048),
-    (Q5_K, 3, 90, 1024), (Q5_K, 4, 300, 4096), (Q5_K, 4, 60, 8192), (Q5_K, 3, 50, 14336), (Q5_K, 4, 28672, 4096),
+    (Q5_K, 3, 90, 1024), (Q5_K, 4, 300, 4096), (Q5_K, 4, 60, 8192), (Q5_K, 3, 50, 14336), (Q5_K, 4, 4096, 4096),
 ])
 def test_four_token_stream_kernels(gpu, kqo, type_, M, N, K):
     """Every K-slice count (1, 2, 4, 7 waves), three tokens run as four with the last masked: the rows of Y
@@ -114,12 +114,12 @@ def test_four_token_stream_kernels(gpu, kqo, type_, M, N, K):
     gpu.check_matmul(kqo, type_, got[:M], X, packed, N, K, bias=bias, label=f"four {type_} {M}x{N}x{K}")
 
 
-# ---- Q5_K: packers, rows and the fp32 matmul (generic kernel) ------------------------
+# ---- Q5_K: the fp32 matmul's automatic choice (lanes-along-K kernel, tile kernel, generic) ---------
 @pytest.mark.parametrize("M,N,K,kernel", [(1, 300, 4096, "gemv_stream"), (2, 64, 768, "gemv_stream"),
                                           (1, 4096, 4096, "gemv_stream"), (2, 6144, 4096, "gemv_stream"),
                                           (1, 77, 256, "gemv_stream"), (1, 500, 3072, "gemv_stream"),
-                                          (5, 130, 2048, "gemv_stream"), (17, 40, 512, "gemv_stream"), (4, 64, 768, "gemv_stream"),
-                                          (13, 700, 4096, "gemv_stream"), (70, 40, 512, "generic"),
+                                          (5, 130, 2048, "mtile"), (17, 40, 512, "mtile"), (4, 64, 768, "gemv_stream"),
+                                          (13, 700, 4096, "mtile"), (70, 40, 512, "mtile"), (300, 40, 512, "generic"),
                                           (1, 1000, 14336, "gemv_stream"), (2, 300, 8192, "gemv_stream"),
                                           (1, 200, 28672, "gemv_stream"), (2, 200, 28672, "generic"),
                                           (1, 50, 32768, "generic")])
@@ -139,16 +139,6 @@ def test_q5k_matmul_vs_oracle(gpu, kqo, M, N, K, kernel):
         finally:
             capi.force_kernel(0)
         gpu.check_matmul(kqo, Q5_K, y1, X, packed, N, K, bias=bias, label=f"q5k generic {M}x{N}x{K}")
-
-
-def test_q5k_is_refused_where_no_kernel_serves_it(gpu):
-    from backpack_amd import capi, kquant
-    raw, packed, w = gpu.make_weight(Q5_K, 64, 512, seed=1)
-    import torch
-    idx = torch.zeros(2, 2, dtype=torch.int32, device="cuda")
-    with pytest.raises(capi.BpkError) as e:
-        kquant.moe_matmul(torch.zeros(2, 512, device="cuda"), w, idx, 4)
-    assert e.value.code == -1
 
 
 # ---- matmul against the oracle ------------------------------------------------------
@@ -199,6 +189,20 @@ SHAPES = [
     (Q4_K, 6, 4100, 5376),      # ... 21 superblocks: runs of unequal length, the last with a partial chunk
     (Q6_K, 5, 4096, 14336),     # ... 7 runs of two chunks
     (Q6_K, 12, 1000, 7168),     # ... two token groups through the same scratch
+    # Q5_K: the lanes-along-K kernel (one pass, two, K slices) and every mode of the tile kernel
+    (Q5_K, 1, 4096, 4096),
+    (Q5_K, 1, 100, 256),
+    (Q5_K, 2, 500, 14336),
+    (Q5_K, 1, 90, 28672),
+    (Q5_K, 3, 130, 2048),
+    (Q5_K, 5, 9, 512),
+    (Q5_K, 7, 300, 4096),
+    (Q5_K, 16, 2000, 4096),     # one tile per workgroup, ragged last tile
+    (Q5_K, 9, 2300, 1280),      # ... partial last chunk of superblocks
+    (Q5_K, 37, 300, 1024),      # groups of 16 tokens
+    (Q5_K, 16, 22500, 512),     # a wave per tile
+    (Q5_K, 16, 6144, 4096),     # K cut over workgroups
+    (Q5_K, 6, 4100, 5376),      # ... runs of unequal length
 ]
 
 
@@ -387,7 +391,8 @@ def test_matmul_linearity_full_size(gpu):
 
 
 # ---- MoE indirection ------------------------------------------------------------------
-@pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 96, 512, False), (Q6_K, 64, 768, True)])
+@pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 96, 512, False), (Q6_K, 64, 768, True), (Q5_K, 96, 512, False),
+                                                 (Q5_K, 64, 768, True)])
 def test_moe_matmul_vs_oracle(gpu, kqo, type_, N, K, per_slot):
     from backpack_amd import kquant
     E, T, k = 6, 5, 3
@@ -532,14 +537,15 @@ def _routing(rng, T, E, k):
 
 
 @pytest.mark.parametrize("family", [0, 1, 3])
+@pytest.mark.parametrize("tgu,tdn", [(Q4_K, Q6_K), (Q5_K, Q5_K), (Q5_K, Q6_K), (Q4_K, Q5_K)])
 @pytest.mark.parametrize("T,E,k,H,I", [(1, 8, 2, 512, 512), (5, 6, 3, 512, 768), (40, 16, 4, 512, 512),
-                                       (3, 4, 2, 512, 256), (70, 5, 4, 768, 512)])
-def test_moe_ffn_vs_oracle(gpu, kqo, family, T, E, k, H, I):
+                                       (3, 4, 2, 512, 256), (70, 5, 4, 768, 512), (20, 64, 4, 512, 512)])
+def test_moe_ffn_vs_oracle(gpu, kqo, family, tgu, tdn, T, E, k, H, I):
     from backpack_amd import capi, kquant
-    _say("moe_ffn", T, E, k, H, I, "family", family)
-    _, gp, gw = gpu.make_weight(Q4_K, E * I, H, seed=41)
-    _, up, uw = gpu.make_weight(Q4_K, E * I, H, seed=42)
-    _, dp, dw = gpu.make_weight(Q6_K, E * H, I, seed=43)
+    _say("moe_ffn", tgu, tdn, T, E, k, H, I, "family", family)
+    _, gp, gw = gpu.make_weight(tgu, E * I, H, seed=41)
+    _, up, uw = gpu.make_weight(tgu, E * I, H, seed=42)
+    _, dp, dw = gpu.make_weight(tdn, E * H, I, seed=43)
     rng = np.random.default_rng(T + E)
     eidx, ew = _routing(rng, T, E, k)
     X = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
@@ -551,23 +557,28 @@ def test_moe_ffn_vs_oracle(gpu, kqo, family, T, E, k, H, I):
         capi.force_kernel(0)
     # two or more pairs per expert on average go to the 16x16 tile kernel (family 3 keeps them on the
     # row kernel); a single-block Q6_K down projection (inter = 256) is outside the row kernel's reach
+    # Q5_K has no row kernel: its thinly spread pairs beyond the lanes-along-K kernel's 64 take the tile kernel
+    q5 = Q5_K in (tgu, tdn)
     if family == 1:
         expect = "moe_ffn_generic"
     elif family == 0 and T * k >= 2 * E:
         expect = "moe_ffn_mtile"
-    elif family == 0:
+    elif family == 0 and T * k <= 64:
         expect = "moe_ffn_stream"     # a handful of pairs: one lanes-along-K matvec each
+    elif family == 0:
+        expect = "moe_ffn_mtile" if q5 else "moe_ffn_mrow"
     else:
-        expect = "moe_ffn_generic" if I == 256 else "moe_ffn_mrow"
+        expect = "moe_ffn_generic" if I == 256 or q5 else "moe_ffn_mrow"
     assert kern == expect, (kern, expect)
-    want = kqo.moe_ffn(Q4_K, Q6_K, X, gp, up, dp, eidx, ew, H, I)
+    want = kqo.moe_ffn(tgu, tdn, X, gp, up, dp, eidx, ew, H, I)
     rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
     err = np.abs(got - want)
     # three chained fp32 matvecs and an exp(): 1e-3 relative, floor 1e-3 of the output rms
     assert np.all(err <= 1e-3 * rms + 1e-3 * np.abs(want)), f"max err {err.max():.3g} rms {rms:.3g}"
 
 
-def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
+@pytest.mark.parametrize("tgu,tdn", [(Q4_K, Q6_K), (Q5_K, Q5_K)])
+def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo, tgu, tdn):
     """Qwen3-30B-A3B-shaped experts (128 x [768x2048 Q4_K gate/up, 2048x768 Q6_K down]),
     top-8 routing: T=1 against the oracle, T=256 grouped path against the ungrouped
     one on the GPU plus an oracle spot check of four tokens."""
@@ -576,7 +587,7 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
     E, k, H, I = 128, 8, 2048, 768
     mk = lambda t, N, K, seed: kquant.KQuantPacked(synth.make_packed_device(t, N, K, seed=seed), t, N, K,
                                                    synth.row_stride_words(t, K), synth.n_blocks(K))
-    gw, uw, dw = mk(Q4_K, E * I, H, 51), mk(Q4_K, E * I, H, 52), mk(Q6_K, E * H, I, 53)
+    gw, uw, dw = mk(tgu, E * I, H, 51), mk(tgu, E * I, H, 52), mk(tdn, E * H, I, 53)
     host = lambda w: w.data[: w.N * w.row_stride_bytes].cpu().numpy().view(np.uint32)
     gp, up, dp = host(gw), host(uw), host(dw)
     rng = np.random.default_rng(5)
@@ -588,7 +599,7 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
         got = kquant.moe_ffn(xd, gw, uw, dw, ed, wd, E).cpu().numpy()
         assert capi.last_kernel() == ("moe_ffn_stream" if T == 1 else "moe_ffn_mtile")
         sel = np.arange(T) if T == 1 else np.array([0, 100, 101, 255])
-        want = kqo.moe_ffn(Q4_K, Q6_K, X[sel], gp, up, dp, eidx[sel], ew[sel], H, I)
+        want = kqo.moe_ffn(tgu, tdn, X[sel], gp, up, dp, eidx[sel], ew[sel], H, I)
         rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
         assert np.all(np.abs(got[sel] - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
         if T > 1:
@@ -603,7 +614,7 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
             capi.force_kernel(3)   # the row kernel's grouped mode on the same routing
             try:
                 rowk = kquant.moe_ffn(xd, gw, uw, dw, ed, wd, E).cpu().numpy()
-                assert capi.last_kernel() == "moe_ffn_mrow"
+                assert capi.last_kernel() == ("moe_ffn_mrow" if tgu == Q4_K else "moe_ffn_generic")
             finally:
                 capi.force_kernel(0)
             assert np.all(np.abs(rowk - ref) <= 1e-3 * rms + 1e-3 * np.abs(ref))
@@ -613,7 +624,8 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo):
 @pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True),
                                                  # K of one chunk: waves walk several tiles per staged X; ragged last tile
                                                  (Q6_K, 2000, 768, True), (Q4_K, 1104, 1024, False),
-                                                 (Q6_K, 520, 512, False)])
+                                                 (Q6_K, 520, 512, False),
+                                                 (Q5_K, 768, 2048, False), (Q5_K, 2048, 768, True), (Q5_K, 1104, 1024, False)])
 def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot, family, kernel):
     """Ragged lists: some experts get many pairs, some none; repeated experts inside a token."""
     from backpack_amd import capi, kquant
@@ -622,6 +634,8 @@ def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot, family, kern
     rng = np.random.default_rng(62)
     eidx = rng.choice([0, 1, 1, 1, 5, 5, 7, 11], size=(T, k)).astype(np.uint32)   # experts 2,3,4,6,8,9,10 idle
     X = rng.standard_normal((T * k if per_slot else T, K)).astype(np.float32)
+    if type_ == Q5_K and family == 3:
+        kernel = "generic_indirect"      # no row kernel for the type
     capi.force_kernel(family)
     try:
         got = kquant.moe_matmul(gpu.dev(X), w, gpu.dev(eidx.view(np.int32)), E, x_per_slot=per_slot).cpu().numpy()
@@ -633,7 +647,8 @@ def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot, family, kern
     assert np.all(np.abs(got - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
 
 
-@pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True), (Q6_K, 300, 4096, False)])
+@pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True), (Q6_K, 300, 4096, False),
+                                                 (Q5_K, 768, 2048, False), (Q5_K, 2048, 768, True), (Q5_K, 300, 4096, False)])
 def test_moe_matmul_few_pairs_stream(gpu, kqo, type_, N, K, per_slot):
     """Decode-sized routing (fewer than two pairs per expert): one lanes-along-K matvec per pair."""
     from backpack_amd import capi, kquant
