@@ -29,8 +29,13 @@
 // half of k) in slot m and (m, second half) in slot m + 8, each with the other
 // half of its operand zeroed.  One MFMA then yields both 16-element sums, each
 // in lanes of its own that apply their own scale, and the two are added once
-// at the end.  (9..16 tokens are served as two calls of 8.)  The -32 offset of
-// the 6-bit values is applied against the sums of x over 16 elements.
+// at the end.  The -32 offset of the 6-bit values is applied against the sums
+// of x over 16 elements.  With 9..16 tokens every token keeps a slot of its own
+// and the weights pay instead: each run of 32 is multiplied twice, once whole
+// and once with the operand lanes of its second half zeroed, which gives the
+// sum over the first 16 elements and, by difference, the sum over the second
+// (twice the matrix instructions, but every weight byte is still fetched and
+// unpacked once for all 16 tokens).
 //
 // Work split.  A workgroup owns R tiles of 16 rows.  With R = NW every wave
 // owns a tile and walks all of K; with R = 1 (matrices of few rows) the waves of
@@ -58,10 +63,13 @@ __device__ __forceinline__ void wave_window_fence()
 
 constexpr int MT_KC = 4;                       // superblocks of X staged at a time
 constexpr int MT_XA_BYTES = MT_KC * 8 * 2 * 1024;   // [block][sub-block][hi/lo][lane] 16 B
-constexpr int MT_XS_FLOATS = MT_KC * 8 * 16;        // [block][sub-block][token]
+constexpr int MT_XS_FLOATS = MT_KC * 8 * 32;        // [block][sub-block][token], or [block][sub-block][half][token]
 constexpr int MT_INV_FLOATS = MT_KC * 16;           // [block][token]
 constexpr int MT_XV_BYTES = MT_KC * 2 * 1024;       // [block][hi/lo][lane] 16 B: the sub-block sums as an A operand (Q4_K)
 constexpr int MT_STAGE_BYTES = MT_XA_BYTES + (MT_XS_FLOATS + MT_INV_FLOATS) * 4 + MT_XV_BYTES;
+
+// Kernel variant beside the GGUF type codes: Q6_K blocks, 16 token slots.
+constexpr int MT_TYPE_Q6K_WIDE = 114;
 
 struct MtileParams {
     const float* X;
@@ -93,8 +101,11 @@ struct MtileParams {
 // TOK = 16 or 8 (4 works too): the tokens the workgroup's threads are spread over; a launch with few tokens takes a
 // small TOK so that every wave converts a share instead of the first waves converting everything.
 // XV: also stage the sub-block sums as an A operand (the Q4_K kernels that put the minima on the matrix cores).
-template <int NT, bool SPLIT16, int TOK, bool XV>
+// HALF: the sums of x go out per half run of 16 elements, [run][half][token] (the 16-token Q6_K kernel).
+template <int NT, bool SPLIT16, int TOK, bool XV, bool HALF = false>
 struct MtileStager {
+    static_assert(!(SPLIT16 && HALF), "half sums live in token slots (SPLIT16) or in a second plane (HALF)");
+    static constexpr uint32_t XSR = HALF ? 32u : 16u;   // floats of xs per run
     static constexpr int TPP = NT / (MT_KC * TOK);  // threads per (token, block) pair
     static constexpr int EPT = 256 / TPP;           // elements per thread
     static_assert(TPP <= 64 && (EPT == 64 || EPT == 32 || EPT == 16 || EPT == 8), "a pair is converted inside one wave");
@@ -195,8 +206,9 @@ struct MtileStager {
                     h0 += (v[8 * q + i].x + v[8 * q + i].y) + (v[8 * q + i].z + v[8 * q + i].w);
                     h1 += (v[8 * q + 4 + i].x + v[8 * q + 4 + i].y) + (v[8 * q + 4 + i].z + v[8 * q + 4 + i].w);
                 }
-                float* dst = xs + (bb * 8u + (sub * EPT) / 32u + q) * 16u + token;
+                float* dst = xs + (bb * 8u + (sub * EPT) / 32u + q) * XSR + token;
                 if (SPLIT16) { dst[0] = h0; dst[8] = h1; }
+                else if (HALF) { dst[0] = h0; dst[16] = h1; }
                 else { dst[0] = h0 + h1; put_sum((sub * EPT) / 32u + q, h0 + h1); }
             }
         } else {
@@ -207,9 +219,11 @@ struct MtileStager {
             constexpr int PER16 = 16 / EPT;   // threads per half run: 1 (EPT 16) or 2 (EPT 8)
             if (PER16 == 2) h += group_partner<1>(h);
             const uint32_t half = (sub / PER16) & 1u, run = sub / (2u * PER16);
-            float* dst = xs + (bb * 8u + run) * 16u + token;
+            float* dst = xs + (bb * 8u + run) * XSR + token;
             if (SPLIT16) {
                 if (sub % PER16 == 0u) dst[8u * half] = h;
+            } else if (HALF) {
+                if (sub % PER16 == 0u) dst[16u * half] = h;
             } else {
                 h += group_partner<PER16>(h);
                 if (sub % (2u * PER16) == 0u) { dst[0] = h; put_sum(run, h); }
@@ -439,6 +453,71 @@ __device__ __forceinline__ void q6k_mtile_block(const Q6TileW& w, const uint8_t*
     tot.w += fmaf(d24 * inv.w, U.w, -(d32 * V.w));
 }
 
+// Q6_K with 16 tokens: lane l holds tokens 4*(l/16) .. +3 of weight row l%16 as in the Q4_K kernel.  Every run of
+// 32 elements is multiplied whole and with the second half of the weight operand zeroed (the lanes of k >= 16):
+// D1 = sum over the first 16 elements, Dw - D1 = sum over the second, each with its own scale:
+// sc1 * D1 + sc2 * (Dw - D1) = (sc1 - sc2) * D1 + sc2 * Dw.  xs_b holds the sums of x per half run.
+__device__ __forceinline__ void q6k_mtile_block_wide(const Q6TileW& w, const uint8_t* xa_b, const float* xs_b,
+                                                     const float* xinv_b, uint32_t lane, t_f32x4& tot)
+{
+    const uint32_t tq = lane >> 4;
+    const uint32_t first = tq < 2u ? 0xFFFFFFFFu : 0u;   // this lane's k belong to the first half of a run
+    t_f32x4 U = {0, 0, 0, 0}, V = {0, 0, 0, 0};
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        t_u32x4 bq[4];   // B operands of runs t = 0..3 of this half
+#pragma unroll
+        for (int wd = 0; wd < 2; ++wd) {
+            const uint32_t A = w.ql[h][0][wd], B = w.ql[h][1][wd], H = w.qh[h][wd];
+            const uint32_t A8 = A >> 8, B8 = B >> 8;
+            const uint32_t Hl4 = H << 4, Hl2 = H << 2, Hr4 = H >> 4, Hr6 = H >> 6;
+            bq[0][2 * wd] = (A & 0x000F000Fu) | (Hl4 & 0x00300030u);
+            bq[0][2 * wd + 1] = (A8 & 0x000F000Fu) | (Hr4 & 0x00300030u);
+            bq[1][2 * wd] = (B & 0x000F000Fu) | (Hl2 & 0x00300030u);
+            bq[1][2 * wd + 1] = (B8 & 0x000F000Fu) | (Hr6 & 0x00300030u);
+            bq[2][2 * wd] = (A & 0x00F000F0u) | (Hl4 & 0x03000300u);
+            bq[2][2 * wd + 1] = (A8 & 0x00F000F0u) | (Hr4 & 0x03000300u);
+            bq[3][2 * wd] = (B & 0x00F000F0u) | (Hl2 & 0x03000300u);
+            bq[3][2 * wd + 1] = (B8 & 0x00F000F0u) | (Hr6 & 0x03000300u);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int run = 4 * h + t;
+            const uint8_t* ap = xa_b + ((size_t)(run * 2) * 64u + lane) * 16u;
+            const t_half8 ahi = *(const t_half8*)ap;
+            const t_half8 alo = *(const t_half8*)(ap + 1024);
+            const t_u32x4 b1 = {bq[t].x & first, bq[t].y & first, bq[t].z & first, bq[t].w & first};
+            const t_half8 bw8 = __builtin_bit_cast(t_half8, bq[t]);
+            const t_half8 b18 = __builtin_bit_cast(t_half8, b1);
+            t_f32x4 Dw = {0, 0, 0, 0}, D1 = {0, 0, 0, 0};
+            Dw = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bw8, Dw, 0, 0, 0);
+            D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, b18, D1, 0, 0, 0);
+            Dw = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bw8, Dw, 0, 0, 0);
+            D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, b18, D1, 0, 0, 0);
+            // scales of (half h, t): bytes 8h + 2t (first 16 elements) and 8h + 2t + 1 of the 16
+            const uint32_t word = w.sc[(8 * h + 2 * t) >> 2];
+            const uint32_t sh = 8u * ((2u * t) & 3u);
+            const float sv1 = (float)(int)(int8_t)((word >> sh) & 255u);
+            const float sv2 = (float)(int)(int8_t)((word >> (sh + 8u)) & 255u);
+            const float f = t >= 2 ? 0.0625f : 1.0f;   // t >= 2: the field sits four bits up
+            const float s2 = sv2 * f, s12 = (sv1 - sv2) * f;
+            const float4 x1 = *(const float4*)(xs_b + run * 32 + 4u * tq);
+            const float4 x2 = *(const float4*)(xs_b + run * 32 + 16 + 4u * tq);
+            U.x = fmaf(s12, D1.x, fmaf(s2, Dw.x, U.x)); U.y = fmaf(s12, D1.y, fmaf(s2, Dw.y, U.y));
+            U.z = fmaf(s12, D1.z, fmaf(s2, Dw.z, U.z)); U.w = fmaf(s12, D1.w, fmaf(s2, Dw.w, U.w));
+            V.x = fmaf(sv1, x1.x, fmaf(sv2, x2.x, V.x)); V.y = fmaf(sv1, x1.y, fmaf(sv2, x2.y, V.y));
+            V.z = fmaf(sv1, x1.z, fmaf(sv2, x2.z, V.z)); V.w = fmaf(sv1, x1.w, fmaf(sv2, x2.w, V.w));
+        }
+    }
+    const float4 inv = *(const float4*)(xinv_b + 4u * tq);
+    const float d = half_bits_to_float(w.d);
+    const float d24 = d * 16777216.0f, d32 = d * 32.0f;
+    tot.x += fmaf(d24 * inv.x, U.x, -(d32 * V.x));
+    tot.y += fmaf(d24 * inv.y, U.y, -(d32 * V.y));
+    tot.z += fmaf(d24 * inv.z, U.z, -(d32 * V.z));
+    tot.w += fmaf(d24 * inv.w, U.w, -(d32 * V.w));
+}
+
 // Weights travel HBM -> registers -> LDS in 16-byte units that are consecutive along a row, so every cache
 // line is fetched once and whole (a lane fetching only the 8-byte pieces its operands need makes each line
 // cross the L2 -> L1 path five times).  A wave stages SPAN bytes of each of its 16 rows in a private LDS
@@ -506,7 +585,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         if (blockIdx.y >= *p.n_tiles) return;   // whole workgroup
         rec = p.tiles + (size_t)blockIdx.y * p.tile_stride;
         // a record may hold more pairs than a pass of this kernel has token slots: blockIdx.z takes a slice
-        const uint32_t slots = TYPE == KQ_TYPE_Q6_K ? 8u : 16u;
+        const uint32_t slots = TYPE == KQ_TYPE_Q6_K ? 8u : 16u;   // (the 16-token Q6_K kernel has its own code: 16)
         const uint32_t first = blockIdx.z * slots;
         if (first >= rec[1]) return;            // whole workgroup
         count = min(rec[1] - first, slots);
@@ -518,8 +597,10 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     const uint32_t row = has_tile ? tile * 16u + (lane & 15u) : p.N;
     const uint32_t kq = lane >> 4;
 
-    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K, Q5 = TYPE == KQ_TYPE_Q5_K;
+    // Q6: the block format; Q6S: the 8-token kernel whose tokens take two slots each; Q6W: the 16-token one
+    constexpr bool Q6W = TYPE == MT_TYPE_Q6K_WIDE, Q6S = TYPE == KQ_TYPE_Q6_K, Q6 = Q6W || Q6S, Q5 = TYPE == KQ_TYPE_Q5_K;
     constexpr uint32_t BB = Q6 ? KQ_Q6K_BYTES : Q5 ? KQ_Q5K_BYTES : KQ_Q4K_BYTES;
+    constexpr uint32_t XSB = Q6W ? 256u : 128u;   // floats of xs per superblock
     constexpr uint32_t QOFF = Q5 ? 48u : 16u;   // where the quants start inside a block
     // A wave with a tile of its own stages two superblocks of its 16 rows at a time (two passes per chunk);
     // waves that share a tile stage the one superblock of the chunk that is theirs.
@@ -540,13 +621,13 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     const uint32_t c_begin = (p.tiles ? 0u : blockIdx.z) * p.chunks_per_split * MT_KC;
     const uint32_t c_end = min(p.n_blocks, c_begin + p.chunks_per_split * MT_KC);
 
-    MtileStager<64 * NW, Q6, TOK, STAGED && !Q6> stager;
+    MtileStager<64 * NW, Q6S, TOK, STAGED && !Q6, Q6W> stager;
     stager.init(p, rec, count);
     stager.fetch(p, c_begin);
     t_f32x4 tot = {0, 0, 0, 0};
     // a finished tile: lane l holds tokens 4*(l/16) .. +3 of weight row row_t
     auto put_tile = [&](uint32_t row_t, const t_f32x4& t) {
-        if (row_t < p.N && (!Q6 || kq < 2u)) {
+        if (row_t < p.N && (!Q6S || kq < 2u)) {
             const float bias = p.bias ? p.bias[row_t] : 0.0f;
             const float t4[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
@@ -560,7 +641,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         }
     };
     auto store_tile = [&](uint32_t row_t, t_f32x4 t) {
-        if constexpr (Q6) {   // lanes l and l + 32 hold the two 16-element halves of the same tokens
+        if constexpr (Q6S) {   // lanes l and l + 32 hold the two 16-element halves of the same tokens
             t.x += __shfl_xor(t.x, 32, 64);
             t.y += __shfl_xor(t.y, 32, 64);
             t.z += __shfl_xor(t.z, 32, 64);
@@ -599,7 +680,10 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                     if constexpr (Q6) {
                         Q6TileW w6;
                         q6k_mtile_load(blk, kq, w6);
-                        q6k_mtile_block(w6, xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                        if constexpr (Q6W)
+                            q6k_mtile_block_wide(w6, xa + (size_t)bb * (8 * 2 * 1024), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                        else
+                            q6k_mtile_block(w6, xa + (size_t)bb * (8 * 2 * 1024), xs + bb * XSB, xinv + bb * 16, lane, tot);
                     } else {
                         const t_u32x4 hdr = *(const t_u32x4*)blk;
                         t_u32x2 w[4], qhw = {0, 0};
@@ -656,8 +740,10 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
             for (int i = 0; i < BPC; ++i) {
                 const uint32_t bb = R == 1 ? wave + i * NW : i;
                 if (bb < MT_KC && c0 + bb < c_end) {
-                    if constexpr (Q6)
-                        q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                    if constexpr (Q6W)
+                        q6k_mtile_block_wide(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                    else if constexpr (Q6)
+                        q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * XSB, xinv + bb * 16, lane, tot);
                     else
                         q4k_mtile_block_compact<Q5>(hdr[i], w[i], qhw[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
                 }
@@ -681,7 +767,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
             tot.x += o.x; tot.y += o.y; tot.z += o.z; tot.w += o.w;
         }
     }
-    if constexpr (Q6) {
+    if constexpr (Q6S) {
         // lanes l and l + 32 hold the two 16-element halves of tokens 4*(l/16) .. +3: add them
         tot.x += __shfl_xor(tot.x, 32, 64);
         tot.y += __shfl_xor(tot.y, 32, 64);
@@ -693,7 +779,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         // ticket once they are acknowledged, and the last one in reads all of them back past the
         // non-coherent cache levels and adds them in split order.
         const size_t plane = (size_t)gridDim.x * p.tiles_per_wg * 16u;   // rows of all tiles
-        const bool mine = has_tile && (!Q6 || kq < 2u);
+        const bool mine = has_tile && (!Q6S || kq < 2u);
         const uint32_t prow = tile * 16u + (lane & 15u);
         if (mine) {
             const float t4[4] = {tot.x, tot.y, tot.z, tot.w};
@@ -737,7 +823,7 @@ bool mtile_supported(const MatmulArgs& a)
 template <int TYPE, int NW, int R, bool STAGED = true, int TOK = 16>
 static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s, uint32_t wgs_z = 1)
 {
-    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K, Q5 = TYPE == KQ_TYPE_Q5_K;
+    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K || TYPE == MT_TYPE_Q6K_WIDE, Q5 = TYPE == KQ_TYPE_Q5_K;
     constexpr int PITCH = Q6 ? (R == 1 ? 240 : 464) : Q5 ? (R == 1 ? 176 : 368) : (R == 1 ? 160 : 304);   // as in the kernel
     constexpr size_t shmem = MT_STAGE_BYTES + (STAGED ? (size_t)NW * 16 * PITCH : 0);
     auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK>;
@@ -751,13 +837,14 @@ static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t 
     return hipGetLastError();
 }
 
-uint32_t mtile_group_cap(int type) { return type == KQ_TYPE_Q6_K ? 8u : 16u; }
+uint32_t mtile_group_cap(int) { return 16u; }
 
 hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, const uint32_t* n_tiles,
                                 uint32_t tiles_bound, uint32_t cap, hipStream_t s)
 {
-    // records of up to cap pairs; a record beyond the kernel's token slots (Q6_K: 8) is served in slices
-    const uint32_t slices = (cap + mtile_group_cap(a.type) - 1u) / mtile_group_cap(a.type);
+    // records of up to cap pairs: Q6_K runs its 8-token kernel for records of up to 8, the 16-token one beyond
+    const bool q6_wide = a.type == KQ_TYPE_Q6_K && cap > 8u;
+    const uint32_t slices = 1;
     if (cap == 0 || cap > 16u || tiles_bound == 0 || tiles_bound > 65535u) return hipErrorInvalidValue;
     MtileParams p;
     p.X = (const float*)a.X;
@@ -789,6 +876,7 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
         p.tile_iters = groups >= 32u ? 8u : groups >= 16u ? 4u : groups >= 8u ? 2u : 1u;
     }
     const uint32_t wgs = (row_tiles + tpw * p.tile_iters - 1u) / (tpw * p.tile_iters);
+    if (q6_wide) return launch_mtile_one<MT_TYPE_Q6K_WIDE, 4, 4, false>(p, wgs, tiles_bound, s, slices);
     if (a.type == KQ_TYPE_Q6_K) return launch_mtile_one<KQ_TYPE_Q6_K, 4, 4, false>(p, wgs, tiles_bound, s, slices);
     if (a.type == KQ_TYPE_Q5_K) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, false>(p, wgs, tiles_bound, s, slices);
     return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, false>(p, wgs, tiles_bound, s, slices);
@@ -797,8 +885,9 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
 hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s)
 {
     const bool q6 = a.type == KQ_TYPE_Q6_K;
-    // Q6_K tiles hold 8 tokens: more are served in groups of 8, each reading the weights again
-    const uint32_t group = q6 ? 8u : 16u;
+    // Q6_K: up to 8 tokens on the kernel whose tokens take two slots each, more on the 16-token kernel
+    const bool q6_wide = q6 && a.M > 8u;
+    const uint32_t group = 16u;
     const uint32_t tiles = (a.N + 15u) / 16u;
     const uint32_t n_chunks = (a.n_blocks + MT_KC - 1) / MT_KC;
     const uint32_t cus = device_cu_count();
@@ -844,7 +933,8 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
         hipError_t e;
         const bool q5 = a.type == KQ_TYPE_Q5_K;
         if (shared_tile) {
-            e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 4, 1>(p, tiles, 1, s)
+            e = q6_wide ? launch_mtile_one<MT_TYPE_Q6K_WIDE, 4, 1>(p, tiles, 1, s)
+                : q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 4, 1>(p, tiles, 1, s)
                 : q5 ? launch_mtile_one<KQ_TYPE_Q5_K, 4, 1>(p, tiles, 1, s) : launch_mtile_one<KQ_TYPE_Q4_K, 4, 1>(p, tiles, 1, s);
         } else {
             p.tiles_per_wg = best_tpw;
@@ -858,7 +948,8 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
                     : q5 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits)
                          : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits);
             else
-                e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits)
+                e = q6_wide ? launch_mtile_one<MT_TYPE_Q6K_WIDE, 8, 8, true, 16>(p, wgs, 1, s, best_splits)
+                    : q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits)
                     : q5 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits)
                          : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits);
         }
