@@ -518,6 +518,16 @@ int bpk_kq_matmul_fused(int type, const float* X, const void* W, const float* bi
         }
         if (t_family == 5) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");
     }
+    // verify batches: one launch of the tile kernel
+    if (!t_fused_separate && (t_family == 0 || t_family == 6)) {
+        a.pro = f->prologue; a.norm_w = f->norm_w; a.eps = f->eps; a.residual = f->residual; a.epi = f->epilogue;
+        if (kq::mtile_fused_supported(a)) {
+            t_kernel = "mtile_fused";
+            const hipError_t e = kq::launch_mtile_fused(a, st->split, s);
+            return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+        }
+        if (t_family == 6) return fail(BPK_ERR_SHAPE, "16x16 tile kernel cannot serve this call");
+    }
     // otherwise the same function in up to three launches through the caller's workspace
     const size_t x_bytes = ((size_t)M * K * sizeof(float) + 255u) & ~(size_t)255u;
     const bool need_x = f->prologue != BPK_PRO_NONE, need_y = f->residual != nullptr || epi;

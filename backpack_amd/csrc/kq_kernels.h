@@ -106,6 +106,9 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
 // grouped by expert: records {expert, count, pair ids...} of up to cap pairs, as launch_moe_group
 // writes them with sets = cap / 2; cap at most mtile_group_cap(type)
 uint32_t mtile_group_cap(int type);
+// the fused forms (MatmulArgs pro / residual / epi) on the tile kernel, up to 16 tokens, one launch
+bool mtile_fused_supported(const MatmulArgs& a);
+hipError_t launch_mtile_fused(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s);
 hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, const uint32_t* n_tiles,
                                 uint32_t tiles_bound, uint32_t cap, hipStream_t s);
 

@@ -86,6 +86,16 @@ struct MtileParams {
     uint32_t* counters;      // one per blockIdx.x, zero between launches
     // grouped mode (tiles != nullptr): blockIdx.y walks records {expert, count, pair ids...} of up to
     // 16 (Q4_K) / 8 (Q6_K) (token, slot) pairs that share an expert; N is the rows of one expert
+    // fused forms (the FUSED instantiations, dense calls of up to 16 tokens).  pro 1: x = X * rsqrt(mean(X^2) + eps)
+    // * norm_w; pro 2 / 3: X rows are gate | up, 2K floats, x = silu / gelu_tanh (gate) * up.  residual is added to
+    // every output (indexed like Y, may be Y).  epi 2 / 3: W is gate | up stacked, the first half of a workgroup's
+    // waves own gate tiles, the second half the up tiles pair_tile0 further on, and Y = act(gate) * up.
+    int pro, epi;
+    float eps;
+    const float* norm_w;
+    const float* residual;
+    uint32_t x_stride;      // floats between rows of X
+    uint32_t pair_tile0;    // tiles of gate rows (= outputs / 16)
     const uint32_t* tiles;
     const uint32_t* n_tiles;
     uint32_t tile_iters;    // grouped calls whose K is a single chunk: tiles a wave walks with X staged once
@@ -93,6 +103,19 @@ struct MtileParams {
     uint32_t k_slots;
     int x_per_slot;         // X row of a pair: the pair itself (1) or its token, pair / k_slots (0)
 };
+
+// silu(g) * u (ACT 2) or gelu_tanh(g) * u (ACT 3), as the fused entry point defines them
+template <int ACT>
+__device__ __forceinline__ float mtile_act(float g, float u)
+{
+    if constexpr (ACT == 2) {
+        return g / (__expf(-g) + 1.0f) * u;
+    } else {
+        const float inner = 0.7978845608f * (g + 0.044715f * g * g * g);
+        // tanh(z) = 1 - 2 / (exp(2z) + 1); 0.5 g (1 + tanh z) = g - g / (exp(2z) + 1)
+        return (g - g / (__expf(2.0f * inner) + 1.0f)) * u;
+    }
+}
 
 // Conversion of a chunk's activations.  Thread (pair, sub) handles EPT
 // consecutive elements of one (token, superblock) pair; pairs are numbered
@@ -102,7 +125,9 @@ struct MtileParams {
 // small TOK so that every wave converts a share instead of the first waves converting everything.
 // XV: also stage the sub-block sums as an A operand (the Q4_K kernels that put the minima on the matrix cores).
 // HALF: the sums of x go out per half run of 16 elements, [run][half][token] (the 16-token Q6_K kernel).
-template <int NT, bool SPLIT16, int TOK, bool XV, bool HALF = false>
+// PRO: the prologues of the fused forms.  1: RMSNorm, the chunk's norm weights are read from LDS (nw, staged by
+// the kernel); 2: act(gate) * up, up travels with X.
+template <int NT, bool SPLIT16, int TOK, bool XV, bool HALF = false, int PRO = 0>
 struct MtileStager {
     static_assert(!(SPLIT16 && HALF), "half sums live in token slots (SPLIT16) or in a second plane (HALF)");
     static constexpr uint32_t XSR = HALF ? 32u : 16u;   // floats of xs per run
@@ -110,6 +135,8 @@ struct MtileStager {
     static constexpr int EPT = 256 / TPP;           // elements per thread
     static_assert(TPP <= 64 && (EPT == 64 || EPT == 32 || EPT == 16 || EPT == 8), "a pair is converted inside one wave");
     float4 v[EPT / 4];
+    float4 v2[PRO == 2 ? EPT / 4 : 1];
+    float ss = 0.0f;   // norm prologue: sum of squares of this thread's elements so far
     uint32_t token, bb, sub;
     bool live_token;
 
@@ -133,9 +160,51 @@ struct MtileStager {
     {
         if (!live_token) return;   // wave-uniform for whole waves of dead tokens
         const uint32_t b = min(c0 + bb, p.n_blocks - 1u);
+        if constexpr (PRO == 2) {
+            const float4* src = (const float4*)(p.X + (size_t)xrow * p.x_stride + (size_t)b * KQ_QK + sub * EPT);
+            const float4* src2 = (const float4*)((const float*)src + p.K);
+#pragma unroll
+            for (int i = 0; i < EPT / 4; ++i) v[i] = src[i];
+#pragma unroll
+            for (int i = 0; i < EPT / 4; ++i) v2[i] = src2[i];
+            return;
+        }
         const float4* src = (const float4*)(p.X + (size_t)xrow * p.K + (size_t)b * KQ_QK + sub * EPT);
 #pragma unroll
         for (int i = 0; i < EPT / 4; ++i) v[i] = src[i];
+    }
+    // the prologue on what fetch() brought.  The norm's 1 / rms is a factor per token: it is applied to the
+    // outputs, and the sum of squares it needs is gathered here (live: the superblock exists).  nw: the chunk's
+    // norm weights in LDS, [superblock of the chunk][256].
+    __device__ __forceinline__ void prologue(const MtileParams& p, bool live, const float* nw)
+    {
+        if (!live_token) return;
+        if constexpr (PRO == 1) {
+            const float4* w4 = (const float4*)(nw + bb * KQ_QK + sub * EPT);
+#pragma unroll
+            for (int i = 0; i < EPT / 4; ++i) {
+                if (live) {
+                    ss = fmaf(v[i].x, v[i].x, ss); ss = fmaf(v[i].y, v[i].y, ss);
+                    ss = fmaf(v[i].z, v[i].z, ss); ss = fmaf(v[i].w, v[i].w, ss);
+                }
+                const float4 w = w4[i];
+                v[i].x *= w.x; v[i].y *= w.y; v[i].z *= w.z; v[i].w *= w.w;
+            }
+        } else if constexpr (PRO == 2) {
+            if (p.pro == 2) {
+#pragma unroll
+                for (int i = 0; i < EPT / 4; ++i) {
+                    v[i].x = mtile_act<2>(v[i].x, v2[i].x); v[i].y = mtile_act<2>(v[i].y, v2[i].y);
+                    v[i].z = mtile_act<2>(v[i].z, v2[i].z); v[i].w = mtile_act<2>(v[i].w, v2[i].w);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < EPT / 4; ++i) {
+                    v[i].x = mtile_act<3>(v[i].x, v2[i].x); v[i].y = mtile_act<3>(v[i].y, v2[i].y);
+                    v[i].z = mtile_act<3>(v[i].z, v2[i].z); v[i].w = mtile_act<3>(v[i].w, v2[i].w);
+                }
+            }
+        }
     }
     // converts what fetch() brought and parks it in LDS (slots of tokens beyond M stay zero)
     __device__ __forceinline__ void park(uint8_t* xa, float* xs, float* xinv, uint8_t* xv)
@@ -527,16 +596,19 @@ template <int SPAN, int PITCH>
 struct MtileWStage {
     static constexpr int UPR = (SPAN + 15) / 16;            // units per row
     static constexpr int NU = (16 * UPR + 63) / 64;         // units per lane
-    const uint8_t* src[NU];
+    const uint8_t* base;        // the tile's first row (the same for all lanes)
+    uint32_t src[NU];           // byte offset of the unit's row from there (16 rows: fits 32 bits)
     uint32_t dst[NU], col[NU];
     t_u32x4 raw[NU];
     __device__ __forceinline__ void init(const uint8_t* wmat, uint32_t row0, uint32_t N, uint32_t row_stride, uint32_t lane)
     {
+        const uint32_t first = min(row0, N - 1u);
+        base = wmat + (size_t)first * row_stride;
 #pragma unroll
         for (int i = 0; i < NU; ++i) {
             const uint32_t u = min((uint32_t)i * 64u + lane, 16u * UPR - 1u);   // spare lanes repeat the last unit
             const uint32_t r = u / UPR, c = u - r * UPR;
-            src[i] = wmat + (size_t)min(row0 + r, N - 1u) * row_stride;
+            src[i] = (min(row0 + r, N - 1u) - first) * row_stride;
             col[i] = c * 16u;
             dst[i] = r * PITCH + c * 16u;
         }
@@ -548,7 +620,7 @@ struct MtileWStage {
 #pragma unroll
         for (int i = 0; i < NU; ++i) {
             const uint32_t o = off + col[i];
-            __builtin_memcpy(&raw[i], src[i] + (o < row_bytes ? o : row_bytes - 16u), 16);
+            __builtin_memcpy(&raw[i], base + (src[i] + (o < row_bytes ? o : row_bytes - 16u)), 16);
         }
     }
     __device__ __forceinline__ void store(uint8_t* window) const
@@ -562,7 +634,8 @@ struct MtileWStage {
 // chunks per workgroup and run thousands of workgroups: there the windows' LDS (one workgroup per CU instead
 // of two) costs more than the line re-fetches, so they load each lane's pieces straight from global memory.
 // (the grouped Q4_K kernel is held to 128 registers so that two of its workgroups share a CU)
-template <int TYPE, int NW, int R, bool STAGED, int TOK>
+// FUSED: residual and pair epilogue; PRO: the prologue (1 RMSNorm, 2 act(gate) * up)
+template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0>
 __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1) void mtile_kernel(MtileParams p)
 // (Q5_K: the Q4_K code with blocks of 176 bytes — header, 32 bytes of fifth bits, quants — and one more
 // 8-byte piece per lane and superblock)
@@ -592,8 +665,18 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         wmat += (size_t)rec[0] * p.N * p.row_stride_bytes;
         rec += first;                           // rec[2 + token] is now the slice's pair
     }
-    const bool has_tile = R == 1 || wave < p.tiles_per_wg;
-    const uint32_t tile = R == 1 ? blockIdx.x : blockIdx.x * p.tiles_per_wg + wave;
+    static_assert(!FUSED || (R == NW && STAGED), "the fused forms come with a wave per tile, weights staged");
+    static_assert(FUSED || PRO == 0, "prologues belong to the fused kernels");
+    bool has_tile = R == 1 || wave < p.tiles_per_wg;
+    uint32_t tile = R == 1 ? blockIdx.x : blockIdx.x * p.tiles_per_wg + wave;
+    const bool pairs = FUSED && p.epi != 0;
+    const uint32_t half_waves = p.tiles_per_wg >> 1;
+    if (pairs) {
+        // waves 0 .. h-1: gate tiles g*h .. +h-1; waves h .. 2h-1: the up tiles of the same outputs
+        const uint32_t gate = blockIdx.x * half_waves + (wave < half_waves ? wave : wave - half_waves);
+        has_tile = wave < p.tiles_per_wg && gate < p.pair_tile0;
+        tile = wave < half_waves ? gate : p.pair_tile0 + gate;
+    }
     const uint32_t row = has_tile ? tile * 16u + (lane & 15u) : p.N;
     const uint32_t kq = lane >> 4;
 
@@ -621,9 +704,34 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     const uint32_t c_begin = (p.tiles ? 0u : blockIdx.z) * p.chunks_per_split * MT_KC;
     const uint32_t c_end = min(p.n_blocks, c_begin + p.chunks_per_split * MT_KC);
 
-    MtileStager<64 * NW, Q6S, TOK, STAGED && !Q6, Q6W> stager;
+    MtileStager<64 * NW, Q6S, TOK, STAGED && !Q6, Q6W, PRO> stager;
     stager.init(p, rec, count);
     stager.fetch(p, c_begin);
+    // norm prologue: the sums of squares per token are gathered while X is converted and meet here at the end
+    // (16 floats behind the staging area); the outputs are scaled, not the activations
+    float* rinv = (float*)(smem + MT_STAGE_BYTES + NW * (16 * PITCH));
+    static_assert(!FUSED || (NW == 8 && TOK == 16), "a token's 32 converting threads are half a wave");
+    // ... and the norm weights of a chunk (4 x 256 floats) are shared by all tokens: 256 threads bring them two
+    // chunks ahead into registers and one chunk ahead into one of two LDS buffers behind the sums
+    float* nwbuf = rinv + 16;
+    float4 nwv = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto nw_fetch = [&](uint32_t c0) {
+        if constexpr (PRO == 1) {
+            if (threadIdx.x < 256u) {
+                const uint32_t b = min(c0 + (threadIdx.x >> 6), p.n_blocks - 1u);
+                nwv = *(const float4*)(p.norm_w + (size_t)b * KQ_QK + (threadIdx.x & 63u) * 4u);
+            }
+        }
+    };
+    auto nw_park = [&](uint32_t parity) {
+        if constexpr (PRO == 1) {
+            if (threadIdx.x < 256u) *(float4*)(nwbuf + parity * (MT_KC * KQ_QK) + threadIdx.x * 4u) = nwv;
+        }
+    };
+    uint32_t nw_parity = 0;
+    nw_fetch(c_begin);
+    nw_park(0);
+    nw_fetch(c_begin + MT_KC);
     t_f32x4 tot = {0, 0, 0, 0};
     // a finished tile: lane l holds tokens 4*(l/16) .. +3 of weight row row_t
     auto put_tile = [&](uint32_t row_t, const t_f32x4& t) {
@@ -635,7 +743,12 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                 const uint32_t token = 4u * kq + r;
                 if (token < count) {
                     const uint32_t yrow = rec ? rec[2u + token] : token;
-                    p.Y[(size_t)yrow * p.ldy + p.y_offset + row_t] = t4[r] + bias;
+                    const size_t at = (size_t)yrow * p.ldy + p.y_offset + row_t;
+                    float y = t4[r] + bias;
+                    if constexpr (FUSED) {
+                        if (p.residual) y += p.residual[at];
+                    }
+                    p.Y[at] = y;
                 }
             }
         }
@@ -658,11 +771,15 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     __syncthreads();
 
     for (uint32_t c0 = c_begin; c0 < c_end; c0 += MT_KC) {
+        stager.prologue(p, c0 + stager.bb < c_end, nwbuf + nw_parity * (MT_KC * KQ_QK));
         stager.park(xa, xs, xinv, xv);
+        nw_parity ^= 1u;
+        nw_park(nw_parity);           // the next chunk's norm weights (this buffer was last read one barrier ago)
         ws[0].store(wwin);
         __syncthreads();
         // the next chunk of X and of the weights travels while this one is multiplied
         stager.fetch(p, c0 + MT_KC);
+        nw_fetch(c0 + 2u * MT_KC);
         ws[0].load(pass_block(c0 + MT_KC, 0) * BB, row_bytes);
 #pragma unroll
         for (int h = 0; h < PASSES; ++h) {
@@ -774,13 +891,24 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         tot.z += __shfl_xor(tot.z, 32, 64);
         tot.w += __shfl_xor(tot.w, 32, 64);
     }
+    constexpr bool normed = PRO == 1;
+    if constexpr (PRO == 1) {
+        if (normed) {
+            // thread t converted for token t / 32: the sums of this workgroup's part of K, per token
+            float ss = stager.ss;
+            ss += __shfl_xor(ss, 16, 64); ss += __shfl_xor(ss, 8, 64); ss += __shfl_xor(ss, 4, 64);
+            ss += __shfl_xor(ss, 2, 64); ss += __shfl_xor(ss, 1, 64);
+            if ((threadIdx.x & 31u) == 0u) rinv[threadIdx.x >> 5] = ss;
+            __syncthreads();
+        }
+    }
     if (R == NW && p.n_splits > 1) {   // (only the wave-per-tile kernels are launched with splits)
         // Same hand-over as the split GEMV: partial sums go out as agent-scope stores, the workgroup takes a
         // ticket once they are acknowledged, and the last one in reads all of them back past the
         // non-coherent cache levels and adds them in split order.
         const size_t plane = (size_t)gridDim.x * p.tiles_per_wg * 16u;   // rows of all tiles
         const bool mine = has_tile && (!Q6S || kq < 2u);
-        const uint32_t prow = tile * 16u + (lane & 15u);
+        const uint32_t prow = (blockIdx.x * p.tiles_per_wg + wave) * 16u + (lane & 15u);
         if (mine) {
             const float t4[4] = {tot.x, tot.y, tot.z, tot.w};
 #pragma unroll
@@ -788,6 +916,10 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                 __hip_atomic_store(p.partial + ((size_t)blockIdx.z * 16u + 4u * kq + r) * plane + prow, t4[r], __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
         }
+        // (norm prologue: the splits' sums of squares travel the same way, behind the partial tiles)
+        float* ssq = p.partial + (size_t)p.n_splits * 16u * plane + (size_t)blockIdx.x * p.n_splits * 16u;
+        if (normed && threadIdx.x < 16u)
+            __hip_atomic_store(ssq + blockIdx.z * 16u + threadIdx.x, rinv[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         uint32_t* ticket = (uint32_t*)(smem + 16);
@@ -804,7 +936,44 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
                                                __HIP_MEMORY_SCOPE_AGENT);
             tot = t_f32x4{t4[0], t4[1], t4[2], t4[3]};
         }
+        if (normed) {
+            if (threadIdx.x < 16u) {
+                float t = 0.0f;
+                for (uint32_t z = 0; z < p.n_splits; ++z)
+                    t += __hip_atomic_load(ssq + z * 16u + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                rinv[threadIdx.x] = t;
+            }
+            __syncthreads();
+        }
         if (threadIdx.x == 0) __hip_atomic_store(&p.counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if constexpr (PRO == 1) {
+        if (normed) {
+            const float4 q = *(const float4*)(rinv + 4u * kq);
+            const float k1 = 1.0f / (float)p.K;
+            tot.x *= 1.0f / sqrtf(fmaf(q.x, k1, p.eps)); tot.y *= 1.0f / sqrtf(fmaf(q.y, k1, p.eps));
+            tot.z *= 1.0f / sqrtf(fmaf(q.z, k1, p.eps)); tot.w *= 1.0f / sqrtf(fmaf(q.w, k1, p.eps));
+        }
+    }
+    if constexpr (FUSED) {
+        if (pairs) {
+            // the up waves hand their tiles (bias added) to the gate waves of the same outputs
+            __syncthreads();   // the staging area is free
+            const float b = (has_tile && p.bias) ? p.bias[row] : 0.0f;
+            if (wave >= half_waves && wave < p.tiles_per_wg)
+                *(t_f32x4*)(red + ((wave - half_waves) * 64u + lane) * 4u) = t_f32x4{tot.x + b, tot.y + b, tot.z + b, tot.w + b};
+            __syncthreads();
+            if (wave >= half_waves || !has_tile || (Q6S && kq >= 2u)) return;
+            const t_f32x4 up = *(const t_f32x4*)(red + (wave * 64u + lane) * 4u);
+            const float g4[4] = {tot.x + b, tot.y + b, tot.z + b, tot.w + b}, u4[4] = {up.x, up.y, up.z, up.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t token = 4u * kq + r;
+                if (token < count)
+                    p.Y[(size_t)token * p.ldy + p.y_offset + row] = p.epi == 2 ? mtile_act<2>(g4[r], u4[r]) : mtile_act<3>(g4[r], u4[r]);
+            }
+            return;
+        }
     }
     put_tile(row, tot);
 }
@@ -820,13 +989,15 @@ bool mtile_supported(const MatmulArgs& a)
     return false;
 }
 
-template <int TYPE, int NW, int R, bool STAGED = true, int TOK = 16>
+template <int TYPE, int NW, int R, bool STAGED = true, int TOK = 16, bool FUSED = false, int PRO = 0>
 static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s, uint32_t wgs_z = 1)
 {
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K || TYPE == MT_TYPE_Q6K_WIDE, Q5 = TYPE == KQ_TYPE_Q5_K;
     constexpr int PITCH = Q6 ? (R == 1 ? 240 : 464) : Q5 ? (R == 1 ? 176 : 368) : (R == 1 ? 160 : 304);   // as in the kernel
-    constexpr size_t shmem = MT_STAGE_BYTES + (STAGED ? (size_t)NW * 16 * PITCH : 0);
-    auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK>;
+    // + the sums of squares per token and two chunks of norm weights
+    constexpr size_t shmem = MT_STAGE_BYTES + (STAGED ? (size_t)NW * 16 * PITCH : 0) + (FUSED ? 64 : 0) +
+                             (PRO == 1 ? 2 * MT_KC * KQ_QK * 4 : 0);
+    auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK, FUSED, PRO>;
     static bool raised = false;   // per instantiation
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -862,6 +1033,7 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
     p.n_splits = 1; p.chunks_per_split = (a.n_blocks + MT_KC - 1) / MT_KC; p.partial = nullptr; p.counters = nullptr;
     p.k_slots = a.k_slots;
     p.x_per_slot = a.x_per_slot;
+    p.pro = 0; p.epi = 0; p.eps = 0.0f; p.norm_w = nullptr; p.residual = nullptr; p.x_stride = a.K; p.pair_tile0 = 0;
     // a wave per 16-row tile of the expert, X of the record converted once per workgroup.  These workgroups walk
     // one or two chunks and are bound by their latencies, so two must share a CU: Q4_K runs 8 tiles per
     // workgroup at 128 registers, Q6_K (160 registers) 4 tiles per workgroup of 4 waves.
@@ -930,6 +1102,7 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
         p.tiles_per_wg = 1;
         p.tiles = nullptr; p.n_tiles = nullptr; p.tile_stride = 0; p.tile_iters = 1; p.k_slots = 1; p.x_per_slot = 0;
         p.n_splits = 1; p.chunks_per_split = n_chunks; p.partial = sc.partial; p.counters = sc.counters;
+        p.pro = 0; p.epi = 0; p.eps = 0.0f; p.norm_w = nullptr; p.residual = nullptr; p.x_stride = a.K; p.pair_tile0 = 0;
         hipError_t e;
         const bool q5 = a.type == KQ_TYPE_Q5_K;
         if (shared_tile) {
@@ -956,6 +1129,75 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
+}
+
+// The fused forms of the decode matvec for verify batches (3..16 tokens; one or two as well where the
+// lanes-along-K kernel declines): prologue in the conversion of X, residual in the store, act(gate) * up between
+// the waves of a workgroup.  One launch, a wave per tile.
+bool mtile_fused_supported(const MatmulArgs& a)
+{
+    if (a.expert_idx || a.M < 1 || a.M > 16 || !mtile_supported(a)) return false;
+    if (a.pro == 1 && ((uintptr_t)a.norm_w & 15u)) return false;
+    if (a.pro >= 2 && a.type == KQ_TYPE_Q6_K && a.M > 8u) return false;   // no registers for up beside 16 Q6_K token slots
+    if (a.epi && (a.N & 31u)) return false;   // gate and up tiles of 16 rows each
+    return true;
+}
+
+hipError_t launch_mtile_fused(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s)
+{
+    const bool q6 = a.type == KQ_TYPE_Q6_K, q5 = a.type == KQ_TYPE_Q5_K, q6_wide = q6 && a.M > 8u;
+    const uint32_t tiles = (a.N + 15u) / 16u;
+    const uint32_t n_chunks = (a.n_blocks + MT_KC - 1) / MT_KC;
+    const uint32_t cus = device_cu_count();
+    // the work split of launch_mtile; pairs take an even number of tiles per workgroup
+    uint32_t best_tpw = 8, best_splits = 1, best_cps = n_chunks;
+    float best_cost = 1e30f;
+    for (uint32_t tpw = 8; tpw >= 4; tpw -= a.epi ? 2u : 1u) {
+        const uint32_t groups = a.epi ? (tiles / 2u + tpw / 2u - 1u) / (tpw / 2u) : (tiles + tpw - 1u) / tpw;
+        for (uint32_t splits = 1; splits <= n_chunks && splits <= 16u; ++splits) {
+            const uint32_t cps = (n_chunks + splits - 1u) / splits;
+            if ((splits - 1u) * cps >= n_chunks) continue;   // a split would be empty
+            // (partial tiles, then 16 sums of squares per workgroup for the norm prologue)
+            if (splits > 1u && ((size_t)splits * 16u * groups * (tpw * 16u + 1u) > sc.capacity_floats || groups > sc.n_counters)) continue;
+            const uint32_t wgs = groups * splits, rounds = (wgs + cus - 1u) / cus;
+            const float idle = 1.0f - (float)wgs / (float)(rounds * cus);
+            const float cost = (float)rounds * ((float)cps + 1.5f) * (1.0f + 0.5f * idle);
+            if (cost < best_cost) { best_cost = cost; best_tpw = tpw; best_splits = splits; best_cps = cps; }
+        }
+    }
+    MtileParams p;
+    p.X = (const float*)a.X;
+    p.W = a.W;
+    p.bias = a.bias;
+    p.Y = a.Y;
+    p.M = a.M; p.N = a.N; p.K = a.K;
+    p.n_blocks = a.n_blocks;
+    p.row_stride_bytes = a.row_stride_bytes;
+    p.y_offset = a.y_offset;
+    p.ldy = a.ldy;
+    p.tiles_per_wg = best_tpw;
+    p.tiles = nullptr; p.n_tiles = nullptr; p.tile_stride = 0; p.tile_iters = 1; p.k_slots = 1; p.x_per_slot = 0;
+    p.n_splits = best_splits; p.chunks_per_split = best_cps; p.partial = sc.partial; p.counters = sc.counters;
+    p.pro = a.pro; p.epi = a.epi; p.eps = a.eps; p.norm_w = a.norm_w; p.residual = a.residual;
+    p.x_stride = a.pro >= 2 ? 2u * a.K : a.K;
+    p.pair_tile0 = tiles / 2u;
+    const uint32_t wgs = a.epi ? (tiles / 2u + best_tpw / 2u - 1u) / (best_tpw / 2u) : (tiles + best_tpw - 1u) / best_tpw;
+    if (a.pro == 1) {
+        if (q6_wide) return launch_mtile_one<MT_TYPE_Q6K_WIDE, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
+        if (q6) return launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
+        if (q5) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
+        return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
+    }
+    if (a.pro != 0) {
+        // (the 16-slot Q6_K kernel has no registers for a second operand: mtile_fused_supported declines)
+        if (q6) return launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16, true, 2>(p, wgs, 1, s, best_splits);
+        if (q5) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true, 2>(p, wgs, 1, s, best_splits);
+        return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true, 2>(p, wgs, 1, s, best_splits);
+    }
+    if (q6_wide) return launch_mtile_one<MT_TYPE_Q6K_WIDE, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
+    if (q6) return launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
+    if (q5) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
+    return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
 }
 
 }  // namespace kq

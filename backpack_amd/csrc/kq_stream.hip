@@ -526,7 +526,7 @@ bool gemv_stream_supported(const MatmulArgs& a)
     // grouped calls: M counts (token, slot) pairs, each a matvec of its own
     if (!a.expert_idx && (a.M < 1 || a.M > 4)) return false;
     // three and four tokens: plain calls, rows of at most 56 superblocks
-    if (!a.expert_idx && a.M > 2 && (a.n_blocks > 56 || a.pro != 0 || a.residual)) return false;
+    if (!a.expert_idx && a.M > 2 && (a.n_blocks > 56 || a.pro != 0 || a.residual || a.epi)) return false;
     if (a.expert_idx && (a.M < 1 || a.M > 65535u || a.bias)) return false;
     if (((uintptr_t)a.X & 15u)) return false;
     if (a.n_blocks < 1) return false;

@@ -221,9 +221,11 @@ BPK_API int bpk_kq_matmul(int type, const float *X, const void *W,
  * 0.044715 g^3))).  residual may be NULL (= zeros) and may be Y itself (the
  * in-place add).  M <= 2 with rows the decode kernel holds in registers
  * (K <= 28672 for one token, K <= 14336 for two; N <= 32768) is one launch
- * and needs no workspace.  Other shapes run the same function as prologue,
- * matmul and add launches through `workspace` (device memory, 16-byte aligned,
- * at least bpk_kq_matmul_fused_workspace_bytes(M, N, K) bytes) and fail with
+ * and needs no workspace; so are verify batches, M <= 16, on the tile kernel
+ * (X, W and norm_w 16-byte aligned; not Q6_K with M > 8 under an act * up
+ * prologue).  Other shapes run the same function as prologue, matmul and add
+ * launches through `workspace` (device memory, 16-byte aligned, at least
+ * bpk_kq_matmul_fused_workspace_bytes(M, N, K) bytes) and fail with
  * BPK_ERR_WORKSPACE without it.
  *
  * Epilogue BPK_EPI_SILU_MUL / BPK_EPI_GELU_MUL folds the same activation into
@@ -232,7 +234,8 @@ BPK_API int bpk_kq_matmul(int type, const float *X, const void *W,
  *   Y[m*N + y_offset + n] = act(bias[n] + gate_n . x[m]) * (bias[N+n] + up_n . x[m])
  * so the 2N-float gate|up buffer is never written (the down matvec then takes
  * Y as a plain X).  bias is f32 [2N] or NULL; residual must be NULL.  One launch
- * for Q4_K / Q5_K with M <= 2; other shapes go through the workspace. */
+ * for Q4_K / Q5_K with M <= 2, and for every type with M <= 16 when N is a
+ * multiple of 16; other shapes go through the workspace. */
 enum { BPK_PRO_NONE = 0, BPK_PRO_RMS_NORM = 1, BPK_PRO_SILU_MUL = 2, BPK_PRO_GELU_MUL = 3 };
 enum { BPK_EPI_NONE = 0, BPK_EPI_SILU_MUL = 2, BPK_EPI_GELU_MUL = 3 };
 

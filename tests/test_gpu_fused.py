@@ -99,12 +99,65 @@ def test_fused_residual_in_place_and_same_as_separate_launches(gpu, kqo):
     assert float((y - y2).abs().max()) <= 2e-5 * scale
 
 
+# verify batches (and one or two tokens the decode kernel declines): one launch of the tile kernel
+TILE_FUSED = [
+    # type, M, N, K, prologue, residual, bias
+    (Q4_K, 1, 60, 32768, SILU, True, False),     # rows longer than the decode kernel's K slices hold
+    (Q4_K, 5, 96, 2048, NORM, True, False),
+    (Q6_K, 16, 64, 1024, NORM, False, False),    # 16 tokens: the Q6_K kernel with 16 token slots
+    (Q6_K, 8, 64, 1024, GELU, False, False),
+    (Q6_K, 2, 48, 28672, NORM, True, False),     # the two-token long-row decode kernel carries no norm
+    (Q4_K, 3, 40, 512, NONE, True, False),
+    (Q4_K, 4, 4096, 4096, NORM, False, False),   # norm -> q at its real shape: K cut over workgroups
+    (Q4_K, 8, 4096, 4096, NONE, True, True),     # o + residual
+    (Q4_K, 16, 6144, 4096, NORM, False, True),   # norm -> q|k|v
+    (Q6_K, 4, 4096, 14336, SILU, True, False),   # act -> down -> residual, the FFN tail at its real shape
+    (Q6_K, 8, 4096, 14336, SILU, True, False),
+    (Q6_K, 16, 4096, 14336, NONE, True, False),  # (x = the gate|up epilogue's output)
+    (Q6_K, 11, 1000, 4096, NORM, False, True),
+    (Q6_K, 13, 300, 2048, NORM, True, True),
+    (Q6_K, 7, 2000, 768, GELU, True, False),
+    (13, 6, 700, 4096, NORM, True, False),       # Q5_K
+    (13, 16, 200, 14336, SILU, True, True),
+    (Q4_K, 9, 2300, 1280, NORM, True, False),    # ragged last tile, partial last chunk
+]
+
+
+@pytest.mark.parametrize("type_,M,N,K,pro,with_res,with_bias", TILE_FUSED)
+def test_fused_tile_kernel_one_launch(gpu, kqo, type_, M, N, K, pro, with_res, with_bias):
+    """The same function as the decode forms on the 16x16 tile kernel: the prologue in its conversion of X, the
+    residual in its store.  No workspace; also checked against the three-launch path on the same inputs."""
+    from backpack_amd import capi, kquant
+    print("fused tile", type_, M, N, K, pro, with_res, with_bias, flush=True)
+    w, packed, X, norm_w, res, bias, xp = _case(gpu, kqo, type_, M, N, K, pro, with_res, with_bias, seed=M + N + K)
+    args = dict(norm_w=gpu.dev(norm_w) if norm_w is not None else None, eps=1e-5,
+                bias=gpu.dev(bias) if bias is not None else None)
+    y = kquant.matmul_fused(gpu.dev(X), w, pro, residual=gpu.dev(res) if res is not None else None,
+                            allow_workspace=False, **args)
+    assert capi.last_kernel() == "mtile_fused"
+    got = y.cpu().numpy()
+    _check(gpu, kqo, type_, got, xp, packed, N, K, res, bias, f"fused tile {type_} {M}x{N}x{K} pro={pro}")
+    if with_res:      # in place: the residual is the output buffer
+        y2 = gpu.dev(res.copy())
+        kquant.matmul_fused(gpu.dev(X), w, pro, residual=y2, out=y2, allow_workspace=False, **args)
+        assert np.array_equal(y2.cpu().numpy(), got)
+    capi.set_option("fused_separate", 1)      # prologue, matmul and add launches
+    try:
+        y3 = kquant.matmul_fused(gpu.dev(X), w, pro, residual=gpu.dev(res) if res is not None else None, **args)
+        assert capi.last_kernel() != "mtile_fused"
+    finally:
+        capi.set_option("fused_separate", 0)
+    ref = y3.cpu().numpy()
+    base = ref - res if res is not None else ref
+    scale = float(np.sqrt(np.mean(base.astype(np.float64) ** 2)))
+    assert float(np.abs(got - ref).max()) <= 5e-5 * scale + 1e-6 * float(np.abs(ref).max())
+
+
 WORKSPACE = [
-    (Q4_K, 1, 60, 32768, SILU, True),      # rows longer than the decode kernel's K slices hold
-    (Q4_K, 5, 96, 2048, NORM, True),       # more than two tokens
-    (Q6_K, 16, 64, 1024, GELU, False),
-    (Q6_K, 2, 48, 28672, NORM, True),      # the two-token long-row kernel carries no norm
-    (Q4_K, 3, 40, 512, NONE, True),
+    (Q4_K, 20, 96, 2048, NORM, True),      # more than 16 tokens
+    (Q6_K, 16, 64, 1024, GELU, False),     # Q6_K beyond 8 tokens with a two-operand prologue
+    (Q6_K, 33, 64, 1024, GELU, False),
+    (Q4_K, 17, 40, 512, NONE, True),
 ]
 
 
@@ -119,7 +172,7 @@ def test_fused_workspace_path(gpu, kqo, type_, M, N, K, pro, with_res):
         kquant.matmul_fused(gpu.dev(X), w, pro, allow_workspace=False, **args)
     assert e.value.code == -7
     y = kquant.matmul_fused(gpu.dev(X), w, pro, **args)
-    assert capi.last_kernel() != "gemv_stream_fused"
+    assert capi.last_kernel() not in ("gemv_stream_fused", "mtile_fused")
     _check(gpu, kqo, type_, y.cpu().numpy(), xp, packed, N, K, res, None, f"fused ws {type_} {M}x{N}x{K}")
 
 
@@ -152,7 +205,15 @@ EPI = [
     (13, 1, 500, 4096, SILU, NONE, False, "gemv_stream_fused"),         # Q5_K
     (Q4_K, 1, 33, 256, SILU, NONE, False, "gemv_stream_fused"),         # fewer pairs than waves
     (Q6_K, 1, 200, 2048, SILU, NONE, False, None),                      # workspace path: Q6_K gate|up
-    (Q4_K, 5, 120, 1024, GELU, NORM, True, None),                       # ... more than two tokens
+    (Q4_K, 5, 120, 1024, GELU, NORM, True, None),                       # ... more than two tokens, outputs not in tiles of 16
+    (Q4_K, 5, 128, 1024, GELU, NORM, True, "mtile_fused"),              # verify batches: gate and up tiles meet in the workgroup
+    (Q4_K, 16, 14336, 4096, SILU, NORM, False, "mtile_fused"),          # ... the FFN head at its real shape
+    (Q4_K, 4, 14336, 4096, SILU, NONE, False, "mtile_fused"),
+    (Q4_K, 8, 1040, 5376, GELU, NONE, True, "mtile_fused"),             # ... K cut over workgroups, a ragged last group
+    (Q6_K, 8, 256, 2048, SILU, NONE, True, "mtile_fused"),
+    (Q6_K, 12, 96, 1024, GELU, NORM, False, "mtile_fused"),             # ... the 16-slot Q6_K kernel
+    (13, 3, 512, 4096, SILU, NORM, False, "mtile_fused"),               # Q5_K
+    (Q6_K, 1, 208, 2048, SILU, NONE, False, "mtile_fused"),             # one token where the decode kernel has no pair mode
 ]
 
 
