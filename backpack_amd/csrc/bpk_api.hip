@@ -411,8 +411,10 @@ int bpk_weight_destroy(bpk_weight* w)
     return e == hipSuccess ? BPK_OK : hip_fail(e, "hipFree(weights)");
 }
 
-int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, float* Y, uint32_t M, uint32_t N,
-                  uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, uint32_t y_offset, void* stream)
+// fold: the greedy pick over the outputs, taken along by the launch where its kernel can (*folded says so)
+static int matmul_impl(int type, const float* X, const void* W, const float* bias, float* Y, uint32_t M, uint32_t N,
+                       uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, uint32_t y_offset, void* stream,
+                       const kq::ArgmaxFold* fold, bool* folded)
 {
     if (int rc = check_matmul(type, X, W, Y, M, N, K, n_blocks, row_stride_words)) return rc;
     if (M == 0) return BPK_OK;
@@ -461,8 +463,10 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
     const bool use_rows = rows_ok && (t_family == 2 || (t_family == 0 && (M <= 2 || !mrow_ok)));
     const bool use_mrow = mrow_ok && !use_rows && (t_family == 0 || t_family == 3);
     if (use_rows) {
-        t_kernel = "gemv_rows";
-        e = kq::launch_gemv_rows(a, st->split, t_gemv, s);
+        const bool take = fold && kq::gemv_rows_can_fold(a, *fold);
+        t_kernel = take ? "gemv_rows_argmax" : "gemv_rows";
+        e = kq::launch_gemv_rows(a, st->split, t_gemv, s, take ? fold : nullptr);
+        if (take && e == hipSuccess) *folded = true;
     } else if (use_mrow) {
         t_kernel = "mrow";
         e = kq::launch_mrow(a, st->split, t_gemv, nullptr, nullptr, 1, 0, s);
@@ -471,6 +475,12 @@ int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, fl
         e = kq::launch_matmul_generic(a, s);
     }
     return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+}
+
+int bpk_kq_matmul(int type, const float* X, const void* W, const float* bias, float* Y, uint32_t M, uint32_t N,
+                  uint32_t K, uint32_t n_blocks, uint32_t row_stride_words, uint32_t y_offset, void* stream)
+{
+    return matmul_impl(type, X, W, bias, Y, M, N, K, n_blocks, row_stride_words, y_offset, stream, nullptr, nullptr);
 }
 
 size_t bpk_kq_matmul_fused_workspace_bytes(uint32_t M, uint32_t N, uint32_t K)
@@ -935,7 +945,16 @@ int bpk_kq_matmul_argmax(int type, const float* X, const void* W, const float* b
                          float* out_val, void* stream)
 {
     if (!out_idx) return fail(BPK_ERR_NULL, "out_idx must be non-null");
-    if (int rc = bpk_kq_matmul(type, X, W, bias, logits, M, N, K, n_blocks, row_stride_words, 0, stream)) return rc;
+    DeviceState* st;
+    if (int rc = current_state(&st)) return rc;
+    // the row-per-lane kernel (one or two tokens over a vocabulary-sized Q6_K matrix) picks as it stores;
+    // other launches are followed by the pick as a launch of its own
+    const uint32_t cells = kq::ARGMAX_MAX_ROWS * kq::ARGMAX_PARTS;
+    const kq::ArgmaxFold fold{out_idx, out_val, (float*)st->argmax_scratch, st->argmax_scratch + cells,
+                              st->argmax_scratch + 2u * (size_t)cells, cells};
+    bool folded = false;
+    if (int rc = matmul_impl(type, X, W, bias, logits, M, N, K, n_blocks, row_stride_words, 0, stream, &fold, &folded)) return rc;
+    if (folded || M == 0) return BPK_OK;
     return bpk_argmax_rows(logits, M, N, N, out_idx, out_val, stream);
 }
 

@@ -22,6 +22,7 @@
 // group) adds them in split order, so results do not depend on scheduling.
 #include "kq_format.h"
 #include "kq_kernels.h"
+#include "kq_wave.h"
 
 namespace kq {
 
@@ -62,6 +63,7 @@ struct GemvParams {
     uint32_t blocks_per_split, n_splits;
     float* partial;       // [n_splits][MT][groups*64]
     uint32_t* counters;   // [groups], zero between launches
+    ArgmaxFold am;        // am.out_idx != nullptr: the greedy pick over the outputs rides along
 };
 
 // Sums of X over every aligned run of SEG elements of the workgroup's K range,
@@ -138,12 +140,62 @@ __device__ __forceinline__ void finish_rows(const GemvParams& p, float (&acc)[MT
         if (lane == 0)
             __hip_atomic_store(&p.counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    const float b = (row < p.N && p.bias) ? p.bias[row] : 0.0f;
     if (row < p.N) {
-        const float b = p.bias ? p.bias[row] : 0.0f;
 #pragma unroll
         for (int m = 0; m < MT; ++m)
             if ((uint32_t)m < p.M) p.Y[(size_t)m * p.ldy + p.y_offset + row] = tot[m] + b;
     }
+    if (!p.am.out_idx) return;
+    // The greedy pick (argmax + argmax_reduce behind lm_head, runtime/model_runner.cpp:2441-2453): this wave's
+    // best per token goes out as a partial, the last workgroup to take the ticket reduces them all.
+    const uint32_t groups = gridDim.x;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        if ((uint32_t)m >= p.M) break;
+        float v = tot[m] + b;
+        uint32_t i = row;
+        if (!(row < p.N && v > -1e30f)) { v = -1e30f; i = 0xFFFFFFFFu; }   // "none": any real index is lower
+        wave_best(v, i);
+        if (lane == 0) {
+            __hip_atomic_store(&p.am.part_val[(size_t)m * groups + blockIdx.x], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&p.am.part_idx[(size_t)m * groups + blockIdx.x], i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    // (as in the fold above: write-through stores acknowledged before the ticket, agent-scope loads by the last
+    // arriver; no fence, which would write back and invalidate the XCD's L2 once per workgroup)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    uint32_t ticket = 0;
+    if (lane == 0)
+        ticket = __hip_atomic_fetch_add(p.am.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ticket = __builtin_amdgcn_readfirstlane(ticket);
+    if (ticket != groups - 1u) return;
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        if ((uint32_t)m >= p.M) break;
+        float v = -1e30f;
+        uint32_t i = 0xFFFFFFFFu;
+        // eight partials per lane in flight at a time (each load travels past the non-coherent cache levels)
+        for (uint32_t q0 = lane; q0 < groups; q0 += 8u * 64u) {
+            float pv[8];
+            uint32_t pi[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const uint32_t q = min(q0 + 64u * (uint32_t)u, groups - 1u);   // (a repeated partial changes nothing)
+                pv[u] = __hip_atomic_load(&p.am.part_val[(size_t)m * groups + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                pi[u] = __hip_atomic_load(&p.am.part_idx[(size_t)m * groups + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) best_of(v, i, pv[u], pi[u]);
+        }
+        wave_best(v, i);
+        if (lane == 0) {
+            p.am.out_idx[m] = i == 0xFFFFFFFFu ? 0 : (int32_t)i;
+            if (p.am.out_val) p.am.out_val[m] = v;
+        }
+    }
+    if (lane == 0) __hip_atomic_store(p.am.ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // re-armed
 }
 
 // ---------------------------------------------------------------------------
@@ -512,10 +564,22 @@ static hipError_t launch_mt(const GemvParams& p, hipStream_t s)
     }
 }
 
-hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const GemvTuning& t, hipStream_t s)
+bool gemv_rows_can_fold(const MatmulArgs& a, const ArgmaxFold& f)
+{
+    // one partial per token and group of 64 rows; the kernels hold up to four tokens
+    return a.M >= 1 && a.M <= 4 && a.y_offset == 0 && (uint64_t)a.M * ((a.N + 63u) / 64u) <= f.cells;
+}
+
+hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const GemvTuning& t, hipStream_t s,
+                            const ArgmaxFold* fold)
 {
     const GemvPlan pl = plan_gemv(a, t);
     GemvParams p;
+    p.am = ArgmaxFold{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+    if (fold) {
+        if (!gemv_rows_can_fold(a, *fold)) return hipErrorInvalidValue;
+        p.am = *fold;
+    }
     p.X = (const float*)a.X;
     p.W = a.W;
     p.bias = a.bias;

@@ -92,8 +92,21 @@ struct GemvTuning {
 };
 bool gemv_rows_supported(const MatmulArgs& a);
 size_t gemv_rows_scratch_floats(const MatmulArgs& a, const GemvTuning& t);
+// The greedy pick folded into a matvec launch: every workgroup leaves the best (value, index) of the outputs it
+// stored, per token, in part_val / part_idx[token * groups + group]; the last one to take the ticket reduces them
+// into out_idx / out_val (lowest index among equal maxima, index 0 when nothing exceeds -1e30) and re-arms
+// the ticket.  cells: capacity of the partial arrays.
+struct ArgmaxFold {
+    int32_t* out_idx;
+    float* out_val;       // may be null
+    float* part_val;
+    uint32_t* part_idx;
+    uint32_t* ticket;     // zero between launches
+    uint32_t cells;
+};
+bool gemv_rows_can_fold(const MatmulArgs& a, const ArgmaxFold& f);
 hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const GemvTuning& t,
-                            hipStream_t s);
+                            hipStream_t s, const ArgmaxFold* fold = nullptr);
 
 // Lanes-along-K decode GEMV (M = 1): a wave owns whole rows, activations stay
 // in registers.  t.splits, when set, overrides the rows per wave.

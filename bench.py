@@ -433,16 +433,25 @@ def fused_leg(mats, use_graph):
     res["chain_ms"] = round(timed(chain_pass), 4)
     ch.status()
     res["chain_launches"] = len(cuts)
-    # the greedy pick behind lm_head: one launch over the 128256 logits, timed in a graph of 50
-    logits = next(y for n_, _, _, y in mats if n_ == "lm_head")
+    # the greedy pick behind lm_head rides in the lm_head launch (bpk_kq_matmul_argmax): the launch with and
+    # without it, graphs of 20 over the layer set's lm_head
+    _, w_lm, x_lm, logits = next(m for m in mats if m[0] == "lm_head")
     idx = torch.empty(1, dtype=torch.int32, device="cuda")
     val = torch.empty(1, dtype=torch.float32, device="cuda")
+    stream = lambda: torch.cuda.current_stream().cuda_stream
 
-    def picks():
-        for _ in range(50):
-            capi.check(capi.lib().bpk_argmax_rows(logits.data_ptr(), 1, logits.shape[1], logits.shape[1], idx.data_ptr(),
-                                                  val.data_ptr(), torch.cuda.current_stream().cuda_stream))
-    res["argmax_us"] = round(timed(picks) * 1e3 / 50, 2)
+    def lm_plain():
+        for _ in range(20):
+            kquant.matmul(x_lm, w_lm, out=logits)
+
+    def lm_pick():
+        for _ in range(20):
+            capi.check(capi.lib().bpk_kq_matmul_argmax(w_lm.type, x_lm.data_ptr(), w_lm.data.data_ptr(), None, logits.data_ptr(),
+                                                       1, w_lm.N, w_lm.K, w_lm.n_blocks, w_lm.row_stride_words,
+                                                       idx.data_ptr(), val.data_ptr(), stream()))
+    res["lm_head_us"] = round(timed(lm_plain) * 1e3 / 20, 2)
+    res["lm_head_with_pick_us"] = round(timed(lm_pick) * 1e3 / 20, 2)
+    res["pick"] = capi.last_kernel()
     n = sum(1 for name, *_ in mats if name == "qkv")
     res["launches_saved"] = 5 * n     # per layer: two norms, act*mul, two residual adds
     return res

@@ -66,3 +66,48 @@ def test_lm_head_with_argmax(gpu, kqo):
         top2 = np.sort(ref, axis=1)[:, -2:]
         clear = (top2[:, 1] - top2[:, 0]) > 1e-3 * np.abs(top2[:, 1])
         assert np.array_equal(idx.cpu().numpy()[clear], kqo.argmax_rows(ref)[clear])
+
+
+def test_lm_head_pick_inside_the_matvec_launch(gpu, kqo):
+    """One token over a vocabulary-sized Q6_K matrix: the row kernel leaves a partial pick per workgroup and
+    its last workgroup reduces them.  Equal maxima (two identical weight rows), a repeated call (the ticket
+    is re-armed), a bias, nothing above -1e30, and the same pick as the separate launch."""
+    import torch
+    from backpack_amd import capi, kquant
+    N, K = 40000, 2048      # rows of 8 blocks: 16-byte aligned, as the row kernel wants them
+    raw, packed, w = gpu.make_weight(Q6_K, N, K, seed=9)
+    rows = w.data[: N * w.row_stride_bytes].view(N, w.row_stride_bytes)
+    rows[31007] = rows[977]                       # identical rows: identical logits
+    rows[39999] = rows[977]                       # ... and the last row of the last workgroup
+    X = np.random.default_rng(3).standard_normal((1, K)).astype(np.float32)
+    bias = np.zeros(N, np.float32)
+    bias[[977, 31007, 39999]] = 1e4               # lift the three above everything else
+    for rep in range(3):
+        logits, idx, val = kquant.matmul_argmax(gpu.dev(X), w, bias=gpu.dev(bias))
+        assert capi.last_kernel() == "gemv_rows_argmax"
+        lg = logits.cpu().numpy()
+        assert lg[0, 977] == lg[0, 31007] == lg[0, 39999]
+        assert int(idx[0]) == 977 and float(val[0]) == lg[0, 977]
+    # plain logits: the separate launch agrees
+    logits, idx, val = kquant.matmul_argmax(gpu.dev(X), w)
+    idx2, val2 = kquant.argmax_rows(logits)
+    assert int(idx[0]) == int(idx2[0]) and float(val[0]) == float(val2[0])
+    assert np.array_equal(idx.cpu().numpy(), kqo.argmax_rows(logits.cpu().numpy()))
+    # nothing above -1e30: index 0, as the reference's scan from best = -1e30 leaves it
+    low = gpu.dev(np.full(N, -3e30, np.float32))
+    logits, idx, val = kquant.matmul_argmax(gpu.dev(X), w, bias=low)
+    assert int(idx[0]) == 0 and float(val[0]) == np.float32(-1e30)
+    # two tokens go to another kernel family and are followed by the pick's own launch
+    X2 = np.random.default_rng(4).standard_normal((2, K)).astype(np.float32)
+    logits, idx, val = kquant.matmul_argmax(gpu.dev(X2), w)
+    assert capi.last_kernel() != "gemv_rows_argmax"
+    assert np.array_equal(idx.cpu().numpy(), kqo.argmax_rows(logits.cpu().numpy()))
+    # forced onto the row kernel, two tokens are picked inside the launch as well
+    capi.force_kernel(2)
+    try:
+        l2, i2, v2 = kquant.matmul_argmax(gpu.dev(X2), w)
+        assert capi.last_kernel() == "gemv_rows_argmax"
+    finally:
+        capi.force_kernel(0)
+    assert np.array_equal(i2.cpu().numpy(), kqo.argmax_rows(l2.cpu().numpy()))
+    assert np.array_equal(v2.cpu().numpy(), l2.cpu().numpy().max(axis=1))
