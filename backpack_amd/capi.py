@@ -50,6 +50,23 @@ class GgufTensor(C.Structure):
                 ("offset", C.c_uint64), ("bytes", C.c_uint64), ("data", C.c_void_p)]
 
 
+class ModelConfig(C.Structure):
+    """bpk_model_config: the reference's ModelConfig (runtime/gguf_loader.h:164-218) as a flat record."""
+    _fields_ = [("arch", C.c_char * 64),
+                ("n_layer", C.c_uint32), ("n_head", C.c_uint32), ("n_kv_heads", C.c_uint32), ("n_embd", C.c_uint32),
+                ("intermediate_size", C.c_uint32), ("n_vocab", C.c_uint32), ("head_dim", C.c_uint32),
+                ("kv_head_dim", C.c_uint32), ("rms_norm_eps", C.c_float), ("rope_theta", C.c_float),
+                ("tie_word_embeddings", C.c_int), ("has_qk_norm", C.c_int), ("activation", C.c_int),
+                ("embedding_scale", C.c_float), ("logit_softcap", C.c_float), ("sliding_window", C.c_uint32),
+                ("n_layer_attn_types", C.c_uint32), ("has_sandwich_norm", C.c_int), ("ple_size", C.c_uint32),
+                ("shared_kv_layers", C.c_uint32), ("has_mtp", C.c_int), ("mtp_num_layers", C.c_uint32),
+                ("num_experts", C.c_uint32), ("num_experts_per_tok", C.c_uint32), ("moe_intermediate_size", C.c_uint32),
+                ("moe_shared_intermediate_size", C.c_uint32), ("ssm_inner_size", C.c_uint32),
+                ("ssm_state_size", C.c_uint32), ("ssm_conv_kernel", C.c_uint32), ("ssm_group_count", C.c_uint32),
+                ("ssm_time_step_rank", C.c_uint32), ("full_attention_interval", C.c_uint32),
+                ("rope_sections", C.c_int32 * 4)]
+
+
 _SIGS = {
     "bpk_version": (C.c_int, []),
     "bpk_last_error": (C.c_char_p, []),
@@ -79,6 +96,7 @@ _SIGS = {
     "bpk_gguf_array_len": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)]),
     "bpk_gguf_array_string": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_void_p, C.c_size_t,
                                         C.POINTER(C.c_size_t)]),
+    "bpk_gguf_model_config": (C.c_int, [C.c_void_p, C.POINTER(ModelConfig), C.c_void_p, C.c_uint32]),
     "bpk_gguf_array_data": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_uint64),
                                       C.POINTER(C.c_uint32)]),
     "bpk_gguf_weight_create": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.c_uint32, C.POINTER(C.c_void_p)]),

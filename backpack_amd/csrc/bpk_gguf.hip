@@ -478,6 +478,101 @@ int bpk_gguf_array_string(const bpk_gguf* g, const char* key, uint64_t index, ch
 // (q|k|v, gate|up).  All parts must share the type and K.
 static int gguf_weight_create_body(const bpk_gguf* g, const char* const* names, uint32_t n_names, bpk_weight** out);
 
+// Model hyper-parameters from the metadata and the tensor directory (extractModelConfig,
+// runtime/gguf_loader.cpp:184-317): the same keys, defaults and probes.
+static int model_config_body(const bpk_gguf* g, bpk_model_config* c, uint8_t* layer_types, uint32_t cap)
+{
+    memset(c, 0, sizeof(*c));
+    std::string a = "llama";
+    if (const MetaValue* v = find_meta(g, "general.architecture"); v && v->type == META_STRING) a.assign(v->str, (size_t)v->len);
+    snprintf(c->arch, sizeof(c->arch), "%s", a.c_str());
+    auto u32 = [&](const std::string& key, uint32_t def = 0) {
+        uint32_t x = def;
+        bpk_gguf_get_u32(g, key.c_str(), def, &x);
+        return x;
+    };
+    auto f32 = [&](const std::string& key, float def) {
+        float x = def;
+        bpk_gguf_get_f32(g, key.c_str(), def, &x);
+        return x;
+    };
+    auto has_tensor = [&](const std::string& name) { return g->index.count(name) > 0; };
+    c->n_layer = u32(a + ".block_count");
+    c->n_embd = u32(a + ".embedding_length");
+    c->intermediate_size = u32(a + ".feed_forward_length");
+    c->n_head = u32(a + ".attention.head_count");
+    c->n_kv_heads = u32(a + ".attention.head_count_kv", c->n_head);
+    c->rms_norm_eps = f32(a + ".attention.layer_norm_rms_epsilon", 1e-6f);
+    c->rope_theta = f32(a + ".rope.freq_base", 1000000.0f);
+    c->tie_word_embeddings = find_meta(g, "output.weight") ? 0 : 1;   // (a metadata key of that name, as the reference asks)
+    // attention.key_length is the head width where rotary embedding covers only part of it
+    const uint32_t dense_head = c->n_head ? c->n_embd / c->n_head : 0;
+    c->kv_head_dim = u32(a + ".attention.key_length", dense_head);
+    c->head_dim = c->kv_head_dim ? c->kv_head_dim : dense_head;
+    if (auto it = g->index.find("token_embd.weight"); it != g->index.end()) {
+        const Tensor& t = g->tensors[it->second];
+        c->n_vocab = (uint32_t)(t.n_dims >= 2 ? t.dims[1] : t.dims[0]);   // GGUF shapes are (columns, rows)
+    }
+    c->has_qk_norm = has_tensor("blk.0.attn_q_norm.weight");
+    for (uint32_t i = 1; i < c->n_layer && !c->has_qk_norm; ++i)   // hybrids carry it on their attention layers only
+        c->has_qk_norm = has_tensor("blk." + std::to_string(i) + ".attn_q_norm.weight");
+    const bool gemma = a == "gemma" || a == "gemma2" || a == "gemma3" || a == "gemma4";
+    c->activation = gemma ? BPK_ACT_GELU : BPK_ACT_SILU;
+    c->embedding_scale = gemma ? sqrtf((float)c->n_embd) : 0.0f;
+    c->logit_softcap = f32(a + ".final_logit_softcapping", 0.0f);
+    c->sliding_window = u32(a + ".attention.sliding_window");
+    // per-layer attention kinds: 0 = global, 1 = sliding window
+    c->n_layer_attn_types = c->sliding_window > 0 && c->n_layer > 0 ? c->n_layer : 0;
+    if (layer_types && c->n_layer_attn_types) {
+        if (cap < c->n_layer) return fail(BPK_ERR_SHAPE, "layer_types holds %u entries, the model has %u layers", cap, c->n_layer);
+        const MetaValue* pat = find_meta(g, (a + ".attention.sliding_window_pattern").c_str());
+        const bool use_pat = a == "gemma4" && pat && pat->type == META_ARRAY && pat->elem_type == META_BOOL && pat->arr &&
+                             pat->len == c->n_layer;
+        for (uint32_t i = 0; i < c->n_layer; ++i) {
+            uint8_t t = 0;
+            if (a == "gemma2") t = i % 2 == 0;                         // even layers slide
+            else if (a == "gemma3") t = (i + 1) % 6 != 0;              // five sliding, one global
+            else if (a == "gemma4") t = use_pat ? pat->arr[i] != 0 : (i + 1) % 6 != 0;
+            layer_types[i] = t;
+        }
+    }
+    c->shared_kv_layers = u32(a + ".attention.shared_kv_layers");
+    c->ple_size = u32(a + ".embedding_length_per_layer_input");
+    c->has_sandwich_norm = has_tensor("blk.0.post_norm.weight") || has_tensor("blk.0.attn_post_norm.weight") ||
+                           has_tensor("blk.0.post_attention_norm.weight");
+    c->has_mtp = has_tensor("mtp.0.blk.0.attn_q.weight") || has_tensor("mtp.0.enorm.weight");
+    if (!c->has_mtp) {
+        const uint32_t nextn = u32(a + ".nextn_predict_layers");
+        if (nextn > 0) { c->has_mtp = 1; c->mtp_num_layers = nextn; }
+    }
+    c->num_experts = u32(a + ".expert_count");
+    c->num_experts_per_tok = u32(a + ".expert_used_count");
+    c->moe_intermediate_size = u32(a + ".expert_feed_forward_length");
+    c->moe_shared_intermediate_size = u32(a + ".expert_shared_feed_forward_length", c->moe_intermediate_size);
+    c->ssm_inner_size = u32(a + ".ssm.inner_size");
+    c->ssm_state_size = u32(a + ".ssm.state_size");
+    c->ssm_conv_kernel = u32(a + ".ssm.conv_kernel");
+    c->ssm_group_count = u32(a + ".ssm.group_count");
+    c->ssm_time_step_rank = u32(a + ".ssm.time_step_rank");
+    c->full_attention_interval = u32(a + ".full_attention_interval");
+    const int32_t sections[4] = {11, 11, 10, 0};
+    memcpy(c->rope_sections, sections, sizeof(sections));
+    const MetaValue* rs = find_meta(g, (a + ".rope.dimension_sections").c_str());
+    if (rs && rs->type == META_ARRAY && (rs->elem_type == META_INT32 || rs->elem_type == META_UINT32) && rs->arr && rs->len >= 4)
+        memcpy(c->rope_sections, rs->arr, 16);
+    return BPK_OK;
+}
+
+int bpk_gguf_model_config(const bpk_gguf* g, bpk_model_config* out, uint8_t* layer_types, uint32_t layer_types_cap)
+{
+    if (!g || !out) return fail(BPK_ERR_NULL, "file and out must be non-null");
+    try {
+        return model_config_body(g, out, layer_types, layer_types_cap);
+    } catch (const std::exception&) {
+        return fail(BPK_ERR_IO, "out of memory while reading the model configuration");
+    }
+}
+
 int bpk_gguf_weight_create(const bpk_gguf* g, const char* const* names, uint32_t n_names, bpk_weight** out)
 {
     try {

@@ -138,6 +138,22 @@ class GGUFFile:
             out.append(buf.raw[: ln.value].decode("utf-8", errors="replace"))
         return out
 
+    def model_config(self) -> dict:
+        """The model's hyper-parameters (extractModelConfig, runtime/gguf_loader.cpp:184-317) as a dict;
+        'layer_attn_types' lists 0 (global) / 1 (sliding window) per layer, empty without a sliding window."""
+        c = capi.ModelConfig()
+        L = capi.lib()
+        capi.check(L.bpk_gguf_model_config(self.handle, C.byref(c), None, 0))
+        types = (C.c_uint8 * max(1, c.n_layer_attn_types))()
+        if c.n_layer_attn_types:
+            capi.check(L.bpk_gguf_model_config(self.handle, C.byref(c), types, c.n_layer_attn_types))
+        out = {}
+        for name, _ in capi.ModelConfig._fields_:
+            v = getattr(c, name)
+            out[name] = v.decode() if name == "arch" else list(v) if name == "rope_sections" else v
+        out["layer_attn_types"] = list(types)[: c.n_layer_attn_types]
+        return out
+
     def get_array(self, key: str) -> np.ndarray:
         """Fixed-size-element array as a numpy copy (empty when absent or an array of strings)."""
         p, n, et = C.c_void_p(), C.c_uint64(), C.c_uint32()

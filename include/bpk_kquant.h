@@ -170,6 +170,38 @@ BPK_API int bpk_gguf_array_data(const bpk_gguf *g, const char *key,
                                 const void **data, uint64_t *n,
                                 uint32_t *elem_type);
 
+/* Model hyper-parameters (extractModelConfig, runtime/gguf_loader.cpp:184-317;
+ * ModelConfig, runtime/gguf_loader.h:164-218): the reference's keys under
+ * "<general.architecture>.", its defaults, and its probes of the tensor
+ * directory (vocabulary from token_embd.weight, QK norm, sandwich norm, MTP).
+ * layer_types (may be NULL) receives n_layer_attn_types entries, 0 = global
+ * attention, 1 = sliding window (Gemma 2 / 3 / 4 patterns); cap is its size. */
+enum { BPK_ACT_SILU = 0, BPK_ACT_GELU = 1 };
+typedef struct bpk_model_config {
+    char arch[64];
+    uint32_t n_layer, n_head, n_kv_heads, n_embd, intermediate_size, n_vocab;
+    uint32_t head_dim, kv_head_dim;
+    float rms_norm_eps, rope_theta;
+    int tie_word_embeddings, has_qk_norm;
+    int activation;                 /* BPK_ACT_*                                */
+    float embedding_scale;          /* sqrt(n_embd) for the Gemma family, else 0 */
+    float logit_softcap;
+    uint32_t sliding_window;
+    uint32_t n_layer_attn_types;    /* n_layer when sliding_window > 0, else 0  */
+    int has_sandwich_norm;
+    uint32_t ple_size, shared_kv_layers;
+    int has_mtp;
+    uint32_t mtp_num_layers;
+    uint32_t num_experts, num_experts_per_tok, moe_intermediate_size,
+        moe_shared_intermediate_size;
+    uint32_t ssm_inner_size, ssm_state_size, ssm_conv_kernel, ssm_group_count,
+        ssm_time_step_rank, full_attention_interval;
+    int32_t rope_sections[4];       /* default 11, 11, 10, 0                    */
+} bpk_model_config;
+BPK_API int bpk_gguf_model_config(const bpk_gguf *g, bpk_model_config *out,
+                                  uint8_t *layer_types,
+                                  uint32_t layer_types_cap);
+
 /* Named Q4_K / Q6_K matrices of the file (GGUF shape {K, N}) -> one device
  * weight with the rows stacked in the order given: the tensor -> packKQ ->
  * fuseKQ -> uploadKQWeight sequence of runtime/model_runner.cpp:1275-1338

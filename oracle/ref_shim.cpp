@@ -149,4 +149,29 @@ int64_t bpref_gguf_i32_array(const void* h, const char* key, int32_t* out, uint6
     return (int64_t)a->size();
 }
 
+// extractModelConfig(file) as flat arrays: u[28] in the order of the assignments below, f[4], the four rope
+// sections, the architecture name and, per layer, 1 for a sliding-window layer (count returned).
+uint32_t bpref_model_config(const void* h, uint32_t* u, float* f, int32_t* sections, uint8_t* layer_types, uint32_t cap,
+                            char* arch, size_t arch_cap)
+{
+    const ModelConfig c = extractModelConfig(*(const GGUFFile*)h);
+    const uint32_t vals[28] = {c.nLayer, c.nHead, c.nKvHeads, c.nEmbd, c.intermediateSize, c.nVocab, c.headDim, c.kvHeadDim,
+                               c.tieWordEmbeddings, c.hasQkNorm, c.activation == ActivationType::GELU, c.slidingWindow,
+                               (uint32_t)c.layerAttnTypes.size(), c.hasSandwichNorm, c.pleSize, c.sharedKvLayers, c.hasMtp,
+                               c.mtpNumLayers, c.numExperts, c.numExpertsPerTok, c.moeIntermediateSize,
+                               c.moeSharedIntermediateSize, c.ssmInnerSize, c.ssmStateSize, c.ssmConvKernel, c.ssmGroupCount,
+                               c.ssmTimeStepRank, c.fullAttentionInterval};
+    std::memcpy(u, vals, sizeof(vals));
+    f[0] = c.rmsNormEps; f[1] = c.ropeTheta; f[2] = c.embeddingScale; f[3] = c.logitSoftcap;
+    for (int i = 0; i < 4; i++) sections[i] = i < (int)c.ropeSections.size() ? c.ropeSections[i] : 0;
+    for (uint32_t i = 0; i < c.layerAttnTypes.size() && i < cap; i++)
+        layer_types[i] = c.layerAttnTypes[i] == AttnLayerType::SlidingWindow;
+    if (arch_cap) {
+        const size_t n = c.arch.size() < arch_cap - 1 ? c.arch.size() : arch_cap - 1;
+        std::memcpy(arch, c.arch.data(), n);
+        arch[n] = 0;
+    }
+    return (uint32_t)c.layerAttnTypes.size();
+}
+
 }  // extern "C"

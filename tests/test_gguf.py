@@ -336,3 +336,179 @@ def test_weight_create_argument_checks(tmp_path):
         assert L.bpk_gguf_weight_create(g.handle, None, 1, C.byref(w)) == -3
         arr = (C.c_char_p * 1)(b"blk.0.ffn_gate.weight")
         assert L.bpk_gguf_weight_create(g.handle, arr, 0, C.byref(w)) == -2
+
+
+# ---- model hyper-parameters (extractModelConfig, runtime/gguf_loader.cpp:184-317) --------------------
+def _cfg_file(tmp_path, name, metadata, tensor_names=(), embd_dims=None):
+    tensors = [(n, (4,), 0, np.zeros(4, np.float32).tobytes()) for n in tensor_names]
+    if embd_dims:
+        n = int(np.prod(embd_dims))
+        tensors.append(("token_embd.weight", embd_dims, 0, np.zeros(n, np.float32).tobytes()))
+    path = os.path.join(tmp_path, name)
+    gw.write(path, metadata, tensors)
+    return path
+
+
+def test_model_config_llama_defaults_and_probes(tmp_path):
+    """A plain Llama file: keys under 'llama.', the reference's defaults for what the file leaves out."""
+    md = [("general.architecture", gw.STRING, "llama"), ("llama.block_count", gw.U32, 32),
+          ("llama.embedding_length", gw.U32, 4096), ("llama.feed_forward_length", gw.U32, 14336),
+          ("llama.attention.head_count", gw.U32, 32), ("llama.attention.head_count_kv", gw.U32, 8),
+          ("llama.attention.layer_norm_rms_epsilon", gw.F32, 1e-5), ("llama.rope.freq_base", gw.F32, 500000.0)]
+    with GGUFFile(_cfg_file(str(tmp_path), "llama.gguf", md, embd_dims=(64, 1000))) as f:
+        c = f.model_config()
+    assert c["arch"] == "llama"
+    assert (c["n_layer"], c["n_embd"], c["intermediate_size"], c["n_head"], c["n_kv_heads"]) == (32, 4096, 14336, 32, 8)
+    assert (c["head_dim"], c["kv_head_dim"]) == (128, 128)                       # n_embd / n_head
+    assert c["n_vocab"] == 1000                                                  # GGUF shape is (columns, rows)
+    assert c["rms_norm_eps"] == np.float32(1e-5) and c["rope_theta"] == 500000.0
+    assert c["tie_word_embeddings"] == 1 and c["has_qk_norm"] == 0
+    assert c["activation"] == 0 and c["embedding_scale"] == 0.0 and c["logit_softcap"] == 0.0
+    assert c["sliding_window"] == 0 and c["layer_attn_types"] == []
+    assert (c["num_experts"], c["num_experts_per_tok"], c["moe_intermediate_size"]) == (0, 0, 0)
+    assert c["has_mtp"] == 0 and c["has_sandwich_norm"] == 0
+    assert c["rope_sections"] == [11, 11, 10, 0]
+
+
+def test_model_config_missing_architecture_and_fallbacks(tmp_path):
+    """No architecture key: 'llama'; kv heads default to heads, eps 1e-6, theta 1e6; a 1-D embedding."""
+    md = [("llama.block_count", gw.U32, 2), ("llama.embedding_length", gw.U32, 512),
+          ("llama.attention.head_count", gw.U32, 8), ("output.weight", gw.BOOL, 1)]
+    path = os.path.join(str(tmp_path), "bare.gguf")
+    gw.write(path, md, [("token_embd.weight", (77,), 0, np.zeros(77, np.float32).tobytes())])
+    with GGUFFile(path) as f:
+        c = f.model_config()
+    assert c["arch"] == "llama" and c["n_kv_heads"] == 8 and c["head_dim"] == 64
+    assert c["rms_norm_eps"] == np.float32(1e-6) and c["rope_theta"] == 1000000.0
+    assert c["n_vocab"] == 77
+    assert c["tie_word_embeddings"] == 0          # the reference asks for a metadata key of that name
+
+
+def test_model_config_qwen3_moe_with_hybrid_probes(tmp_path):
+    md = [("general.architecture", gw.STRING, "qwen35moe"), ("qwen35moe.block_count", gw.U32, 6),
+          ("qwen35moe.embedding_length", gw.U32, 2048), ("qwen35moe.feed_forward_length", gw.U32, 6144),
+          ("qwen35moe.attention.head_count", gw.U32, 32), ("qwen35moe.attention.head_count_kv", gw.U32, 4),
+          ("qwen35moe.attention.key_length", gw.U32, 256),
+          ("qwen35moe.expert_count", gw.U32, 128), ("qwen35moe.expert_used_count", gw.U32, 8),
+          ("qwen35moe.expert_feed_forward_length", gw.U32, 768),
+          ("qwen35moe.ssm.inner_size", gw.U32, 4096), ("qwen35moe.ssm.state_size", gw.U32, 128),
+          ("qwen35moe.ssm.conv_kernel", gw.U32, 4), ("qwen35moe.ssm.group_count", gw.U32, 16),
+          ("qwen35moe.ssm.time_step_rank", gw.U32, 32), ("qwen35moe.full_attention_interval", gw.U32, 4),
+          ("qwen35moe.nextn_predict_layers", gw.U32, 1),
+          ("qwen35moe.rope.dimension_sections", gw.ARRAY, (gw.I32, [24, 20, 20, 0, 9]))]
+    # QK norm only on the attention layers of a hybrid: layer 3, not layer 0
+    with GGUFFile(_cfg_file(str(tmp_path), "moe.gguf", md, ["blk.3.attn_q_norm.weight"], embd_dims=(2048, 300))) as f:
+        c = f.model_config()
+    assert c["arch"] == "qwen35moe"
+    assert (c["head_dim"], c["kv_head_dim"]) == (256, 256)                        # key_length, not n_embd / n_head = 64
+    assert c["has_qk_norm"] == 1
+    assert (c["num_experts"], c["num_experts_per_tok"], c["moe_intermediate_size"]) == (128, 8, 768)
+    assert c["moe_shared_intermediate_size"] == 768                              # defaults to the routed size
+    assert (c["ssm_inner_size"], c["ssm_state_size"], c["ssm_conv_kernel"], c["ssm_group_count"],
+            c["ssm_time_step_rank"], c["full_attention_interval"]) == (4096, 128, 4, 16, 32, 4)
+    assert c["has_mtp"] == 1 and c["mtp_num_layers"] == 1
+    assert c["rope_sections"] == [24, 20, 20, 0]
+    assert c["n_vocab"] == 300
+
+
+@pytest.mark.parametrize("arch,expect", [
+    ("gemma2", [1, 0, 1, 0, 1, 0, 1, 0, 1, 0, 1, 0]),            # even layers slide
+    ("gemma3", [1, 1, 1, 1, 1, 0, 1, 1, 1, 1, 1, 0]),            # five sliding, one global
+    ("gemma4", [1, 1, 1, 1, 1, 0, 1, 1, 1, 1, 1, 0]),            # no pattern in the file: the same default
+    ("gemma", [0] * 12),                                         # a window but no pattern rule: all global
+])
+def test_model_config_gemma_family(tmp_path, arch, expect):
+    md = [("general.architecture", gw.STRING, arch), (f"{arch}.block_count", gw.U32, 12),
+          (f"{arch}.embedding_length", gw.U32, 2304), (f"{arch}.attention.head_count", gw.U32, 8),
+          (f"{arch}.attention.sliding_window", gw.U32, 4096), (f"{arch}.final_logit_softcapping", gw.F32, 30.0),
+          # per-layer feed-forward lengths: the largest sizes the buffers
+          (f"{arch}.feed_forward_length", gw.ARRAY, (gw.I32, [6144, 12288, 1228])),
+          (f"{arch}.attention.shared_kv_layers", gw.U32, 3), (f"{arch}.embedding_length_per_layer_input", gw.U32, 256)]
+    with GGUFFile(_cfg_file(str(tmp_path), "g.gguf", md, ["blk.0.post_attention_norm.weight", "mtp.0.enorm.weight"])) as f:
+        c = f.model_config()
+    assert c["activation"] == 1 and c["embedding_scale"] == np.float32(np.sqrt(np.float32(2304)))
+    assert c["logit_softcap"] == 30.0 and c["sliding_window"] == 4096
+    assert c["intermediate_size"] == 12288
+    assert c["layer_attn_types"] == expect
+    assert c["has_sandwich_norm"] == 1 and c["has_mtp"] == 1 and c["mtp_num_layers"] == 0
+    assert (c["shared_kv_layers"], c["ple_size"]) == (3, 256)
+    assert c["n_vocab"] == 0                                     # no embedding tensor in the file
+
+
+def test_model_config_gemma4_pattern_from_the_file(tmp_path):
+    pat = [1, 1, 0, 1, 0, 0]
+    md = [("general.architecture", gw.STRING, "gemma4"), ("gemma4.block_count", gw.U32, 6),
+          ("gemma4.embedding_length", gw.U32, 1024), ("gemma4.attention.head_count", gw.U32, 4),
+          ("gemma4.attention.sliding_window", gw.U32, 512),
+          ("gemma4.attention.sliding_window_pattern", gw.ARRAY, (gw.BOOL, pat))]
+    with GGUFFile(_cfg_file(str(tmp_path), "g4.gguf", md)) as f:
+        assert f.model_config()["layer_attn_types"] == pat
+    # a pattern of the wrong length is ignored
+    md[-1] = ("gemma4.attention.sliding_window_pattern", gw.ARRAY, (gw.BOOL, pat[:4]))
+    with GGUFFile(_cfg_file(str(tmp_path), "g4b.gguf", md)) as f:
+        c = f.model_config()
+    assert c["layer_attn_types"] == [1, 1, 1, 1, 1, 0]
+    # the buffer for the per-layer kinds must hold every layer
+    with GGUFFile(_cfg_file(str(tmp_path), "g4c.gguf", md)) as f:
+        out = capi.ModelConfig()
+        small = (C.c_uint8 * 2)()
+        assert capi.lib().bpk_gguf_model_config(f.handle, C.byref(out), small, 2) == -2
+        assert capi.lib().bpk_gguf_model_config(None, C.byref(out), None, 0) == -3
+
+
+_CFG_U = ["n_layer", "n_head", "n_kv_heads", "n_embd", "intermediate_size", "n_vocab", "head_dim", "kv_head_dim",
+          "tie_word_embeddings", "has_qk_norm", "activation", "sliding_window", "n_layer_attn_types", "has_sandwich_norm",
+          "ple_size", "shared_kv_layers", "has_mtp", "mtp_num_layers", "num_experts", "num_experts_per_tok",
+          "moe_intermediate_size", "moe_shared_intermediate_size", "ssm_inner_size", "ssm_state_size", "ssm_conv_kernel",
+          "ssm_group_count", "ssm_time_step_rank", "full_attention_interval"]
+_CFG_F = ["rms_norm_eps", "rope_theta", "embedding_scale", "logit_softcap"]
+
+
+def test_model_config_against_the_compiled_reference(tmp_path, kqref):
+    """Every field, on files of each architecture family, against extractModelConfig itself
+    (runtime/gguf_loader.cpp:184-317, compiled from the reference's sources into oracle/_ref)."""
+    r = kqref.ref()
+    r.bpref_gguf_open.restype = C.c_void_p
+    r.bpref_gguf_open.argtypes = [C.c_char_p]
+    r.bpref_model_config.restype = C.c_uint32
+    r.bpref_model_config.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_char_p,
+                                     C.c_size_t]
+    rng = np.random.default_rng(11)
+    files = []
+    for i, arch in enumerate(["llama", "qwen3", "qwen35moe", "gemma", "gemma2", "gemma3", "gemma4", "gemma4", "mixtral", None]):
+        a = arch or "llama"
+        n_layer = int(rng.integers(2, 20))
+        md = [] if arch is None else [("general.architecture", gw.STRING, arch)]
+        md += [(f"{a}.block_count", gw.U32, n_layer), (f"{a}.embedding_length", gw.U32, int(rng.integers(1, 64)) * 64),
+               (f"{a}.attention.head_count", gw.U32, int(rng.choice([0, 4, 8, 16])))]
+        opt = [(f"{a}.feed_forward_length", gw.ARRAY, (gw.I32, [int(x) for x in rng.integers(100, 9000, 3)])),
+               (f"{a}.attention.head_count_kv", gw.U32, 2), (f"{a}.attention.key_length", gw.U32, 256),
+               (f"{a}.attention.layer_norm_rms_epsilon", gw.F64, 1e-5), (f"{a}.rope.freq_base", gw.F32, 10000.0),
+               (f"{a}.final_logit_softcapping", gw.F32, 30.0), (f"{a}.attention.sliding_window", gw.U32, 1024),
+               (f"{a}.attention.shared_kv_layers", gw.U32, 2), (f"{a}.embedding_length_per_layer_input", gw.U16, 128),
+               (f"{a}.nextn_predict_layers", gw.U32, 2), (f"{a}.expert_count", gw.U32, 64),
+               (f"{a}.expert_used_count", gw.U8, 6), (f"{a}.expert_feed_forward_length", gw.U32, 512),
+               (f"{a}.expert_shared_feed_forward_length", gw.U32, 1024), (f"{a}.ssm.inner_size", gw.U32, 2048),
+               (f"{a}.ssm.state_size", gw.U32, 64), (f"{a}.ssm.conv_kernel", gw.U32, 4), (f"{a}.ssm.group_count", gw.U32, 8),
+               (f"{a}.ssm.time_step_rank", gw.U32, 16), (f"{a}.full_attention_interval", gw.U32, 4),
+               (f"{a}.rope.dimension_sections", gw.ARRAY, (gw.I32, [16, 24, 24, 0])), ("output.weight", gw.U32, 1),
+               (f"{a}.attention.sliding_window_pattern", gw.ARRAY, (gw.BOOL, [int(x) for x in rng.integers(0, 2, n_layer)]))]
+        md += [o for o in opt if rng.random() < (0.6 if i != 7 else 1.0)]
+        names = [n for n in ["blk.0.attn_q_norm.weight", f"blk.{n_layer - 1}.attn_q_norm.weight", "blk.0.post_norm.weight",
+                             "blk.0.attn_post_norm.weight", "mtp.0.blk.0.attn_q.weight", "mtp.0.enorm.weight"]
+                 if rng.random() < 0.4]
+        files.append(_cfg_file(str(tmp_path), f"c{i}.gguf", md, names, embd_dims=(32, 50 + i) if i % 3 else None))
+    for path in files:
+        with GGUFFile(path) as f:
+            mine = f.model_config()
+        h = C.c_void_p(r.bpref_gguf_open(path.encode()))
+        assert h.value
+        u, fl, sec = (C.c_uint32 * 28)(), (C.c_float * 4)(), (C.c_int32 * 4)()
+        types, arch = (C.c_uint8 * 64)(), C.create_string_buffer(64)
+        n_types = r.bpref_model_config(h, u, fl, sec, types, 64, arch, 64)
+        r.bpref_gguf_close(h)
+        assert mine["arch"] == arch.value.decode()
+        assert [mine[k] for k in _CFG_U] == list(u), path
+        assert [np.float32(mine[k]) for k in _CFG_F] == [np.float32(x) for x in fl], path
+        assert mine["rope_sections"] == list(sec)
+        assert mine["layer_attn_types"] == list(types)[:n_types]
