@@ -36,7 +36,7 @@ METRIC = "Q4_K M=1 matvec HBM GB/s (% of peak); M=2048 dequant-GEMM TFLOPS (% MF
 # FETCH_SIZE / WRITE_SIZE summary named below (FETCH_SIZE x 2.000 KiB + WRITE_SIZE x 1.000 KiB, the factors
 # being what the same counters read for a 256 MiB copy kernel); regenerate that file when the kernel changes.
 TRAFFIC_PROFILE = "profiles/decode_gemv_hbm_traffic_pmc.txt"
-MEASURED_TRAFFIC_BYTES = 66557583
+MEASURED_TRAFFIC_BYTES = 66444830
 
 
 def parse():
