@@ -105,6 +105,40 @@ int KQFusedDispatch::run(void* stream) const
     return rc;
 }
 
+KQChain::~KQChain() { bpk_chain_destroy(c_); }
+
+int KQChain::build()
+{
+    bpk_chain_destroy(c_);
+    c_ = nullptr;
+    std::vector<bpk_chain_op> ops(ops_.size());
+    for (size_t i = 0; i < ops_.size(); ++i) {
+        const KQFusedDispatch& f = ops_[i];
+        const KQDispatch& d = f.base;
+        if (d.M != 1) {
+            fprintf(stderr, "%s: a chain takes one token per dispatch\n", d.name.c_str());
+            return BPK_ERR_SHAPE;
+        }
+        ops[i] = bpk_chain_op{(int)d.type, (const float*)d.X.ptr(), d.W.ptr(), (const float*)d.Bias.ptr(), (float*)d.Y.ptr(),
+                              d.P.v[1], d.P.v[0], d.P.v[2], d.P.v[3], d.P.v[4],
+                              bpk_kq_fusion{f.prologue, (const float*)f.NormW.ptr(), f.eps, (const float*)f.Residual.ptr(),
+                                            f.epilogue}};
+    }
+    const int rc = bpk_chain_create(ops.data(), (uint32_t)ops.size(), &c_);
+    if (rc != BPK_OK) fprintf(stderr, "KQChain::build: %s\n", bpk_last_error());
+    return rc;
+}
+
+int KQChain::run(uint32_t first, uint32_t count, void* stream)
+{
+    const int rc = c_ ? bpk_chain_run(c_, first, count, stream) : BPK_ERR_NULL;
+    if (rc != BPK_OK) fprintf(stderr, "KQChain::run: %s\n", c_ ? bpk_last_error() : "not built");
+    return rc;
+}
+
+int KQChain::status() { return c_ ? bpk_chain_status(c_) : BPK_ERR_NULL; }
+int KQChain::reset() { return c_ ? bpk_chain_reset(c_) : BPK_ERR_NULL; }
+
 GGUFFile::~GGUFFile() { bpk_gguf_close(g_); }
 
 bool GGUFFile::open(const std::string& path)
@@ -193,5 +227,31 @@ bool GGUFFile::loadKQWeight(const std::vector<std::string>& names, GPUBuffer& W,
 }
 
 void releaseWeight(bpk_weight* owner) { bpk_weight_destroy(owner); }
+
+ModelConfig extractModelConfig(const GGUFFile& gguf)
+{
+    ModelConfig cfg;
+    bpk_model_config c;
+    if (!gguf.handle() || bpk_gguf_model_config(gguf.handle(), &c, nullptr, 0) != BPK_OK) return cfg;
+    std::vector<uint8_t> kinds(c.n_layer_attn_types);
+    if (!kinds.empty()) bpk_gguf_model_config(gguf.handle(), &c, kinds.data(), (uint32_t)kinds.size());
+    cfg.arch = c.arch;
+    cfg.nLayer = c.n_layer; cfg.nHead = c.n_head; cfg.nKvHeads = c.n_kv_heads; cfg.nEmbd = c.n_embd;
+    cfg.intermediateSize = c.intermediate_size; cfg.nVocab = c.n_vocab; cfg.headDim = c.head_dim; cfg.kvHeadDim = c.kv_head_dim;
+    cfg.rmsNormEps = c.rms_norm_eps; cfg.ropeTheta = c.rope_theta;
+    cfg.tieWordEmbeddings = c.tie_word_embeddings != 0; cfg.hasQkNorm = c.has_qk_norm != 0;
+    cfg.activation = c.activation == BPK_ACT_GELU ? ActivationType::GELU : ActivationType::SiLU;
+    cfg.embeddingScale = c.embedding_scale; cfg.logitSoftcap = c.logit_softcap; cfg.slidingWindow = c.sliding_window;
+    for (uint8_t k : kinds) cfg.layerAttnTypes.push_back(k ? AttnLayerType::SlidingWindow : AttnLayerType::Global);
+    cfg.hasSandwichNorm = c.has_sandwich_norm != 0; cfg.pleSize = c.ple_size; cfg.sharedKvLayers = c.shared_kv_layers;
+    cfg.hasMtp = c.has_mtp != 0; cfg.mtpNumLayers = c.mtp_num_layers;
+    cfg.numExperts = c.num_experts; cfg.numExpertsPerTok = c.num_experts_per_tok;
+    cfg.moeIntermediateSize = c.moe_intermediate_size; cfg.moeSharedIntermediateSize = c.moe_shared_intermediate_size;
+    cfg.ssmInnerSize = c.ssm_inner_size; cfg.ssmStateSize = c.ssm_state_size; cfg.ssmConvKernel = c.ssm_conv_kernel;
+    cfg.ssmGroupCount = c.ssm_group_count; cfg.ssmTimeStepRank = c.ssm_time_step_rank;
+    cfg.fullAttentionInterval = c.full_attention_interval;
+    cfg.ropeSections.assign(c.rope_sections, c.rope_sections + 4);
+    return cfg;
+}
 
 }  // namespace bp

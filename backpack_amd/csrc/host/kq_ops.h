@@ -82,6 +82,27 @@ struct KQFusedDispatch {
     int run(void* stream = nullptr) const;
 };
 
+// A recorded stretch of the decode dispatch list whose entries are fused k-quant matvecs feeding each other
+// (the per-token command buffer, runtime/model_runner.cpp:5725-5759, between two attention blocks): record the
+// dispatches once, then run(first, count) issues a range of them as ONE launch.  An entry whose X or Residual is
+// the Y of an earlier entry follows it inside the launch.
+struct KQChain {
+    KQChain() = default;
+    KQChain(const KQChain&) = delete;
+    KQChain& operator=(const KQChain&) = delete;
+    ~KQChain();
+    void add(const KQFusedDispatch& d) { ops_.push_back(d); }
+    size_t size() const { return ops_.size(); }
+    int build();                                                      // after the last add
+    int run(uint32_t first, uint32_t count, void* stream = nullptr);  // needs build()
+    int status();                                                     // BPK_OK, or what a bounded wait gave up on
+    int reset();
+
+private:
+    std::vector<KQFusedDispatch> ops_;
+    bpk_chain* c_ = nullptr;
+};
+
 // Read-only view of a GGUF file with the reference's member names.  Tensor data pointers stay valid
 // until the object is destroyed.
 struct GGUFTensorInfo {
@@ -113,11 +134,38 @@ struct GGUFFile {
     // Named k-quant tensors stacked into one device weight (q|k|v, gate|up); W.handle is the library's
     // allocation and is released with releaseWeight.
     bool loadKQWeight(const std::vector<std::string>& names, GPUBuffer& W, KQuantPacked& desc, bpk_weight** owner) const;
+    const bpk_gguf* handle() const { return g_; }
 
 private:
     bpk_gguf* g_ = nullptr;
 };
 void releaseWeight(bpk_weight* owner);
+
+// The model's hyper-parameters with the reference's field names (ModelConfig, runtime/gguf_loader.h:164-218;
+// extractModelConfig, runtime/gguf_loader.cpp:184-317).
+enum class ActivationType { SiLU, GELU };
+enum class AttnLayerType : uint8_t { Global, SlidingWindow };
+struct ModelConfig {
+    std::string arch;
+    uint32_t nLayer = 0, nHead = 0, nKvHeads = 0, nEmbd = 0, intermediateSize = 0, nVocab = 0, headDim = 0, kvHeadDim = 0;
+    float rmsNormEps = 1e-6f, ropeTheta = 1e6f;
+    bool tieWordEmbeddings = true, hasQkNorm = false;
+    ActivationType activation = ActivationType::SiLU;
+    float embeddingScale = 0.0f, logitSoftcap = 0.0f;
+    uint32_t slidingWindow = 0;
+    std::vector<AttnLayerType> layerAttnTypes;
+    bool hasSandwichNorm = false;
+    uint32_t pleSize = 0, sharedKvLayers = 0;
+    bool hasMtp = false;
+    uint32_t mtpNumLayers = 0;
+    uint32_t numExperts = 0, numExpertsPerTok = 0, moeIntermediateSize = 0, moeSharedIntermediateSize = 0;
+    uint32_t ssmInnerSize = 0, ssmStateSize = 0, ssmConvKernel = 0, ssmGroupCount = 0, ssmTimeStepRank = 0,
+             fullAttentionInterval = 0;
+    std::vector<int32_t> ropeSections = {11, 11, 10, 0};
+    // hybrid SSM + attention files: every fullAttentionInterval-th layer is attention (0: all of them)
+    bool isAttentionLayer(uint32_t i) const { return fullAttentionInterval == 0 || (i + 1) % fullAttentionInterval == 0; }
+};
+ModelConfig extractModelConfig(const GGUFFile& gguf);
 
 // Dequantised rows (the q6k_gather / q6k_gather_batched dispatch).
 int gatherKQ(GGUFType type, const GPUBuffer& W, uint32_t rowStrideWords, const GPUBuffer& tokens, uint32_t M,

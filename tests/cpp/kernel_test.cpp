@@ -1,6 +1,6 @@
 // The reference's eleven Q4_K / Q5_K / Q6_K kernel tests (runtime/tests/kernel_test.cpp:1669-1748)
 // re-stated against the C++ host layer: same names, same closed-form inputs, same
-// tolerances.  Expected values come from the CPU oracle (test infrastructure),
+// tolerances; then the layer's own additions (fused dispatches, GGUF file, chain, model configuration).  Expected values come from the CPU oracle (test infrastructure),
 // which plays the part of dequant_kquant + the sequential fp32 dot.
 #include <cmath>
 #include <cstdio>
@@ -273,6 +273,100 @@ TEST(gguf_file_to_fused_weight) {
     releaseBuffer(bx); releaseBuffer(by); releaseWeight(owner);
     remove(path);
     return assertClose(got.data(), expected.data(), 2 * N, 2e-4f, 2e-4f);
+}
+
+TEST(chain_of_a_decoder_layer_tail) {
+    // o + residual -> norm -> gate|up -> silu*up -> down + residual, recorded as three fused dispatches and run as
+    // ONE launch; expected = the same composition on the oracle, op after op
+    const int H = 512, I = 768, NBH = H / 256, NBI = I / 256;
+    auto ro = q4kRaw(H, NBH, [](int n, int) { return .004f + .00001f * n; }, [](int, int b) { return .002f + .0001f * b; },
+                     [](int n, int b, int i) { return n * 31 + b * 13 + i * 17; });
+    auto rg = q4kRaw(2 * I, NBH, [](int n, int) { return .003f + .000005f * n; }, [](int, int) { return .0015f; },
+                     [](int n, int b, int i) { return n * 7 + b * 5 + i * 3 + 1; });
+    auto rd = q6kRaw(H, NBI, [](int n, int b) { return .002f + .00001f * n + .0001f * b; },
+                     [](int n, int b, int i) { return n * 29 + b * 23 + i * 19 + 5; });
+    KQuantPacked po = pack_q4k(ro.data(), H, H), pg = pack_q4k(rg.data(), 2 * I, H), pd = pack_q6k(rd.data(), H, I);
+    auto attn = randnVec(11, H), x0 = randnVec(12, H), nw = randnVec(13, H);
+    for (auto& v : nw) v = 1.0f + 0.1f * v;
+    const float eps = 1e-5f;
+    // oracle
+    std::vector<float> x = x0, t(H), xn(H), gu(2 * I), act(I), dn(H);
+    kqo_matmul(KQO_TYPE_Q4_K, attn.data(), po.data.data(), nullptr, t.data(), 1, H, H, po.rowStrideWords, 0, 0);
+    for (int i = 0; i < H; i++) x[i] += t[i];
+    kqo_prologue(1, x.data(), nw.data(), eps, 1, H, xn.data());
+    kqo_matmul(KQO_TYPE_Q4_K, xn.data(), pg.data.data(), nullptr, gu.data(), 1, 2 * I, H, pg.rowStrideWords, 0, 0);
+    kqo_prologue(2, gu.data(), nullptr, 0.0f, 1, I, act.data());
+    kqo_matmul(KQO_TYPE_Q6_K, act.data(), pd.data.data(), nullptr, dn.data(), 1, H, I, pd.rowStrideWords, 0, 0);
+    std::vector<float> expected = x;
+    for (int i = 0; i < H; i++) expected[i] += dn[i];
+    // device
+    GPUBuffer bAttn = createBuffer("attn", H * 4), bX = createBuffer("x", H * 4), bNw = createBuffer("nw", H * 4),
+              bAct = createBuffer("act", I * 4), wo = uploadKQWeight("o", po), wg = uploadKQWeight("gate_up", pg),
+              wd = uploadKQWeight("down", pd);
+    writeBuffer(bAttn, attn.data(), H * 4); writeBuffer(bX, x0.data(), H * 4); writeBuffer(bNw, nw.data(), H * 4);
+    KQChain chain;
+    KQFusedDispatch o; o.base = KQDispatch{GGUF_TYPE_Q4_K, bAttn, wo, GPUBuffer{}, bX, makeKQParams(H, H, po.nBlocks, po.rowStrideWords), 1, "o"};
+    o.Residual = bX;
+    KQFusedDispatch g; g.base = KQDispatch{GGUF_TYPE_Q4_K, bX, wg, GPUBuffer{}, bAct, makeKQParams(H, I, pg.nBlocks, pg.rowStrideWords), 1, "gate_up"};
+    g.prologue = BPK_PRO_RMS_NORM; g.NormW = bNw; g.eps = eps; g.epilogue = BPK_EPI_SILU_MUL;
+    KQFusedDispatch d; d.base = KQDispatch{GGUF_TYPE_Q6_K, bAct, wd, GPUBuffer{}, bX, makeKQParams(I, H, pd.nBlocks, pd.rowStrideWords), 1, "down"};
+    d.Residual = bX;
+    chain.add(o); chain.add(g); chain.add(d);
+    if (chain.build() != BPK_OK) return {false, bpk_last_error()};
+    if (chain.run(0, 3) != BPK_OK || chain.status() != BPK_OK) return {false, bpk_last_error()};
+    std::vector<float> got(H);
+    readBuffer(bX, got.data(), H * 4);
+    // and the same ops as separate fused dispatches give the same residual stream
+    writeBuffer(bX, x0.data(), H * 4);
+    if (o.run() != BPK_OK || g.run() != BPK_OK || d.run() != BPK_OK) return {false, bpk_last_error()};
+    std::vector<float> sep(H);
+    readBuffer(bX, sep.data(), H * 4);
+    releaseBuffer(bAttn); releaseBuffer(bX); releaseBuffer(bNw); releaseBuffer(bAct); releaseBuffer(wo); releaseBuffer(wg); releaseBuffer(wd);
+    CheckResult r = assertClose(got.data(), expected.data(), H, 2e-4f, 2e-4f);
+    if (!r.ok) return r;
+    return assertClose(sep.data(), got.data(), H, 2e-5f, 2e-5f);
+}
+TEST(model_config_from_gguf) {
+    // a metadata-only file of a Gemma-3-shaped model, read through the GGUFFile mirror and extractModelConfig
+    std::vector<uint8_t> f;
+    auto put = [&](const void* p, size_t n) { f.insert(f.end(), (const uint8_t*)p, (const uint8_t*)p + n); };
+    auto u32 = [&](uint32_t v) { put(&v, 4); };
+    auto u64 = [&](uint64_t v) { put(&v, 8); };
+    auto f32 = [&](float v) { put(&v, 4); };
+    auto str = [&](const std::string& s) { u64(s.size()); put(s.data(), s.size()); };
+    u32(0x46554747); u32(3); u64(2); u64(8);
+    str("general.architecture"); u32(8); str("gemma3");
+    str("gemma3.block_count"); u32(4); u32(12);
+    str("gemma3.embedding_length"); u32(4); u32(2560);
+    str("gemma3.attention.head_count"); u32(4); u32(8);
+    str("gemma3.attention.head_count_kv"); u32(4); u32(4);
+    str("gemma3.attention.key_length"); u32(4); u32(256);
+    str("gemma3.attention.sliding_window"); u32(4); u32(1024);
+    str("gemma3.feed_forward_length"); u32(9); u32(5); u64(3); u32(6144); u32(10240); u32(1228);   // int32 array: the largest counts
+    str("token_embd.weight"); u32(2); u64(8); u64(3); u32(0); u64(0);
+    str("blk.0.post_attention_norm.weight"); u32(1); u64(8); u32(0); u64(96);
+    const size_t data_offset = (f.size() + 31) / 32 * 32;
+    f.resize(data_offset + 96 + 32, 0);
+    const char* path = "/tmp/bpk_kernel_test_cfg.gguf";
+    FILE* fp = fopen(path, "wb");
+    if (!fp) return {false, "cannot write the temporary file"};
+    fwrite(f.data(), 1, f.size(), fp);
+    fclose(fp);
+    (void)f32;
+    GGUFFile g;
+    if (!g.open(path)) return {false, bpk_last_error()};
+    const ModelConfig c = extractModelConfig(g);
+    remove(path);
+    if (c.arch != "gemma3" || c.nLayer != 12 || c.nEmbd != 2560 || c.nHead != 8 || c.nKvHeads != 4) return {false, "dimensions"};
+    if (c.headDim != 256 || c.kvHeadDim != 256 || c.intermediateSize != 10240 || c.nVocab != 3) return {false, "derived dimensions"};
+    if (c.rmsNormEps != 1e-6f || c.ropeTheta != 1000000.0f || !c.tieWordEmbeddings) return {false, "defaults"};
+    if (c.activation != ActivationType::GELU || c.embeddingScale != sqrtf(2560.0f) || !c.hasSandwichNorm) return {false, "gemma family"};
+    if (c.slidingWindow != 1024 || c.layerAttnTypes.size() != 12) return {false, "sliding window"};
+    for (uint32_t i = 0; i < 12; i++)
+        if (c.layerAttnTypes[i] != ((i + 1) % 6 == 0 ? AttnLayerType::Global : AttnLayerType::SlidingWindow)) return {false, "layer pattern"};
+    if (c.numExperts != 0 || c.hasMtp || c.ropeSections != std::vector<int32_t>({11, 11, 10, 0}) || !c.isAttentionLayer(5))
+        return {false, "remaining defaults"};
+    return {true, ""};
 }
 
 int main()

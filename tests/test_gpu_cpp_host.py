@@ -14,4 +14,4 @@ def test_reference_kernel_tests_through_cpp_host_layer():
     r = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert "14 tests, 0 failed" in r.stdout
+    assert "16 tests, 0 failed" in r.stdout
