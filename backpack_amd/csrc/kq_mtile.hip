@@ -127,8 +127,11 @@ __device__ __forceinline__ float mtile_act(float g, float u)
 // HALF: the sums of x go out per half run of 16 elements, [run][half][token] (the 16-token Q6_K kernel).
 // PRO: the prologues of the fused forms.  1: RMSNorm, the chunk's norm weights are read from LDS (nw, staged by
 // the kernel); 2: act(gate) * up, up travels with X.
-template <int NT, bool SPLIT16, int TOK, bool XV, bool HALF = false, int PRO = 0>
+// HL8: at most 8 tokens; a token's hi part goes to slot token and its lo part to slot token + 8 of ONE operand, so
+// that a single matrix instruction multiplies both (the two partial tiles are added once at the end).
+template <int NT, bool SPLIT16, int TOK, bool XV, bool HALF = false, int PRO = 0, bool HL8 = false>
 struct MtileStager {
+    static_assert(!(HL8 && (SPLIT16 || HALF)), "hi / lo slots are a form of the Q4_K / Q5_K kernels");
     static_assert(!(SPLIT16 && HALF), "half sums live in token slots (SPLIT16) or in a second plane (HALF)");
     static constexpr uint32_t XSR = HALF ? 32u : 16u;   // floats of xs per run
     static constexpr int TPP = NT / (MT_KC * TOK);  // threads per (token, block) pair
@@ -147,7 +150,7 @@ struct MtileStager {
         sub = threadIdx.x % TPP;
         bb = pair % MT_KC;
         token = pair / MT_KC;
-        live_token = token < count && (!SPLIT16 || token < 8u);
+        live_token = token < count && (!(SPLIT16 || HL8) || token < 8u);
         xrow = token;
         if (rec && live_token) {
             const uint32_t pr = rec[2u + token];
@@ -231,7 +234,7 @@ struct MtileStager {
         const float inv = __builtin_bit_cast(float, (e - 14u) << 23);    // 2^(e-141)
         if (sub == 0) {
             xinv[bb * 16u + token] = inv;
-            if (SPLIT16) xinv[bb * 16u + token + 8u] = inv;
+            if (SPLIT16 || HL8) xinv[bb * 16u + token + 8u] = inv;
         }
         // Q4_K: the sum over sub-block sb also goes out as element sb of an A operand (lane = token, the
         // lanes of k >= 8 stay zero), scaled by s / 32 so that 32 elements of at most 2^15 fit an fp16
@@ -242,7 +245,7 @@ struct MtileStager {
             const _Float16 l = (_Float16)(a - (float)h);
             _Float16* dst = (_Float16*)(xv + ((size_t)(bb * 2u) * 64u + token) * 16u) + sb;
             dst[0] = h;
-            dst[512] = l;   // the lo operand: 1024 bytes on
+            dst[HL8 ? 64 : 512] = l;   // the lo operand: 1024 bytes on, or (HL8) slot token + 8
         };
         // groups of 8 consecutive k -> one operand slot: halves in the order k+0, k+2, k+1, k+3, k+4, k+6, k+5, k+7
 #pragma unroll
@@ -263,7 +266,7 @@ struct MtileStager {
             const uint32_t slot = SPLIT16 ? token + 8u * (kq >> 1) : token;
             uint8_t* dst = xa + ((size_t)((bb * 8u + sb) * 2u) * 64u + slot + 16u * kq) * 16u;
             *(t_half8*)dst = hv;
-            *(t_half8*)(dst + 1024) = lv;
+            *(t_half8*)(dst + (HL8 ? 8 * 16 : 1024)) = lv;
         }
         // sums of the unscaled x over each run of 32 (or, SPLIT16, each half run of 16)
         if constexpr (EPT >= 32) {
@@ -278,7 +281,7 @@ struct MtileStager {
                 float* dst = xs + (bb * 8u + (sub * EPT) / 32u + q) * XSR + token;
                 if (SPLIT16) { dst[0] = h0; dst[8] = h1; }
                 else if (HALF) { dst[0] = h0; dst[16] = h1; }
-                else { dst[0] = h0 + h1; put_sum((sub * EPT) / 32u + q, h0 + h1); }
+                else { if (!HL8) dst[0] = h0 + h1; put_sum((sub * EPT) / 32u + q, h0 + h1); }   // (HL8 reads xv only)
             }
         } else {
             // the run is spread over 32 / EPT neighbouring threads: partial sums meet by lane exchange
@@ -295,7 +298,7 @@ struct MtileStager {
                 if (sub % PER16 == 0u) dst[16u * half] = h;
             } else {
                 h += group_partner<PER16>(h);
-                if (sub % (2u * PER16) == 0u) { dst[0] = h; put_sum(run, h); }
+                if (sub % (2u * PER16) == 0u) { if (!HL8) dst[0] = h; put_sum(run, h); }
             }
         }
     }
@@ -308,12 +311,14 @@ struct MtileStager {
 struct MtileA {
     t_half8 hi, lo;
 };
+template <bool HL8 = false>
 __device__ __forceinline__ MtileA mtile_read_a(const uint8_t* xa_b, int sb, uint32_t lane)
 {
     const uint8_t* ap = xa_b + ((size_t)(sb * 2) * 64u + lane) * 16u;
     MtileA a;
     a.hi = *(const t_half8*)ap;
-    a.lo = *(const t_half8*)(ap + 1024);
+    a.lo = a.hi;
+    if constexpr (!HL8) a.lo = *(const t_half8*)(ap + 1024);   // (HL8: hi and lo share the one operand)
     return a;
 }
 
@@ -335,7 +340,7 @@ __device__ __forceinline__ void q5_join(t_u32x4& blo, t_u32x4& bhi, const t_u32x
     }
 }
 
-template <bool Q5>
+template <bool Q5, bool HL8 = false>
 __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2 (&w)[4], const t_u32x2 qhw, const uint8_t* xa_b,
                                                 const uint8_t* xv_b, const float* xinv_b, uint32_t lane,
                                                 t_f32x4& tot)
@@ -347,9 +352,10 @@ __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2
     const uint32_t scB = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
     const uint32_t mnB = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
     t_f32x4 U = {0, 0, 0, 0};
-    MtileA a_cur = mtile_read_a(xa_b, 0, lane);
+    MtileA a_cur = mtile_read_a<HL8>(xa_b, 0, lane);
     const t_half8 vhi = *(const t_half8*)(xv_b + (size_t)lane * 16u);
-    const t_half8 vlo = *(const t_half8*)(xv_b + 1024 + (size_t)lane * 16u);
+    t_half8 vlo = vhi;
+    if constexpr (!HL8) vlo = *(const t_half8*)(xv_b + 1024 + (size_t)lane * 16u);
     t_f32x4 D_prev = {0, 0, 0, 0};
     t_u32x4 blo = {0, 0, 0, 0}, bhi = {0, 0, 0, 0};
     auto scale_in = [&](int sb, const t_f32x4& D) {
@@ -361,7 +367,7 @@ __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2
 #pragma unroll
     for (int sb = 0; sb < 8; ++sb) {
         MtileA a_next = a_cur;
-        if (sb < 7) a_next = mtile_read_a(xa_b, sb + 1, lane);
+        if (sb < 7) a_next = mtile_read_a<HL8>(xa_b, sb + 1, lane);
         if ((sb & 1) == 0) {
             const uint32_t d0 = w[sb >> 1].x, d1 = w[sb >> 1].y;
             const uint32_t e0 = d0 >> 8, e1 = d1 >> 8;
@@ -372,7 +378,7 @@ __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2
         const t_half8 bq = __builtin_bit_cast(t_half8, (sb & 1) ? bhi : blo);
         t_f32x4 D = {0, 0, 0, 0};
         D = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur.hi, bq, D, 0, 0, 0);
-        D = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur.lo, bq, D, 0, 0, 0);
+        if constexpr (!HL8) D = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur.lo, bq, D, 0, 0, 0);
         if (sb > 0) scale_in(sb - 1, D_prev);
         __builtin_amdgcn_sched_barrier(0);   // keeps the three stages of this step together
         D_prev = D;
@@ -384,7 +390,7 @@ __device__ __forceinline__ void q4k_mtile_block(const t_u32x4 hdr, const t_u32x2
     const t_half8 bmn = __builtin_bit_cast(t_half8, bm);
     t_f32x4 V = {0, 0, 0, 0};
     V = __builtin_amdgcn_mfma_f32_16x16x32_f16(vhi, bmn, V, 0, 0, 0);
-    V = __builtin_amdgcn_mfma_f32_16x16x32_f16(vlo, bmn, V, 0, 0, 0);
+    if constexpr (!HL8) V = __builtin_amdgcn_mfma_f32_16x16x32_f16(vlo, bmn, V, 0, 0, 0);
     scale_in(7, D_prev);
     // U carries 2^-24 from the subnormal nibbles and the token's scale s; V carries 2^-24 and s / 32
     const float4 inv = *(const float4*)(xinv_b + 4u * (lane >> 4));
@@ -635,7 +641,7 @@ struct MtileWStage {
 // of two) costs more than the line re-fetches, so they load each lane's pieces straight from global memory.
 // (the grouped Q4_K kernel is held to 128 registers so that two of its workgroups share a CU)
 // FUSED: residual and pair epilogue; PRO: the prologue (1 RMSNorm, 2 act(gate) * up)
-template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0>
+template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0, bool HL8 = false>
 __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1) void mtile_kernel(MtileParams p)
 // (Q5_K: the Q4_K code with blocks of 176 bytes — header, 32 bytes of fifth bits, quants — and one more
 // 8-byte piece per lane and superblock)
@@ -667,6 +673,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     }
     static_assert(!FUSED || (R == NW && STAGED), "the fused forms come with a wave per tile, weights staged");
     static_assert(FUSED || PRO == 0, "prologues belong to the fused kernels");
+    static_assert(!HL8 || (STAGED && (TYPE == KQ_TYPE_Q4_K || TYPE == KQ_TYPE_Q5_K)), "hi / lo slots: dense Q4_K / Q5_K");
     bool has_tile = R == 1 || wave < p.tiles_per_wg;
     uint32_t tile = R == 1 ? blockIdx.x : blockIdx.x * p.tiles_per_wg + wave;
     const bool pairs = FUSED && p.epi != 0;
@@ -682,6 +689,8 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
 
     // Q6: the block format; Q6S: the 8-token kernel whose tokens take two slots each; Q6W: the 16-token one
     constexpr bool Q6W = TYPE == MT_TYPE_Q6K_WIDE, Q6S = TYPE == KQ_TYPE_Q6_K, Q6 = Q6W || Q6S, Q5 = TYPE == KQ_TYPE_Q5_K;
+    // lanes l and l + 32 hold two addends of the same outputs (Q6_K's 16-element halves, or hi and lo parts)
+    constexpr bool HALVES = Q6S || HL8;
     constexpr uint32_t BB = Q6 ? KQ_Q6K_BYTES : Q5 ? KQ_Q5K_BYTES : KQ_Q4K_BYTES;
     constexpr uint32_t XSB = Q6W ? 256u : 128u;   // floats of xs per superblock
     constexpr uint32_t QOFF = Q5 ? 48u : 16u;   // where the quants start inside a block
@@ -704,7 +713,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     const uint32_t c_begin = (p.tiles ? 0u : blockIdx.z) * p.chunks_per_split * MT_KC;
     const uint32_t c_end = min(p.n_blocks, c_begin + p.chunks_per_split * MT_KC);
 
-    MtileStager<64 * NW, Q6S, TOK, STAGED && !Q6, Q6W, PRO> stager;
+    MtileStager<64 * NW, Q6S, TOK, STAGED && !Q6, Q6W, PRO, HL8> stager;
     stager.init(p, rec, count);
     stager.fetch(p, c_begin);
     // norm prologue: the sums of squares per token are gathered while X is converted and meet here at the end
@@ -735,7 +744,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     t_f32x4 tot = {0, 0, 0, 0};
     // a finished tile: lane l holds tokens 4*(l/16) .. +3 of weight row row_t
     auto put_tile = [&](uint32_t row_t, const t_f32x4& t) {
-        if (row_t < p.N && (!Q6S || kq < 2u)) {
+        if (row_t < p.N && (!HALVES || kq < 2u)) {
             const float bias = p.bias ? p.bias[row_t] : 0.0f;
             const float t4[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
@@ -754,7 +763,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         }
     };
     auto store_tile = [&](uint32_t row_t, t_f32x4 t) {
-        if constexpr (Q6S) {   // lanes l and l + 32 hold the two 16-element halves of the same tokens
+        if constexpr (HALVES) {   // lanes l and l + 32 hold two addends of the same tokens
             t.x += __shfl_xor(t.x, 32, 64);
             t.y += __shfl_xor(t.y, 32, 64);
             t.z += __shfl_xor(t.z, 32, 64);
@@ -770,9 +779,16 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
     __syncthreads();
 
+    // HL8 leaves the second plane of every operand pair unused: consecutive chunks alternate between the planes
+    // (the token scales between xinv and the unused xs), so a chunk is parked while slower waves still multiply
+    // the one before, and one barrier per chunk is enough.
+    uint32_t plane = 0;
     for (uint32_t c0 = c_begin; c0 < c_end; c0 += MT_KC) {
+        uint8_t* xa_c = xa + (HL8 ? plane * 1024u : 0u);
+        uint8_t* xv_c = xv + (HL8 ? plane * 1024u : 0u);
+        float* xinv_c = HL8 && plane ? xs : xinv;
         stager.prologue(p, c0 + stager.bb < c_end, nwbuf + nw_parity * (MT_KC * KQ_QK));
-        stager.park(xa, xs, xinv, xv);
+        stager.park(xa_c, xs, xinv_c, xv_c);
         nw_parity ^= 1u;
         nw_park(nw_parity);           // the next chunk's norm weights (this buffer was last read one barrier ago)
         ws[0].store(wwin);
@@ -807,12 +823,17 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
 #pragma unroll
                         for (int g = 0; g < 4; ++g) w[g] = *(const t_u32x2*)(blk + QOFF + 32u * g + 8u * kq);
                         if constexpr (Q5) qhw = *(const t_u32x2*)(blk + 16u + 8u * kq);
-                        q4k_mtile_block<Q5>(hdr, w, qhw, xa + (size_t)bb * (8 * 2 * 1024), xv + (size_t)bb * 2048, xinv + bb * 16, lane, tot);
+                        q4k_mtile_block<Q5, HL8>(hdr, w, qhw, xa_c + (size_t)bb * (8 * 2 * 1024), xv_c + (size_t)bb * 2048, xinv_c + bb * 16, lane, tot);
                     }
                 }
             }
         }
-        __syncthreads();
+        if constexpr (HL8) {
+            plane ^= 1u;
+            wave_window_fence();   // this wave's reads of its window are done before the next chunk is stored there
+        } else {
+            __syncthreads();
+        }
     }
     } else {
     for (uint32_t i = threadIdx.x; i < MT_STAGE_BYTES / 16; i += 64 * NW)
@@ -884,8 +905,8 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
             tot.x += o.x; tot.y += o.y; tot.z += o.z; tot.w += o.w;
         }
     }
-    if constexpr (Q6S) {
-        // lanes l and l + 32 hold the two 16-element halves of tokens 4*(l/16) .. +3: add them
+    if constexpr (HALVES) {
+        // lanes l and l + 32 hold the two addends of tokens 4*(l/16) .. +3: add them
         tot.x += __shfl_xor(tot.x, 32, 64);
         tot.y += __shfl_xor(tot.y, 32, 64);
         tot.z += __shfl_xor(tot.z, 32, 64);
@@ -907,7 +928,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
         // ticket once they are acknowledged, and the last one in reads all of them back past the
         // non-coherent cache levels and adds them in split order.
         const size_t plane = (size_t)gridDim.x * p.tiles_per_wg * 16u;   // rows of all tiles
-        const bool mine = has_tile && (!Q6S || kq < 2u);
+        const bool mine = has_tile && (!HALVES || kq < 2u);
         const uint32_t prow = (blockIdx.x * p.tiles_per_wg + wave) * 16u + (lane & 15u);
         if (mine) {
             const float t4[4] = {tot.x, tot.y, tot.z, tot.w};
@@ -963,7 +984,7 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
             if (wave >= half_waves && wave < p.tiles_per_wg)
                 *(t_f32x4*)(red + ((wave - half_waves) * 64u + lane) * 4u) = t_f32x4{tot.x + b, tot.y + b, tot.z + b, tot.w + b};
             __syncthreads();
-            if (wave >= half_waves || !has_tile || (Q6S && kq >= 2u)) return;
+            if (wave >= half_waves || !has_tile || (HALVES && kq >= 2u)) return;
             const t_f32x4 up = *(const t_f32x4*)(red + (wave * 64u + lane) * 4u);
             const float g4[4] = {tot.x + b, tot.y + b, tot.z + b, tot.w + b}, u4[4] = {up.x, up.y, up.z, up.w};
 #pragma unroll
@@ -989,7 +1010,7 @@ bool mtile_supported(const MatmulArgs& a)
     return false;
 }
 
-template <int TYPE, int NW, int R, bool STAGED = true, int TOK = 16, bool FUSED = false, int PRO = 0>
+template <int TYPE, int NW, int R, bool STAGED = true, int TOK = 16, bool FUSED = false, int PRO = 0, bool HL8 = false>
 static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s, uint32_t wgs_z = 1)
 {
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K || TYPE == MT_TYPE_Q6K_WIDE, Q5 = TYPE == KQ_TYPE_Q5_K;
@@ -997,7 +1018,7 @@ static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t 
     // + the sums of squares per token and two chunks of norm weights
     constexpr size_t shmem = MT_STAGE_BYTES + (STAGED ? (size_t)NW * 16 * PITCH : 0) + (FUSED ? 64 : 0) +
                              (PRO == 1 ? 2 * MT_KC * KQ_QK * 4 : 0);
-    auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK, FUSED, PRO>;
+    auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK, FUSED, PRO, HL8>;
     static bool raised = false;   // per instantiation
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -1116,10 +1137,14 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
             const uint32_t wgs = (tiles + best_tpw - 1u) / best_tpw;
             // 5..8 tokens: the conversion of X is spread over twice the threads per (token, superblock), so
             // that all waves take part (measured +2-3 %; with 4 tokens or fewer the wider exchange costs more)
+            // Q4_K / Q5_K with at most 8 tokens: hi and lo parts as token slots of one matrix instruction
             if (p.M > 4u && p.M <= 8u)
                 e = q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits)
-                    : q5 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits)
-                         : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 8>(p, wgs, 1, s, best_splits);
+                    : q5 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 8, false, 0, true>(p, wgs, 1, s, best_splits)
+                         : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 8, false, 0, true>(p, wgs, 1, s, best_splits);
+            else if (p.M <= 4u && !q6)
+                e = q5 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, false, 0, true>(p, wgs, 1, s, best_splits)
+                       : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, false, 0, true>(p, wgs, 1, s, best_splits);
             else
                 e = q6_wide ? launch_mtile_one<MT_TYPE_Q6K_WIDE, 8, 8, true, 16>(p, wgs, 1, s, best_splits)
                     : q6 ? launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16>(p, wgs, 1, s, best_splits)
@@ -1182,22 +1207,29 @@ hipError_t launch_mtile_fused(const MatmulArgs& a, const SplitScratch& sc, hipSt
     p.x_stride = a.pro >= 2 ? 2u * a.K : a.K;
     p.pair_tile0 = tiles / 2u;
     const uint32_t wgs = a.epi ? (tiles / 2u + best_tpw / 2u - 1u) / (best_tpw / 2u) : (tiles + best_tpw - 1u) / best_tpw;
+    const bool hl8 = !q6 && a.M <= 8u;   // hi and lo parts as token slots of one matrix instruction
     if (a.pro == 1) {
         if (q6_wide) return launch_mtile_one<MT_TYPE_Q6K_WIDE, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
         if (q6) return launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
-        if (q5) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
-        return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
+        if (q5) return hl8 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true, 1, true>(p, wgs, 1, s, best_splits)
+                           : launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
+        return hl8 ? launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true, 1, true>(p, wgs, 1, s, best_splits)
+                   : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true, 1>(p, wgs, 1, s, best_splits);
     }
     if (a.pro != 0) {
         // (the 16-slot Q6_K kernel has no registers for a second operand: mtile_fused_supported declines)
         if (q6) return launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16, true, 2>(p, wgs, 1, s, best_splits);
-        if (q5) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true, 2>(p, wgs, 1, s, best_splits);
-        return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true, 2>(p, wgs, 1, s, best_splits);
+        if (q5) return hl8 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true, 2, true>(p, wgs, 1, s, best_splits)
+                           : launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true, 2>(p, wgs, 1, s, best_splits);
+        return hl8 ? launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true, 2, true>(p, wgs, 1, s, best_splits)
+                   : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true, 2>(p, wgs, 1, s, best_splits);
     }
     if (q6_wide) return launch_mtile_one<MT_TYPE_Q6K_WIDE, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
     if (q6) return launch_mtile_one<KQ_TYPE_Q6_K, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
-    if (q5) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
-    return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
+    if (q5) return hl8 ? launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true, 0, true>(p, wgs, 1, s, best_splits)
+                       : launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
+    return hl8 ? launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true, 0, true>(p, wgs, 1, s, best_splits)
+               : launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, true, 16, true>(p, wgs, 1, s, best_splits);
 }
 
 }  // namespace kq
