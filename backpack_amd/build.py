@@ -102,12 +102,20 @@ def check_ring_registers(asm_path: str) -> list[str]:
     return problems
 
 
+# A source that carries this marker has kernels whose arguments are scalars and few enough to arrive in scalar
+# registers with the wave (kernel-argument preloading, up to 16 dwords); kernels with struct arguments are unaffected.
+PRELOAD_MARKER = "KQ_KERNARG_PRELOAD"
+
+
 def _compile(src: str) -> str:
     base = os.path.basename(src).replace(".hip", "")
     obj = os.path.join(OBJ, base + ".o")
     extra = os.environ.get("BPK_EXTRA_FLAGS", "").split()   # experiments only
     with open(src) as f:
-        guarded = NO_SPILL_MARKER in f.read()
+        text = f.read()
+    guarded = NO_SPILL_MARKER in text
+    if PRELOAD_MARKER in text and os.environ.get("BPK_NO_KERNARG_PRELOAD") != "1":
+        extra += ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
     tracked = os.environ.get("BPK_TRACKED_LOADS") == "1"
     if guarded:
         extra.append("-Rpass-analysis=kernel-resource-usage")

@@ -31,13 +31,14 @@ namespace kq {
 // Kernel arguments come in three sizes, and a kernel is compiled for each: the wave's first
 // instructions fetch them, and every further 64 bytes of them cost a launch a measurable fraction of a
 // microsecond, so the dense decode matvec gets the smallest set that describes it.
-struct StreamDense {          // 60 bytes
+struct StreamDense {          // 64 bytes = the 16 dwords that kernel-argument preloading holds
     const float* X;
     const uint8_t* W;
     const float* bias;
     float* Y;
     uint32_t N, K, n_blocks, row_stride_bytes, y_offset, ldy;
     uint32_t M;   // tokens; read only by the four-token kernels (three tokens run as four, the last one masked)
+    uint32_t grid_x;   // workgroups of the launch along x (as an argument: the hidden one would be a fetch of its own)
     static constexpr bool kGrouped = false, kFused = false;
 };
 
@@ -57,6 +58,7 @@ struct StreamFused {
     // 0, or STREAM_PRO_SILU / STREAM_PRO_GELU: W is gate | up stacked (N rows in all, N/2 outputs) and
     // Y[n] = act(gate_n . x) * (up_n . x): a wave takes both rows of a pair, one after the other
     int epi;
+    uint32_t grid_x;   // workgroups of the launch along x
     static constexpr bool kGrouped = false, kFused = true;
 };
 
@@ -93,6 +95,9 @@ __device__ __forceinline__ void stream_select_pair(StreamGrouped& p)
     p.Y += (size_t)pair * p.ldy;
 }
 __device__ __forceinline__ void stream_select_pair(StreamDense&) {}
+__device__ __forceinline__ uint32_t stream_grid_x(const StreamDense& p) { return p.grid_x; }
+__device__ __forceinline__ uint32_t stream_grid_x(const StreamFused& p) { return p.grid_x; }
+template <typename PT> __device__ __forceinline__ uint32_t stream_grid_x(const PT&) { return gridDim.x; }
 __device__ __forceinline__ void stream_select_pair(StreamFused&) {}
 
 // Which prologue a launch runs, where the second activation input lies relative to the first (in
@@ -157,7 +162,7 @@ __device__ __forceinline__ void stream_dispatch_pro(const PT& p, F&& f)
 // each with rows of its own.  KW > 1: the KW waves of a workgroup walk the same rows, one K slice each,
 // and their sums meet in LDS once per 64 rows (the form of the Q6_K kernel below).
 template <int P, int NW, int D, int MT, typename PT, bool Q5 = false, int KW = 1>
-__global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT p)
+__device__ __forceinline__ void q4k_stream_body(PT p)
 {
     stream_select_pair(p);
     __shared__ float part[KW > 1 ? KW : 1][MT][64];
@@ -166,7 +171,7 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
     const uint32_t gw = KW > 1 ? blockIdx.x : blockIdx.x * NW + wave;
     // rows gw, gw + stride, ...: at any moment the waves of the grid read
     // consecutive rows, one contiguous stream across the memory channels
-    const uint32_t stride = KW > 1 ? gridDim.x : gridDim.x * NW;
+    const uint32_t stride = KW > 1 ? stream_grid_x(p) : stream_grid_x(p) * NW;
     // pair mode (fused kernels only): the wave walks pairs gw, gw + stride, ... of the N/2 outputs and its
     // ring alternates between a pair's gate row and its up row, N/2 rows further on
     const bool pairs = PT::kFused && stream_epi(p) != 0;
@@ -351,13 +356,13 @@ __global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT 
 // Workgroup = KW waves, one K slice of 8*P superblocks each; the workgroup walks
 // rows blockIdx.x, + gridDim.x, ...; D rows in flight per wave.
 template <int P, int KW, int D, int MT, typename PT>
-__global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(PT p)
+__device__ __forceinline__ void q6k_stream_body(PT p)
 {
     stream_select_pair(p);
     __shared__ float part[KW > 1 ? KW : 1][MT][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t g = blockIdx.x, stride = gridDim.x;
+    const uint32_t g = blockIdx.x, stride = stream_grid_x(p);
     const uint32_t n_rows = g < p.N ? (p.N - g + stride - 1u) / stride : 0u;
     const uint32_t bl = lane >> 3, t = lane & 7u, n = t >> 2, lg = t & 3u;
     const uint32_t sc_shift = 8u * (lg >> 1);
@@ -510,6 +515,79 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(PT p)
 
 static uint32_t cu_count() { return device_cu_count(); }
 
+// Kernel entries.  The dense decode matvec takes its arguments as scalars (16 dwords): built with kernel-argument
+// preloading (KQ_KERNARG_PRELOAD: the build adds the compiler option for this file) they arrive in scalar registers with the wave, and the kernel starts without the two dependent
+// fetches of an argument struct; the fused and grouped forms keep their structs.
+// (14 dwords are preloaded: what the first instructions need comes first, the bias, read at the stores, last)
+#define KQ_DENSE_PARAMS                                                                                                   \
+    const uint8_t *W, const float *X, float *Y, uint32_t N, uint32_t K, uint32_t n_blocks, uint32_t row_stride_bytes,     \
+        uint32_t grid_x, uint32_t M, uint32_t y_offset, uint32_t ldy, const float *bias
+#define KQ_DENSE_STRUCT StreamDense{X, W, bias, Y, N, K, n_blocks, row_stride_bytes, y_offset, ldy, M, grid_x}
+#define KQ_DENSE_ARGS(p, gx) (p).W, (p).X, (p).Y, (p).N, (p).K, (p).n_blocks, (p).row_stride_bytes, (gx), (p).M, (p).y_offset, (p).ldy, (p).bias
+
+// The fused forms likewise: the 14 preloaded dwords are what the prologue and the first loads need.
+#define KQ_FUSED_PARAMS                                                                                                   \
+    const uint8_t *W, const float *X, uint32_t N, uint32_t K, uint32_t n_blocks, uint32_t row_stride_bytes,               \
+        uint32_t grid_x, const float *norm_w, int pro, int epi, float eps, float *Y, uint32_t M, uint32_t y_offset,       \
+        uint32_t ldy, const float *bias, const float *residual
+#define KQ_FUSED_STRUCT StreamFused{X, W, bias, Y, N, K, n_blocks, row_stride_bytes, y_offset, ldy, M, pro, eps, norm_w, residual, epi, grid_x}
+#define KQ_FUSED_ARGS(p, gx)                                                                                              \
+    (p).W, (p).X, (p).N, (p).K, (p).n_blocks, (p).row_stride_bytes, (gx), (p).norm_w, (p).pro, (p).epi, (p).eps, (p).Y,    \
+        (p).M, (p).y_offset, (p).ldy, (p).bias, (p).residual
+
+template <int P, int NW, int D, int MT, typename PT, bool Q5 = false, int KW = 1>
+__global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT p)
+{
+    q4k_stream_body<P, NW, D, MT, PT, Q5, KW>(p);
+}
+template <int P, int NW, int D, int MT, bool Q5 = false, int KW = 1>
+__global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_fused_kernel(KQ_FUSED_PARAMS)
+{
+    q4k_stream_body<P, NW, D, MT, StreamFused, Q5, KW>(KQ_FUSED_STRUCT);
+}
+template <int P, int KW, int D, int MT>
+__global__ __launch_bounds__(64 * KW) void q6k_stream_fused_kernel(KQ_FUSED_PARAMS)
+{
+    q6k_stream_body<P, KW, D, MT, StreamFused>(KQ_FUSED_STRUCT);
+}
+template <int P, int NW, int D, int MT, bool Q5 = false, int KW = 1>
+__global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_dense_kernel(KQ_DENSE_PARAMS)
+{
+    q4k_stream_body<P, NW, D, MT, StreamDense, Q5, KW>(KQ_DENSE_STRUCT);
+}
+template <int P, int KW, int D, int MT, typename PT>
+__global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(PT p)
+{
+    q6k_stream_body<P, KW, D, MT, PT>(p);
+}
+template <int P, int KW, int D, int MT>
+__global__ __launch_bounds__(64 * KW) void q6k_stream_dense_kernel(KQ_DENSE_PARAMS)
+{
+    q6k_stream_body<P, KW, D, MT, StreamDense>(KQ_DENSE_STRUCT);
+}
+
+// One launch of an instantiation: the scalar-argument entry for dense calls, the struct entry otherwise.
+template <int P, int NW, int D, int MT, bool Q5, int KW, typename PT>
+static void launch_q4k_entry(dim3 grid, dim3 block, hipStream_t s, const PT& p)
+{
+    if constexpr (std::is_same<PT, StreamDense>::value)
+        hipLaunchKernelGGL((q4k_stream_dense_kernel<P, NW, D, MT, Q5, KW>), grid, block, 0, s, KQ_DENSE_ARGS(p, grid.x));
+    else if constexpr (std::is_same<PT, StreamFused>::value)
+        hipLaunchKernelGGL((q4k_stream_fused_kernel<P, NW, D, MT, Q5, KW>), grid, block, 0, s, KQ_FUSED_ARGS(p, grid.x));
+    else
+        hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT, Q5, KW>), grid, block, 0, s, p);
+}
+template <int P, int KW, int D, int MT, typename PT>
+static void launch_q6k_entry(dim3 grid, dim3 block, hipStream_t s, const PT& p)
+{
+    if constexpr (std::is_same<PT, StreamDense>::value)
+        hipLaunchKernelGGL((q6k_stream_dense_kernel<P, KW, D, MT>), grid, block, 0, s, KQ_DENSE_ARGS(p, grid.x));
+    else if constexpr (std::is_same<PT, StreamFused>::value)
+        hipLaunchKernelGGL((q6k_stream_fused_kernel<P, KW, D, MT>), grid, block, 0, s, KQ_FUSED_ARGS(p, grid.x));
+    else
+        hipLaunchKernelGGL((q6k_stream_kernel<P, KW, D, MT, PT>), grid, block, 0, s, p);
+}
+
 // Workgroups for a kernel whose workgroups walk rows g, g + wgs, ...: a whole
 // multiple of the CU count, so that every CU gets the same number of workgroups,
 // at least two rows each so that the activations are not loaded for a single row.
@@ -558,7 +636,7 @@ template <int P, int KW, int D, int MT, typename PT>
 static void launch_q6k_one(dim3 grid, hipStream_t s, const PT& p)
 {
     constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && (D != 2 || (P == 2 && KW == 7 && MT == 2)));
-    if constexpr (!absent) hipLaunchKernelGGL((q6k_stream_kernel<P, KW, D, MT, PT>), grid, dim3(64 * KW), 0, s, p);
+    if constexpr (!absent) launch_q6k_entry<P, KW, D, MT>(grid, dim3(64 * KW), s, p);
 }
 
 // (Q5_K: at most two rows in flight, the third load per pass leaves no registers for four.)
@@ -566,7 +644,7 @@ template <int P, int NW, int D, int MT, typename PT, bool Q5>
 static void launch_q4k_one(dim3 grid, hipStream_t s, const PT& p)
 {
     constexpr bool absent = (PT::kGrouped && MT == 2) || (PT::kFused && (D == 1 || (D == 4 && MT == 2))) || (Q5 && D > 2);
-    if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT, Q5>), grid, dim3(64 * NW), 0, s, p);
+    if constexpr (!absent) launch_q4k_entry<P, NW, D, MT, Q5, 1>(grid, dim3(64 * NW), s, p);
 }
 
 // Rows longer than 16 superblocks: K slices over KW waves, two rows in flight, dense and fused calls.
@@ -574,7 +652,7 @@ template <int P, int KW, int MT, typename PT, bool Q5>
 static void launch_q4k_sliced(dim3 grid, hipStream_t s, const PT& p)
 {
     constexpr bool absent = PT::kGrouped || (P == 2 && KW == 7 && MT == 2 && (PT::kFused || Q5));
-    if constexpr (!absent) hipLaunchKernelGGL((q4k_stream_kernel<P, 1, 2, MT, PT, Q5, KW>), grid, dim3(64 * KW), 0, s, p);
+    if constexpr (!absent) launch_q4k_entry<P, 1, 2, MT, Q5, KW>(grid, dim3(64 * KW), s, p);
 }
 
 // Three or four tokens (dense calls): every wave holds a K slice of eight superblocks for four tokens (128
@@ -588,20 +666,20 @@ static hipError_t launch_stream_four(const MatmulArgs& a, hipStream_t s, const P
     const uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 8u / (uint32_t)kw, 0);
     const dim3 grid(wgs, 1, 1);
     if (a.type == KQ_TYPE_Q6_K) {
-        if (kw == 1) hipLaunchKernelGGL((q6k_stream_kernel<1, 1, 2, 4, PT>), grid, dim3(64), 0, s, p);
-        else if (kw == 2) hipLaunchKernelGGL((q6k_stream_kernel<1, 2, 2, 4, PT>), grid, dim3(128), 0, s, p);
-        else if (kw == 4) hipLaunchKernelGGL((q6k_stream_kernel<1, 4, 2, 4, PT>), grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL((q6k_stream_kernel<1, 7, 2, 4, PT>), grid, dim3(448), 0, s, p);
+        if (kw == 1) launch_q6k_entry<1, 1, 2, 4>(grid, dim3(64), s, p);
+        else if (kw == 2) launch_q6k_entry<1, 2, 2, 4>(grid, dim3(128), s, p);
+        else if (kw == 4) launch_q6k_entry<1, 4, 2, 4>(grid, dim3(256), s, p);
+        else launch_q6k_entry<1, 7, 2, 4>(grid, dim3(448), s, p);
     } else if (a.type == KQ_TYPE_Q5_K) {
-        if (kw == 1) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, true, 1>), grid, dim3(64), 0, s, p);
-        else if (kw == 2) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, true, 2>), grid, dim3(128), 0, s, p);
-        else if (kw == 4) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, true, 4>), grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, true, 7>), grid, dim3(448), 0, s, p);
+        if (kw == 1) launch_q4k_entry<1, 1, 2, 4, true, 1>(grid, dim3(64), s, p);
+        else if (kw == 2) launch_q4k_entry<1, 1, 2, 4, true, 2>(grid, dim3(128), s, p);
+        else if (kw == 4) launch_q4k_entry<1, 1, 2, 4, true, 4>(grid, dim3(256), s, p);
+        else launch_q4k_entry<1, 1, 2, 4, true, 7>(grid, dim3(448), s, p);
     } else {
-        if (kw == 1) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 1>), grid, dim3(64), 0, s, p);
-        else if (kw == 2) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 2>), grid, dim3(128), 0, s, p);
-        else if (kw == 4) hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 4>), grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL((q4k_stream_kernel<1, 1, 2, 4, PT, false, 7>), grid, dim3(448), 0, s, p);
+        if (kw == 1) launch_q4k_entry<1, 1, 2, 4, false, 1>(grid, dim3(64), s, p);
+        else if (kw == 2) launch_q4k_entry<1, 1, 2, 4, false, 2>(grid, dim3(128), s, p);
+        else if (kw == 4) launch_q4k_entry<1, 1, 2, 4, false, 4>(grid, dim3(256), s, p);
+        else launch_q4k_entry<1, 1, 2, 4, false, 7>(grid, dim3(448), s, p);
     }
     return hipGetLastError();
 }
@@ -692,7 +770,7 @@ static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, h
         const bool eight = t.waves == 8 || (t.waves == 0 && t.depth == 0 && t.splits == 0 && a.N >= 8u * 8u * cu_count());
         if (eight && !q5 && !two && a.n_blocks > 8u) {
             const uint32_t wgs8 = stream_workgroups((a.N + 7u) / 8u, 1u, 0);
-            hipLaunchKernelGGL((q4k_stream_kernel<2, 8, 2, 1, PT, false>), dim3(wgs8, 1, 1), dim3(512), 0, s, p);
+            launch_q4k_entry<2, 8, 2, 1, false, 1>(dim3(wgs8, 1, 1), dim3(512), s, p);
             return hipGetLastError();
         }
     }
@@ -745,10 +823,12 @@ hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStrea
         p.norm_w = a.norm_w;
         p.residual = a.residual;
         p.epi = a.epi;
+        p.grid_x = 0;   // (the launch passes its own grid size)
         return launch_stream_with(a, t, s, p, 1u, 1u);
     }
     StreamDense p;
     stream_fill_common(p, a);
+    p.grid_x = 0;
     return launch_stream_with(a, t, s, p, 1u, 1u);
 }
 
