@@ -121,6 +121,15 @@ __device__ __forceinline__ uint32_t stream_ldx(const StreamFused& p) { return p.
 __device__ __forceinline__ uint32_t stream_ldx(const StreamGrouped& p) { return p.K; }
 
 
+// v where mask is all ones, +0 where it is zero (bitwise: no branch, no NaN from a product with zero)
+__device__ __forceinline__ float4 stream_keep(float4 v, uint32_t mask)
+{
+    return float4{__builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v.x) & mask),
+                  __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v.y) & mask),
+                  __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v.z) & mask),
+                  __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v.w) & mask)};
+}
+
 // Four activations: X as it is (also for the norm, which scales afterwards), or act(X) * X2.
 template <int PRO, bool FAST>
 __device__ __forceinline__ float4 stream_x4(const float4* xp, ptrdiff_t x2_off)
@@ -199,6 +208,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
         for (int pass = 0; pass < P; ++pass) {
             uint32_t b = ((KW > 1 ? wave * P : 0u) + pass) * 8u + bl;
             const bool valid = b < p.n_blocks;
+            const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;   // activations of superblocks beyond K read as zero
             b = valid ? b : p.n_blocks - 1u;
             hoff[pass] = b * BLOCK;
 #pragma unroll
@@ -208,7 +218,8 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float4 lo = stream_x4<PRO, PT::kFused>(xp + i, x2_off), hi = stream_x4<PRO, PT::kFused>(xp + 8 + i, x2_off);
-                    if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
+                    lo = stream_keep(lo, keep);   // (no branch here: one around a load makes every load wait for the one before)
+                    hi = stream_keep(hi, keep);
                     xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
                     xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
                 }
@@ -271,6 +282,11 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
     // fetched and summed again (cache hits, result dropped), so the row loop has
     // no branch and the number of loads in flight is the same at every wait.
     constexpr int SLOT_LOADS = (Q5 ? 3 : 2) * P;
+    // (the activation sums are finished before the first weight is requested)
+#pragma unroll
+    for (int pass = 0; pass < P; ++pass)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) asm volatile("" ::"v"(xs_lo[pass][t]), "v"(xs_hi[pass][t]));
     Q4Slot<P, Q5> ring[D] = {};
     // (The ring is filled after the prologue even where that is long: registers with a load in flight
     // must stay where they are, and across the prologue's arithmetic the compiler moves them.)
@@ -377,6 +393,7 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
         for (int pass = 0; pass < P; ++pass) {
             uint32_t b = (wave * P + pass) * 8u + bl;
             const bool valid = b < p.n_blocks;
+            const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;   // activations of superblocks beyond K read as zero
             b = valid ? b : p.n_blocks - 1u;
             boff[pass] = b * KQ_Q6K_BYTES;
 #pragma unroll
@@ -386,7 +403,8 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     float4 lo = stream_x4<PRO, PT::kFused>(xp + 8 * k, x2_off), hi = stream_x4<PRO, PT::kFused>(xp + 8 * k + 1, x2_off);
-                    if (!valid) { lo = float4{0, 0, 0, 0}; hi = lo; }
+                    lo = stream_keep(lo, keep);
+                    hi = stream_keep(hi, keep);
                     x[pass][tk][k][0] = lo.x; x[pass][tk][k][1] = lo.y; x[pass][tk][k][2] = lo.z; x[pass][tk][k][3] = lo.w;
                     x[pass][tk][k][4] = hi.x; x[pass][tk][k][5] = hi.y; x[pass][tk][k][6] = hi.z; x[pass][tk][k][7] = hi.w;
                     if constexpr (PRO != STREAM_PRO_NORM) {
