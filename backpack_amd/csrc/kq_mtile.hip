@@ -642,7 +642,7 @@ struct MtileWStage {
 // (the grouped Q4_K kernel is held to 128 registers so that two of its workgroups share a CU)
 // FUSED: residual and pair epilogue; PRO: the prologue (1 RMSNorm, 2 act(gate) * up)
 template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0, bool HL8 = false>
-__global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1) void mtile_kernel(MtileParams p)
+__device__ __forceinline__ void mtile_body(const MtileParams& p)
 // (Q5_K: the Q4_K code with blocks of 176 bytes — header, 32 bytes of fifth bits, quants — and one more
 // 8-byte piece per lane and superblock)
 {
@@ -999,6 +999,43 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
     put_tile(row, tot);
 }
 
+// Kernel entry.  What the first instructions need travels as scalars (KQ_KERNARG_PRELOAD: 14 dwords arrive in
+// scalar registers with the wave), the rest as a struct that is fetched when it is used.
+struct MtileRest {
+    const float* bias;
+    float* Y;
+    uint32_t y_offset, ldy;
+    float* partial;
+    uint32_t* counters;
+    int pro, epi;
+    float eps;
+    const float* norm_w;
+    const float* residual;
+    uint32_t pair_tile0;
+    const uint32_t* n_tiles;
+    uint32_t tile_iters, tile_stride, k_slots;
+    int x_per_slot;
+};
+
+template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0, bool HL8 = false>
+__global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1) void mtile_kernel(
+    const uint8_t* W, const float* X, const uint32_t* tiles, uint32_t M, uint32_t N, uint32_t K, uint32_t n_blocks,
+    uint32_t row_stride_bytes, uint32_t tiles_per_wg, uint32_t chunks_per_split, uint32_t n_splits, uint32_t x_stride,
+    MtileRest r)
+{
+    MtileParams p;
+    p.X = X; p.W = W; p.bias = r.bias; p.Y = r.Y;
+    p.M = M; p.N = N; p.K = K; p.n_blocks = n_blocks; p.row_stride_bytes = row_stride_bytes;
+    p.y_offset = r.y_offset; p.ldy = r.ldy;
+    p.tiles_per_wg = tiles_per_wg; p.n_splits = n_splits; p.chunks_per_split = chunks_per_split;
+    p.partial = r.partial; p.counters = r.counters;
+    p.pro = r.pro; p.epi = r.epi; p.eps = r.eps; p.norm_w = r.norm_w; p.residual = r.residual;
+    p.x_stride = x_stride; p.pair_tile0 = r.pair_tile0;
+    p.tiles = tiles; p.n_tiles = r.n_tiles; p.tile_iters = r.tile_iters; p.tile_stride = r.tile_stride;
+    p.k_slots = r.k_slots; p.x_per_slot = r.x_per_slot;
+    mtile_body<TYPE, NW, R, STAGED, TOK, FUSED, PRO, HL8>(p);
+}
+
 bool mtile_supported(const MatmulArgs& a)
 {
     // dense calls of more than 16 tokens run as groups of 16 (8 for Q6_K), each reading the weights again:
@@ -1025,7 +1062,10 @@ static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t 
         if (e != hipSuccess) return e;
         raised = true;
     }
-    hipLaunchKernelGGL(kern, dim3(wgs, wgs_y, wgs_z), dim3(64 * NW), shmem, s, p);
+    const MtileRest r{p.bias, p.Y, p.y_offset, p.ldy, p.partial, p.counters, p.pro, p.epi, p.eps, p.norm_w, p.residual,
+                      p.pair_tile0, p.n_tiles, p.tile_iters, p.tile_stride, p.k_slots, p.x_per_slot};
+    hipLaunchKernelGGL(kern, dim3(wgs, wgs_y, wgs_z), dim3(64 * NW), shmem, s, p.W, p.X, p.tiles, p.M, p.N, p.K, p.n_blocks,
+                       p.row_stride_bytes, p.tiles_per_wg, p.chunks_per_split, p.n_splits, p.x_stride, r);
     return hipGetLastError();
 }
 
