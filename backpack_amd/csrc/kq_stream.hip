@@ -95,6 +95,11 @@ __device__ __forceinline__ void stream_select_pair(StreamGrouped& p)
     p.Y += (size_t)pair * p.ldy;
 }
 __device__ __forceinline__ void stream_select_pair(StreamDense&) {}
+__device__ __forceinline__ void stream_touch_late_args(const StreamFused& p)
+{
+    asm volatile("" ::"s"(p.Y), "s"(p.bias), "s"(p.residual), "s"(p.ldy), "s"(p.y_offset));
+}
+template <typename PT> __device__ __forceinline__ void stream_touch_late_args(const PT&) {}
 __device__ __forceinline__ uint32_t stream_grid_x(const StreamDense& p) { return p.grid_x; }
 __device__ __forceinline__ uint32_t stream_grid_x(const StreamFused& p) { return p.grid_x; }
 template <typename PT> __device__ __forceinline__ uint32_t stream_grid_x(const PT&) { return gridDim.x; }
@@ -293,6 +298,8 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
 #pragma unroll
     for (int d = 0; d < D; ++d)
         ring[d].fill(p.W + row_of((uint32_t)d) * p.row_stride_bytes, hoff, j);
+    // (arguments beyond the preloaded ones are fetched now, under the first weights' flight, not at the stores)
+    stream_touch_late_args(p);
     // Rows are taken 64 at a time: lane i keeps the sums of the chunk's row i, and the
     // chunk is stored (bias added) after its last row.
     for (uint32_t c0 = 0; c0 < n_rows; c0 += 64u) {
@@ -476,6 +483,7 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
 #pragma unroll
     for (int d = 0; d < D; ++d)
         ring[d].fill(p.W + (size_t)(g + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, boff, n, lg);
+    stream_touch_late_args(p);
     // Rows are taken 64 at a time: lane i keeps the sums of the chunk's row i; the K
     // slices are folded and the chunk stored after its last row.  The row loop is
     // the one of the Q4_K kernel.
@@ -536,12 +544,13 @@ static uint32_t cu_count() { return device_cu_count(); }
 // Kernel entries.  The dense decode matvec takes its arguments as scalars (16 dwords): built with kernel-argument
 // preloading (KQ_KERNARG_PRELOAD: the build adds the compiler option for this file) they arrive in scalar registers with the wave, and the kernel starts without the two dependent
 // fetches of an argument struct; the fused and grouped forms keep their structs.
-// (14 dwords are preloaded: what the first instructions need comes first, the bias, read at the stores, last)
+// (14 dwords are preloaded: everything one token needs — a pointer fetched at the stores would cost every wave a
+// round trip at its end; Y arrives with the output offset added; M, read by the four-token kernels only, is the 15th)
 #define KQ_DENSE_PARAMS                                                                                                   \
-    const uint8_t *W, const float *X, float *Y, uint32_t N, uint32_t K, uint32_t n_blocks, uint32_t row_stride_bytes,     \
-        uint32_t grid_x, uint32_t M, uint32_t y_offset, uint32_t ldy, const float *bias
-#define KQ_DENSE_STRUCT StreamDense{X, W, bias, Y, N, K, n_blocks, row_stride_bytes, y_offset, ldy, M, grid_x}
-#define KQ_DENSE_ARGS(p, gx) (p).W, (p).X, (p).Y, (p).N, (p).K, (p).n_blocks, (p).row_stride_bytes, (gx), (p).M, (p).y_offset, (p).ldy, (p).bias
+    const uint8_t *W, const float *X, float *Y, const float *bias, uint32_t N, uint32_t K, uint32_t n_blocks,             \
+        uint32_t row_stride_bytes, uint32_t grid_x, uint32_t ldy, uint32_t M
+#define KQ_DENSE_STRUCT StreamDense{X, W, bias, Y, N, K, n_blocks, row_stride_bytes, 0u, ldy, M, grid_x}
+#define KQ_DENSE_ARGS(p, gx) (p).W, (p).X, (p).Y + (p).y_offset, (p).bias, (p).N, (p).K, (p).n_blocks, (p).row_stride_bytes, (gx), (p).ldy, (p).M
 
 // The fused forms likewise: the 14 preloaded dwords are what the prologue and the first loads need.
 #define KQ_FUSED_PARAMS                                                                                                   \
