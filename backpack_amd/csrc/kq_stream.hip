@@ -190,8 +190,15 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
     // ring alternates between a pair's gate row and its up row, N/2 rows further on
     const bool pairs = PT::kFused && stream_epi(p) != 0;
     const uint32_t n_walk_all = pairs ? p.N / 2u : p.N;
-    if (gw >= n_walk_all) return;   // KW > 1: the whole workgroup
-    const uint32_t n_walk = (n_walk_all - gw + stride - 1u) / stride;
+    // STAGE (whole-row waves, several to a workgroup): the workgroup fetches the activations once and its waves
+    // take their operands from LDS; every wave loading the row for itself costs a CU's vector cache eight times
+    // the bytes (16 KB per wave and token, twice that with norm weights: 1 to 3 us of a launch).
+    constexpr bool STAGE = KW == 1 && NW > 1;
+    __shared__ float4 xstage[STAGE ? MT * P * 8 * 64 : 1];
+    __shared__ float ssq_part[STAGE ? NW : 1][MT];
+    const bool idle = gw >= n_walk_all;   // KW > 1: the whole workgroup
+    if (!STAGE && idle) return;
+    const uint32_t n_walk = idle ? 0u : (n_walk_all - gw + stride - 1u) / stride;
     const uint32_t n_rows = pairs ? 2u * n_walk : n_walk;
     auto row_of = [&](uint32_t i) -> size_t {
         i = min(i, n_rows - 1u);
@@ -207,8 +214,76 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
     uint32_t hoff[P];
     const uint32_t ldx = stream_ldx(p);
     const ptrdiff_t x2_off = stream_x2_off(p);
+    // RMSNorm prologue: the activations are held as x * norm_w (both loaded back to back: one round trip
+    // to memory, not two) and the row's 1/rms, which needs the whole row, scales the finished outputs.
+    float rstd0 = 1.0f, rstd1 = 1.0f;   // (the fused forms take one or two tokens; two scalars: an array went to scratch memory)
     auto load_x = [&](auto pro) {
         constexpr int PRO = decltype(pro)::value;
+        constexpr bool NORM = PRO == STREAM_PRO_NORM && PT::kFused;
+        float ssq[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) ssq[t] = 0.0f;
+        if constexpr (STAGE) {
+            // Slot sl = 8 * pass + q of the staging area holds, for lane L, the q-th 16 bytes of that lane's
+            // operands of the pass (q < 4: low nibbles' elements, else high nibbles'): wave w fetches slots
+            // w, w + NW, ... exactly as the lane would have, and a wave's reads are 1 KB runs.
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+#pragma unroll
+                for (int k = 0; k < P * 8 / NW; ++k) {
+                    const uint32_t sl = wave + (uint32_t)k * NW, q = sl & 7u;
+                    uint32_t b = (sl >> 3) * 8u + bl;
+                    const bool valid = b < p.n_blocks;
+                    const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;   // activations of superblocks beyond K read as zero
+                    b = valid ? b : p.n_blocks - 1u;
+                    const size_t at = (size_t)b * KQ_QK + 64u * g + 16u * h + 32u * (q >> 2) + 4u * (q & 3u);
+                    float4 v = stream_x4<PRO, PT::kFused>((const float4*)(p.X + (size_t)t * ldx + at), x2_off);
+                    v = stream_keep(v, keep);
+                    if constexpr (NORM) {
+                        const float4 w = *(const float4*)(stream_norm_w(p) + at);
+                        ssq[t] = __builtin_fmaf(v.x, v.x, __builtin_fmaf(v.y, v.y, __builtin_fmaf(v.z, v.z, __builtin_fmaf(v.w, v.w, ssq[t]))));
+                        v.x *= w.x; v.y *= w.y; v.z *= w.z; v.w *= w.w;
+                    }
+                    xstage[((uint32_t)t * P * 8u + sl) * 64u + lane] = v;
+                }
+                if constexpr (NORM) {
+                    const float ss = wave_sum(ssq[t]);
+                    if (lane == 0) ssq_part[wave][t] = ss;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int pass = 0; pass < P; ++pass) {
+                const uint32_t b = min((uint32_t)pass * 8u + bl, p.n_blocks - 1u);
+                hoff[pass] = b * BLOCK;
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float4 lo = xstage[((uint32_t)t * P * 8u + pass * 8u + i) * 64u + lane];
+                        const float4 hi = xstage[((uint32_t)t * P * 8u + pass * 8u + 4u + i) * 64u + lane];
+                        xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
+                        xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
+                    }
+                    float sl = 0.0f, sh_ = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
+                    xs_lo[pass][t] = sl;
+                    xs_hi[pass][t] = sh_;
+                }
+            }
+            if constexpr (NORM) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    float ss = ssq_part[0][t];
+#pragma unroll
+                    for (int w = 1; w < NW; ++w) ss += ssq_part[w][t];
+                    const float r = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
+                    if (t == 0) rstd0 = r; else rstd1 = r;
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int pass = 0; pass < P; ++pass) {
             uint32_t b = ((KW > 1 ? wave * P : 0u) + pass) * 8u + bl;
@@ -225,61 +300,47 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
                     float4 lo = stream_x4<PRO, PT::kFused>(xp + i, x2_off), hi = stream_x4<PRO, PT::kFused>(xp + 8 + i, x2_off);
                     lo = stream_keep(lo, keep);   // (no branch here: one around a load makes every load wait for the one before)
                     hi = stream_keep(hi, keep);
+                    if constexpr (NORM) {
+                        const float4* wp = (const float4*)(stream_norm_w(p) + (size_t)b * KQ_QK + 64u * g + 16u * h);
+                        const float4 wl = wp[i], wh = wp[8 + i];
+                        float s = ssq[t];
+                        s = __builtin_fmaf(lo.x, lo.x, s); s = __builtin_fmaf(lo.y, lo.y, s);
+                        s = __builtin_fmaf(lo.z, lo.z, s); s = __builtin_fmaf(lo.w, lo.w, s);
+                        s = __builtin_fmaf(hi.x, hi.x, s); s = __builtin_fmaf(hi.y, hi.y, s);
+                        s = __builtin_fmaf(hi.z, hi.z, s); s = __builtin_fmaf(hi.w, hi.w, s);
+                        ssq[t] = s;
+                        lo.x *= wl.x; lo.y *= wl.y; lo.z *= wl.z; lo.w *= wl.w;
+                        hi.x *= wh.x; hi.y *= wh.y; hi.z *= wh.z; hi.w *= wh.w;
+                    }
                     xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
                     xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
                 }
-                if constexpr (PRO != STREAM_PRO_NORM) {
-                    float sl = 0.0f, sh_ = 0.0f;
+                float sl = 0.0f, sh_ = 0.0f;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
-                    xs_lo[pass][t] = sl;
-                    xs_hi[pass][t] = sh_;
-                }
+                for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
+                xs_lo[pass][t] = sl;
+                xs_hi[pass][t] = sh_;
             }
         }
-        if constexpr (PRO == STREAM_PRO_NORM && PT::kFused) {
-            // the wave holds the whole row: its sum of squares is one reduction away
+        if constexpr (NORM) {
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                float ss = 0.0f;
-#pragma unroll
-                for (int pass = 0; pass < P; ++pass)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i)
-                        ss = __builtin_fmaf(xlo[pass][t][i], xlo[pass][t][i], __builtin_fmaf(xhi[pass][t][i], xhi[pass][t][i], ss));
-                ss = wave_sum(ss);
-                if (KW > 1) {   // the slices' sums of squares meet in LDS
+                float ss = wave_sum(ssq[t]);   // the wave holds the whole row, or a K slice of it
+                if (KW > 1) {                  // the slices' sums of squares meet in LDS
                     if (lane == 0) part[wave][t][0] = ss;
                     __syncthreads();
                     ss = part[0][t][0];
 #pragma unroll
                     for (int w = 1; w < KW; ++w) ss += part[w][t][0];
                 }
-                const float rstd = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
-#pragma unroll
-                for (int pass = 0; pass < P; ++pass) {
-                    const float* wp = stream_norm_w(p) + hoff[pass] / BLOCK * KQ_QK + 64u * g + 16u * h;
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        xlo[pass][t][i] = xlo[pass][t][i] * rstd * wp[i];
-                        xhi[pass][t][i] = xhi[pass][t][i] * rstd * wp[32 + i];
-                    }
-                }
+                const float r = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
+                if (t == 0) rstd0 = r; else rstd1 = r;
             }
             if (KW > 1) __syncthreads();   // part is reused by the row loop
-#pragma unroll
-            for (int pass = 0; pass < P; ++pass)
-#pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    float sl = 0.0f, sh_ = 0.0f;
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
-                    xs_lo[pass][t] = sl;
-                    xs_hi[pass][t] = sh_;
-                }
         }
     };
     stream_dispatch_pro(p, load_x);
+    if (STAGE && idle) return;
 
     // Ring of D rows in flight.  Slot d is refilled as soon as its row has been
     // consumed; the wait before a slot's arithmetic leaves the (D-1) younger
@@ -345,6 +406,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
 #pragma unroll
                     for (int w = 1; w < KW; ++w) y += part[w][t][lane];
                 }
+                if constexpr (PT::kFused) y *= t == 0 ? rstd0 : rstd1;
                 y += bias;
                 if (PT::kFused && pairs) {
                     // lanes 2j and 2j + 1 hold a pair's gate and up products: the even lane stores the output
@@ -394,8 +456,14 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
     uint32_t boff[P];
     const uint32_t ldx = stream_ldx(p);
     const ptrdiff_t x2_off = stream_x2_off(p);
+    // (RMSNorm prologue as in the Q4_K kernel: x * norm_w in one round trip, 1/rms on the outputs)
+    float rstd0 = 1.0f, rstd1 = 1.0f;   // (the fused forms take one or two tokens; two scalars: an array went to scratch memory)
     auto load_x = [&](auto pro) {
         constexpr int PRO = decltype(pro)::value;
+        constexpr bool NORM = PRO == STREAM_PRO_NORM && PT::kFused;
+        float ssq[MT];
+#pragma unroll
+        for (int tk = 0; tk < MT; ++tk) ssq[tk] = 0.0f;
 #pragma unroll
         for (int pass = 0; pass < P; ++pass) {
             uint32_t b = (wave * P + pass) * 8u + bl;
@@ -412,29 +480,31 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
                     float4 lo = stream_x4<PRO, PT::kFused>(xp + 8 * k, x2_off), hi = stream_x4<PRO, PT::kFused>(xp + 8 * k + 1, x2_off);
                     lo = stream_keep(lo, keep);
                     hi = stream_keep(hi, keep);
+                    if constexpr (NORM) {
+                        const float4* wp = (const float4*)(stream_norm_w(p) + (size_t)b * KQ_QK + 128u * n + 8u * lg);
+                        const float4 wl = wp[8 * k], wh = wp[8 * k + 1];
+                        float s = ssq[tk];
+                        s = __builtin_fmaf(lo.x, lo.x, s); s = __builtin_fmaf(lo.y, lo.y, s);
+                        s = __builtin_fmaf(lo.z, lo.z, s); s = __builtin_fmaf(lo.w, lo.w, s);
+                        s = __builtin_fmaf(hi.x, hi.x, s); s = __builtin_fmaf(hi.y, hi.y, s);
+                        s = __builtin_fmaf(hi.z, hi.z, s); s = __builtin_fmaf(hi.w, hi.w, s);
+                        ssq[tk] = s;
+                        lo.x *= wl.x; lo.y *= wl.y; lo.z *= wl.z; lo.w *= wl.w;
+                        hi.x *= wh.x; hi.y *= wh.y; hi.z *= wh.z; hi.w *= wh.w;
+                    }
                     x[pass][tk][k][0] = lo.x; x[pass][tk][k][1] = lo.y; x[pass][tk][k][2] = lo.z; x[pass][tk][k][3] = lo.w;
                     x[pass][tk][k][4] = hi.x; x[pass][tk][k][5] = hi.y; x[pass][tk][k][6] = hi.z; x[pass][tk][k][7] = hi.w;
-                    if constexpr (PRO != STREAM_PRO_NORM) {
-                        float sum = 0.0f;
+                    float sum = 0.0f;
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) sum += x[pass][tk][k][i];
-                        m32xs[pass][tk][k] = -32.0f * sum;
-                    }
+                    for (int i = 0; i < 8; ++i) sum += x[pass][tk][k][i];
+                    m32xs[pass][tk][k] = -32.0f * sum;
                 }
             }
         }
-        if constexpr (PRO == STREAM_PRO_NORM && PT::kFused) {
-            // each wave holds a K slice: the slices' sums of squares meet in LDS
+        if constexpr (NORM) {
 #pragma unroll
             for (int tk = 0; tk < MT; ++tk) {
-                float ss = 0.0f;
-#pragma unroll
-                for (int pass = 0; pass < P; ++pass)
-#pragma unroll
-                    for (int k = 0; k < 4; ++k)
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) ss = __builtin_fmaf(x[pass][tk][k][i], x[pass][tk][k][i], ss);
-                ss = wave_sum(ss);
+                float ss = wave_sum(ssq[tk]);   // each wave holds a K slice: the slices' sums of squares meet in LDS
                 if (KW > 1) {
                     if (lane == 0) part[wave][tk][0] = ss;
                     __syncthreads();
@@ -442,28 +512,10 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
 #pragma unroll
                     for (int w = 1; w < KW; ++w) ss += part[w][tk][0];
                 }
-                const float rstd = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
-#pragma unroll
-                for (int pass = 0; pass < P; ++pass) {
-                    const float* wp = stream_norm_w(p) + boff[pass] / KQ_Q6K_BYTES * KQ_QK + 128u * n + 8u * lg;
-#pragma unroll
-                    for (int k = 0; k < 4; ++k)
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) x[pass][tk][k][i] = x[pass][tk][k][i] * rstd * wp[32 * k + i];
-                }
+                const float r = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
+                if (tk == 0) rstd0 = r; else rstd1 = r;
             }
             if (KW > 1) __syncthreads();   // part is reused by the row loop
-#pragma unroll
-            for (int pass = 0; pass < P; ++pass)
-#pragma unroll
-                for (int tk = 0; tk < MT; ++tk)
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        float sum = 0.0f;
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) sum += x[pass][tk][k][i];
-                        m32xs[pass][tk][k] = -32.0f * sum;
-                    }
         }
     };
     stream_dispatch_pro(p, load_x);
@@ -529,6 +581,7 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
                 }
                 if (MT > 2 && (uint32_t)tk >= p.M) continue;
                 const size_t at = (size_t)tk * p.ldy + p.y_offset + r;
+                if constexpr (PT::kFused) y *= tk == 0 ? rstd0 : rstd1;
                 y += bias;
                 if constexpr (PT::kFused) y += stream_residual(p) ? stream_residual(p)[at] : 0.0f;
                 p.Y[at] = y;
@@ -790,7 +843,7 @@ static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, h
         else if (two) launch_q4k_one<P, NW, D, 2, PT, false>(grid, s, p); \
         else launch_q4k_one<P, NW, D, 1, PT, false>(grid, s, p); \
     } while (0)
-    if constexpr (!PT::kGrouped && !PT::kFused) {
+    if constexpr (!PT::kGrouped) {
         // Matrices that give every wave eight rows or more (gate|up: 28672 x 4096) run faster as eight waves
         // per workgroup with two rows in flight each than as four with four: 15.3 against 16.8 us there.
         // Shorter walks lose with it (6144 x 4096: 7.8 against 7.3 us), so they keep the four-wave form.
