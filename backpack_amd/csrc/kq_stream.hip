@@ -150,7 +150,13 @@ __device__ __forceinline__ float4 stream_x4(const float4* xp, ptrdiff_t x2_off)
     return v;
 }
 
-// One branch around a whole x prologue, so that every form issues its loads back to back.
+// A workgroup barrier that waits for the wave's LDS traffic only (__syncthreads also drains the vector memory
+// counter, i.e. the ring of weight rows in flight).
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // One branch around a whole x prologue, so that every form issues its loads back to back.  A kernel
 // carries only the forms its argument set can ask for.
 template <typename PT, typename F>
@@ -182,7 +188,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
     __shared__ float part[KW > 1 ? KW : 1][MT][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t gw = KW > 1 ? blockIdx.x : blockIdx.x * NW + wave;
+    const uint32_t gw0 = KW > 1 ? blockIdx.x : blockIdx.x * NW + wave;
     // rows gw, gw + stride, ...: at any moment the waves of the grid read
     // consecutive rows, one contiguous stream across the memory channels
     const uint32_t stride = KW > 1 ? stream_grid_x(p) : stream_grid_x(p) * NW;
@@ -196,9 +202,10 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
     constexpr bool STAGE = KW == 1 && NW > 1;
     __shared__ float4 xstage[STAGE ? MT * P * 8 * 64 : 1];
     __shared__ float ssq_part[STAGE ? NW : 1][MT];
-    const bool idle = gw >= n_walk_all;   // KW > 1: the whole workgroup
+    const bool idle = gw0 >= n_walk_all;   // KW > 1: the whole workgroup
     if (!STAGE && idle) return;
-    const uint32_t n_walk = idle ? 0u : (n_walk_all - gw + stride - 1u) / stride;
+    const uint32_t gw = idle ? 0u : gw0;   // (a staged workgroup's idle waves help fetch the activations, then leave)
+    const uint32_t n_walk = (n_walk_all - gw + stride - 1u) / stride;
     const uint32_t n_rows = pairs ? 2u * n_walk : n_walk;
     auto row_of = [&](uint32_t i) -> size_t {
         i = min(i, n_rows - 1u);
@@ -223,67 +230,6 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
         float ssq[MT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) ssq[t] = 0.0f;
-        if constexpr (STAGE) {
-            // Slot sl = 8 * pass + q of the staging area holds, for lane L, the q-th 16 bytes of that lane's
-            // operands of the pass (q < 4: low nibbles' elements, else high nibbles'): wave w fetches slots
-            // w, w + NW, ... exactly as the lane would have, and a wave's reads are 1 KB runs.
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-#pragma unroll
-                for (int k = 0; k < P * 8 / NW; ++k) {
-                    const uint32_t sl = wave + (uint32_t)k * NW, q = sl & 7u;
-                    uint32_t b = (sl >> 3) * 8u + bl;
-                    const bool valid = b < p.n_blocks;
-                    const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;   // activations of superblocks beyond K read as zero
-                    b = valid ? b : p.n_blocks - 1u;
-                    const size_t at = (size_t)b * KQ_QK + 64u * g + 16u * h + 32u * (q >> 2) + 4u * (q & 3u);
-                    float4 v = stream_x4<PRO, PT::kFused>((const float4*)(p.X + (size_t)t * ldx + at), x2_off);
-                    v = stream_keep(v, keep);
-                    if constexpr (NORM) {
-                        const float4 w = *(const float4*)(stream_norm_w(p) + at);
-                        ssq[t] = __builtin_fmaf(v.x, v.x, __builtin_fmaf(v.y, v.y, __builtin_fmaf(v.z, v.z, __builtin_fmaf(v.w, v.w, ssq[t]))));
-                        v.x *= w.x; v.y *= w.y; v.z *= w.z; v.w *= w.w;
-                    }
-                    xstage[((uint32_t)t * P * 8u + sl) * 64u + lane] = v;
-                }
-                if constexpr (NORM) {
-                    const float ss = wave_sum(ssq[t]);
-                    if (lane == 0) ssq_part[wave][t] = ss;
-                }
-            }
-            __syncthreads();
-#pragma unroll
-            for (int pass = 0; pass < P; ++pass) {
-                const uint32_t b = min((uint32_t)pass * 8u + bl, p.n_blocks - 1u);
-                hoff[pass] = b * BLOCK;
-#pragma unroll
-                for (int t = 0; t < MT; ++t) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float4 lo = xstage[((uint32_t)t * P * 8u + pass * 8u + i) * 64u + lane];
-                        const float4 hi = xstage[((uint32_t)t * P * 8u + pass * 8u + 4u + i) * 64u + lane];
-                        xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
-                        xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
-                    }
-                    float sl = 0.0f, sh_ = 0.0f;
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
-                    xs_lo[pass][t] = sl;
-                    xs_hi[pass][t] = sh_;
-                }
-            }
-            if constexpr (NORM) {
-#pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    float ss = ssq_part[0][t];
-#pragma unroll
-                    for (int w = 1; w < NW; ++w) ss += ssq_part[w][t];
-                    const float r = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
-                    if (t == 0) rstd0 = r; else rstd1 = r;
-                }
-            }
-            return;
-        }
 #pragma unroll
         for (int pass = 0; pass < P; ++pass) {
             uint32_t b = ((KW > 1 ? wave * P : 0u) + pass) * 8u + bl;
@@ -339,28 +285,140 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
             if (KW > 1) __syncthreads();   // part is reused by the row loop
         }
     };
-    stream_dispatch_pro(p, load_x);
-    if (STAGE && idle) return;
-
     // Ring of D rows in flight.  Slot d is refilled as soon as its row has been
     // consumed; the wait before a slot's arithmetic leaves the (D-1) younger
     // slots' loads outstanding.  Past the end of the wave's rows the last row is
     // fetched and summed again (cache hits, result dropped), so the row loop has
     // no branch and the number of loads in flight is the same at every wait.
     constexpr int SLOT_LOADS = (Q5 ? 3 : 2) * P;
-    // (the activation sums are finished before the first weight is requested)
-#pragma unroll
-    for (int pass = 0; pass < P; ++pass)
-#pragma unroll
-        for (int t = 0; t < MT; ++t) asm volatile("" ::"v"(xs_lo[pass][t]), "v"(xs_hi[pass][t]));
     Q4Slot<P, Q5> ring[D] = {};
-    // (The ring is filled after the prologue even where that is long: registers with a load in flight
-    // must stay where they are, and across the prologue's arithmetic the compiler moves them.)
+    if constexpr (STAGE) {
+        // Slot sl = 8 * pass + q of the staging area holds, for lane L, the q-th 16 bytes of that lane's
+        // operands of the pass (q < 4: low nibbles' elements, else high nibbles'): wave w fetches slots
+        // w, w + NW, ... exactly as the lane would have, and a wave's reads are 1 KB runs.
+        // Order: the wave's few activation loads, then the ring's first rows (weights never depend on x), then
+        // a wait that leaves exactly the ring outstanding: the whole x path — prologue arithmetic, LDS, the
+        // barrier (which waits for LDS only), the sums — runs under the first weights' flight.
+        constexpr int XL = P * 8 / NW;
+        constexpr bool EXTRA = PT::kFused || PT::kGrouped;   // a second operand: norm weights, or the act's other input
+        s_u32x4 xr[MT][XL] = {}, er[EXTRA ? MT : 1][EXTRA ? XL : 1] = {};
+        uint32_t keep[XL];
+        const int pro_rt = stream_pro(p);
 #pragma unroll
-    for (int d = 0; d < D; ++d)
-        ring[d].fill(p.W + row_of((uint32_t)d) * p.row_stride_bytes, hoff, j);
-    // (arguments beyond the preloaded ones are fetched now, under the first weights' flight, not at the stores)
-    stream_touch_late_args(p);
+        for (int k = 0; k < XL; ++k) {
+            const uint32_t sl = wave + (uint32_t)k * NW, q = sl & 7u;
+            uint32_t b = (sl >> 3) * 8u + bl;
+            const bool valid = b < p.n_blocks;
+            keep[k] = valid ? 0xFFFFFFFFu : 0u;   // activations of superblocks beyond K read as zero
+            b = valid ? b : p.n_blocks - 1u;
+            const size_t at = (size_t)b * KQ_QK + 64u * g + 16u * h + 32u * (q >> 2) + 4u * (q & 3u);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const float* xp = p.X + (size_t)t * ldx + at;
+                ring_load16(xr[t][k], (const uint8_t*)xp);
+                if constexpr (EXTRA) {
+                    const float* ep = pro_rt == STREAM_PRO_NORM ? stream_norm_w(p) + at
+                                    : pro_rt == STREAM_PRO_NONE ? xp : xp + x2_off;
+                    ring_load16(er[t][k], (const uint8_t*)ep);
+                }
+            }
+        }
+#pragma unroll
+        for (int pass = 0; pass < P; ++pass) hoff[pass] = min((uint32_t)pass * 8u + bl, p.n_blocks - 1u) * BLOCK;
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            ring[d].fill(p.W + row_of((uint32_t)d) * p.row_stride_bytes, hoff, j);
+        // (arguments beyond the preloaded ones are fetched now, under the first weights' flight, not at the stores)
+        stream_touch_late_args(p);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * SLOT_LOADS));
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int k = 0; k < XL; ++k) {
+                asm volatile("; ringwait %0" : "+v"(xr[t][k]));
+                if constexpr (EXTRA) asm volatile("; ringwait %0" : "+v"(er[t][k]));
+            }
+        auto stage_x = [&](auto pro) {
+            constexpr int PRO = decltype(pro)::value;
+            constexpr bool NORM = PRO == STREAM_PRO_NORM && PT::kFused;
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                float ssq = 0.0f;
+#pragma unroll
+                for (int k = 0; k < XL; ++k) {
+                    const uint32_t sl = wave + (uint32_t)k * NW;
+                    float4 v = __builtin_bit_cast(float4, xr[t][k]);
+                    if constexpr (PRO == STREAM_PRO_SILU || PRO == STREAM_PRO_GELU) {
+                        const float4 u = __builtin_bit_cast(float4, er[EXTRA ? t : 0][EXTRA ? k : 0]);
+                        v.x = stream_act<PRO, PT::kFused>(v.x, u.x);
+                        v.y = stream_act<PRO, PT::kFused>(v.y, u.y);
+                        v.z = stream_act<PRO, PT::kFused>(v.z, u.z);
+                        v.w = stream_act<PRO, PT::kFused>(v.w, u.w);
+                    }
+                    v = stream_keep(v, keep[k]);
+                    if constexpr (NORM) {
+                        const float4 w = __builtin_bit_cast(float4, er[EXTRA ? t : 0][EXTRA ? k : 0]);
+                        ssq = __builtin_fmaf(v.x, v.x, __builtin_fmaf(v.y, v.y, __builtin_fmaf(v.z, v.z, __builtin_fmaf(v.w, v.w, ssq))));
+                        v.x *= w.x; v.y *= w.y; v.z *= w.z; v.w *= w.w;
+                    }
+                    xstage[((uint32_t)t * P * 8u + sl) * 64u + lane] = v;
+                }
+                if constexpr (NORM) {
+                    const float ss = wave_sum(ssq);
+                    if (lane == 0) ssq_part[wave][t] = ss;
+                }
+            }
+        };
+        stream_dispatch_pro(p, stage_x);
+        // (the workgroup's LDS writes are all the barrier has to wait for: a full fence would drain the ring)
+        lds_barrier();
+        if (idle) {
+            asm volatile("s_waitcnt vmcnt(0)");
+            return;
+        }
+#pragma unroll
+        for (int pass = 0; pass < P; ++pass) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float4 lo = xstage[((uint32_t)t * P * 8u + pass * 8u + i) * 64u + lane];
+                    const float4 hi = xstage[((uint32_t)t * P * 8u + pass * 8u + 4u + i) * 64u + lane];
+                    xlo[pass][t][4 * i + 0] = lo.x; xlo[pass][t][4 * i + 1] = lo.y; xlo[pass][t][4 * i + 2] = lo.z; xlo[pass][t][4 * i + 3] = lo.w;
+                    xhi[pass][t][4 * i + 0] = hi.x; xhi[pass][t][4 * i + 1] = hi.y; xhi[pass][t][4 * i + 2] = hi.z; xhi[pass][t][4 * i + 3] = hi.w;
+                }
+                float sl = 0.0f, sh_ = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { sl += xlo[pass][t][i]; sh_ += xhi[pass][t][i]; }
+                xs_lo[pass][t] = sl;
+                xs_hi[pass][t] = sh_;
+            }
+        }
+        if (PT::kFused && pro_rt == STREAM_PRO_NORM) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                float ss = ssq_part[0][t];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) ss += ssq_part[w][t];
+                const float r = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
+                if (t == 0) rstd0 = r; else rstd1 = r;
+            }
+        }
+    } else {
+        stream_dispatch_pro(p, load_x);
+        // (the activation sums are finished before the first weight is requested)
+#pragma unroll
+        for (int pass = 0; pass < P; ++pass)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) asm volatile("" ::"v"(xs_lo[pass][t]), "v"(xs_hi[pass][t]));
+        // (Here the ring is filled after the prologue even where that is long: the sliced forms' prologue has
+        // a full barrier in it.)
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            ring[d].fill(p.W + row_of((uint32_t)d) * p.row_stride_bytes, hoff, j);
+        // (arguments beyond the preloaded ones are fetched now, under the first weights' flight, not at the stores)
+        stream_touch_late_args(p);
+    }
     // Rows are taken 64 at a time: lane i keeps the sums of the chunk's row i, and the
     // chunk is stored (bias added) after its last row.
     for (uint32_t c0 = 0; c0 < n_rows; c0 += 64u) {
@@ -518,20 +576,20 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
             if (KW > 1) __syncthreads();   // part is reused by the row loop
         }
     };
+    if (n_rows == 0) return;   // whole workgroup
+    constexpr int SLOT_LOADS = 5 * P;
+    Q6Slot<P> ring[D] = {};
     stream_dispatch_pro(p, load_x);
     // The activations' sums are complete before the first weight request goes out: here, arithmetic on
     // them that sank below the ring's fill waited for the weights as well and cost half a microsecond
-    // per launch (volatile statements keep their order, and this one makes the sums its operands).  The
-    // Q4_K kernel measured faster without such a pin.
+    // per launch (volatile statements keep their order, and this one makes the sums its operands).
+    // (The staged Q4_K order — activation loads, ring, a wait that leaves the ring outstanding — measured
+    // slower here: down 12.2 -> 12.6 us, with the act * up prologue's sixteen loads +1 us.)
 #pragma unroll
     for (int pass = 0; pass < P; ++pass)
 #pragma unroll
         for (int tk = 0; tk < MT; ++tk)
             asm volatile("" : "+v"(m32xs[pass][tk][0]), "+v"(m32xs[pass][tk][1]), "+v"(m32xs[pass][tk][2]), "+v"(m32xs[pass][tk][3]));
-
-    if (n_rows == 0) return;   // whole workgroup
-    constexpr int SLOT_LOADS = 5 * P;
-    Q6Slot<P> ring[D] = {};
 #pragma unroll
     for (int d = 0; d < D; ++d)
         ring[d].fill(p.W + (size_t)(g + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, boff, n, lg);
