@@ -62,7 +62,16 @@ __device__ __forceinline__ void wave_window_fence()
 }
 
 constexpr int MT_KC = 4;                       // superblocks of X staged at a time
-constexpr int MT_XA_BYTES = MT_KC * 8 * 2 * 1024;   // [block][sub-block][hi/lo][lane] 16 B
+// The A operands in LDS: [block][sub-block] pairs of planes (hi, lo; or, with hi / lo slots, this chunk's and the
+// next one's) of 64 positions of 16 bytes.  A matrix instruction's lane (slot, kq) reads position
+// mt_xa_pos(slot, kq) of a plane: 1 KB runs, conflict-free.  The converting threads write one position each,
+// 16 lanes at a time spread over sub-blocks and superblocks: the pitch of a pair is 16 bytes more than its 2 KB
+// and a slot is rotated by 4 * kq inside its group of 16, so that those 16 writes (and a 16-thread pair's, whose
+// two halves differ in kq) fall into 16 different bank groups; with pairs 2 KB apart and slots unrotated
+// they all hit one (measured: a quarter of the 16-token kernel's cycles were LDS bank conflicts).
+constexpr int MT_XA_PITCH = 2 * 1024 + 16;
+constexpr int MT_XA_BYTES = MT_KC * 8 * MT_XA_PITCH;
+__device__ __forceinline__ uint32_t mt_xa_pos(uint32_t slot, uint32_t kq) { return ((slot + 4u * kq) & 15u) + 16u * kq; }
 constexpr int MT_XS_FLOATS = MT_KC * 8 * 32;        // [block][sub-block][token], or [block][sub-block][half][token]
 constexpr int MT_INV_FLOATS = MT_KC * 16;           // [block][token]
 constexpr int MT_XV_BYTES = MT_KC * 2 * 1024;       // [block][hi/lo][lane] 16 B: the sub-block sums as an A operand (Q4_K)
@@ -264,9 +273,10 @@ struct MtileStager {
             const uint32_t sb = k >> 5, kq = (k >> 3) & 3u;
             // SPLIT16: the first half of a 32-run goes to slot token, the second to slot token + 8
             const uint32_t slot = SPLIT16 ? token + 8u * (kq >> 1) : token;
-            uint8_t* dst = xa + ((size_t)((bb * 8u + sb) * 2u) * 64u + slot + 16u * kq) * 16u;
-            *(t_half8*)dst = hv;
-            *(t_half8*)(dst + (HL8 ? 8 * 16 : 1024)) = lv;
+            uint8_t* pair = xa + (size_t)(bb * 8u + sb) * MT_XA_PITCH;
+            *(t_half8*)(pair + mt_xa_pos(slot, kq) * 16u) = hv;
+            if (HL8) *(t_half8*)(pair + mt_xa_pos(slot + 8u, kq) * 16u) = lv;
+            else *(t_half8*)(pair + 1024 + mt_xa_pos(slot, kq) * 16u) = lv;
         }
         // sums of the unscaled x over each run of 32 (or, SPLIT16, each half run of 16)
         if constexpr (EPT >= 32) {
@@ -314,7 +324,7 @@ struct MtileA {
 template <bool HL8 = false>
 __device__ __forceinline__ MtileA mtile_read_a(const uint8_t* xa_b, int sb, uint32_t lane)
 {
-    const uint8_t* ap = xa_b + ((size_t)(sb * 2) * 64u + lane) * 16u;
+    const uint8_t* ap = xa_b + (size_t)sb * MT_XA_PITCH + mt_xa_pos(lane & 15u, lane >> 4) * 16u;
     MtileA a;
     a.hi = *(const t_half8*)ap;
     a.lo = a.hi;
@@ -426,7 +436,7 @@ __device__ __forceinline__ void q4k_mtile_block_compact(const t_u32x4 hdr, const
 #pragma unroll
         for (int hn = 0; hn < 2; ++hn) {
             const int sb = 2 * g + hn;
-            const uint8_t* ap = xa_b + ((size_t)(sb * 2) * 64u + lane) * 16u;
+            const uint8_t* ap = xa_b + (size_t)sb * MT_XA_PITCH + mt_xa_pos(lane & 15u, lane >> 4) * 16u;
             const t_half8 ahi = *(const t_half8*)ap;
             const t_half8 alo = *(const t_half8*)(ap + 1024);
             const t_half8 bq = __builtin_bit_cast(t_half8, hn ? bhi : blo);
@@ -502,7 +512,7 @@ __device__ __forceinline__ void q6k_mtile_block(const Q6TileW& w, const uint8_t*
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int run = 4 * h + t;
-            const uint8_t* ap = xa_b + ((size_t)(run * 2) * 64u + lane) * 16u;
+            const uint8_t* ap = xa_b + (size_t)run * MT_XA_PITCH + mt_xa_pos(lane & 15u, lane >> 4) * 16u;
             const t_half8 ahi = *(const t_half8*)ap;
             const t_half8 alo = *(const t_half8*)(ap + 1024);
             const t_half8 b8 = __builtin_bit_cast(t_half8, bq[t]);
@@ -558,7 +568,7 @@ __device__ __forceinline__ void q6k_mtile_block_wide(const Q6TileW& w, const uin
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int run = 4 * h + t;
-            const uint8_t* ap = xa_b + ((size_t)(run * 2) * 64u + lane) * 16u;
+            const uint8_t* ap = xa_b + (size_t)run * MT_XA_PITCH + mt_xa_pos(lane & 15u, lane >> 4) * 16u;
             const t_half8 ahi = *(const t_half8*)ap;
             const t_half8 alo = *(const t_half8*)(ap + 1024);
             const t_u32x4 b1 = {bq[t].x & first, bq[t].y & first, bq[t].z & first, bq[t].w & first};
@@ -814,16 +824,16 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
                         Q6TileW w6;
                         q6k_mtile_load(blk, kq, w6);
                         if constexpr (Q6W)
-                            q6k_mtile_block_wide(w6, xa + (size_t)bb * (8 * 2 * 1024), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                            q6k_mtile_block_wide(w6, xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * XSB, xinv + bb * 16, lane, tot);
                         else
-                            q6k_mtile_block(w6, xa + (size_t)bb * (8 * 2 * 1024), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                            q6k_mtile_block(w6, xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * XSB, xinv + bb * 16, lane, tot);
                     } else {
                         const t_u32x4 hdr = *(const t_u32x4*)blk;
                         t_u32x2 w[4], qhw = {0, 0};
 #pragma unroll
                         for (int g = 0; g < 4; ++g) w[g] = *(const t_u32x2*)(blk + QOFF + 32u * g + 8u * kq);
                         if constexpr (Q5) qhw = *(const t_u32x2*)(blk + 16u + 8u * kq);
-                        q4k_mtile_block<Q5, HL8>(hdr, w, qhw, xa_c + (size_t)bb * (8 * 2 * 1024), xv_c + (size_t)bb * 2048, xinv_c + bb * 16, lane, tot);
+                        q4k_mtile_block<Q5, HL8>(hdr, w, qhw, xa_c + (size_t)bb * (8 * MT_XA_PITCH), xv_c + (size_t)bb * 2048, xinv_c + bb * 16, lane, tot);
                     }
                 }
             }
@@ -879,11 +889,11 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
                 const uint32_t bb = R == 1 ? wave + i * NW : i;
                 if (bb < MT_KC && c0 + bb < c_end) {
                     if constexpr (Q6W)
-                        q6k_mtile_block_wide(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                        q6k_mtile_block_wide(w6[i], xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * XSB, xinv + bb * 16, lane, tot);
                     else if constexpr (Q6)
-                        q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                        q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * XSB, xinv + bb * 16, lane, tot);
                     else
-                        q4k_mtile_block_compact<Q5>(hdr[i], w[i], qhw[i], xa + (size_t)bb * (8 * 2 * 1024), xs + bb * 128, xinv + bb * 16, lane, tot);
+                        q4k_mtile_block_compact<Q5>(hdr[i], w[i], qhw[i], xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * 128, xinv + bb * 16, lane, tot);
                 }
             }
         }
