@@ -36,7 +36,7 @@ METRIC = "Q4_K M=1 matvec HBM GB/s (% of peak); M=2048 dequant-GEMM TFLOPS (% MF
 # FETCH_SIZE / WRITE_SIZE summary named below (FETCH_SIZE x 2.000 KiB + WRITE_SIZE x 1.000 KiB, the factors
 # being what the same counters read for a 256 MiB copy kernel); regenerate that file when the kernel changes.
 TRAFFIC_PROFILE = "profiles/decode_gemv_hbm_traffic_pmc.txt"
-MEASURED_TRAFFIC_BYTES = 66444830
+MEASURED_TRAFFIC_BYTES = 66436321
 
 
 def parse():
@@ -273,7 +273,7 @@ def main():
     dom_bytes = synth.weight_bytes(dom_w.type, dom_w.N, dom_w.K) + (dom_w.K + dom_w.N) * 4
     dom_gbs = dom_bytes / (dsec / launches) / 1e9
     roofline = {
-        "kernel": f"kq::q4k_stream_kernel<2, 8, 2, 1, kq::StreamDense, false> ({capi.last_kernel()}; gate|up 28672x4096 Q4_K, M=1)",
+        "kernel": f"kq::q4k_stream_dense_kernel<2, 8, 2, 1, false, 1> ({capi.last_kernel()}; gate|up 28672x4096 Q4_K, M=1)",
         "bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
         "bytes_per_launch": dom_bytes, "us_per_launch": round(dsec / launches * 1e6, 3),
