@@ -436,11 +436,11 @@ static int matmul_impl(int type, const float* X, const void* W, const float* bia
     const bool mtile_ok = kq::mtile_supported(a);
     if (t_family == 6 && !mtile_ok) return fail(BPK_ERR_SHAPE, "16x16 tile kernel cannot serve this call");
     // three and four tokens on the smaller matrices stay on the lanes-along-K kernel (four tokens share every
-    // weight load and its unpack).  Measured at M = 4: Q4_K 4096x4096 10.0 against 10.8 us on the tile
-    // kernel, 6144x4096 a tie, 28672x4096 34.5 against 23.0; Q6_K 4096x14336 23.6 against 27.1.
+    // weight load and its unpack).  Measured at M = 4: Q4_K 4096x4096 8.5 against 10.6 us on the tile
+    // kernel, 6144x4096 10.8 against 11.8, 28672x4096 32.6 against 19.2; Q6_K 4096x14336 23.2 against 27.0.
     const uint64_t weights = (uint64_t)N * K;
     const bool stream_four = stream_ok && M >= 3 && M <= 4 && N <= 32768u &&
-                             weights <= (type == BPK_TYPE_Q6_K ? (64ull << 20) : (20ull << 20));
+                             weights <= (type == BPK_TYPE_Q6_K ? (64ull << 20) : (32ull << 20));
     // two tokens on a Q4_K / Q5_K matrix of gate|up's size: the tile kernel's form for up to 8 tokens (hi and lo
     // parts as token slots) beats two tokens on the vector units there (28672x4096: 19.6 against 22.7 us; 6144x4096:
     // 11.1 against 8.5, so smaller matrices stay)

@@ -185,13 +185,17 @@ template <int P, int NW, int D, int MT, typename PT, bool Q5 = false, int KW = 1
 __device__ __forceinline__ void q4k_stream_body(PT p)
 {
     stream_select_pair(p);
-    __shared__ float part[KW > 1 ? KW : 1][MT][64];
+    __shared__ float part[KW > 1 ? KW * NW : 1][MT][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t gw0 = KW > 1 ? blockIdx.x : blockIdx.x * NW + wave;
+    // NW > 1 and KW > 1 together: the workgroup is KW K slices x NW walkers; the walkers of a slice share its
+    // activations, the slices of a walker fold their sums (wave = slice * NW + walker)
+    const uint32_t slice = KW > 1 ? (NW > 1 ? wave / NW : wave) : 0u;
+    const uint32_t walker = NW > 1 ? (KW > 1 ? wave % NW : wave) : 0u;
+    const uint32_t gw0 = blockIdx.x * NW + walker;
     // rows gw, gw + stride, ...: at any moment the waves of the grid read
     // consecutive rows, one contiguous stream across the memory channels
-    const uint32_t stride = KW > 1 ? stream_grid_x(p) : stream_grid_x(p) * NW;
+    const uint32_t stride = stream_grid_x(p) * NW;
     // pair mode (fused kernels only): the wave walks pairs gw, gw + stride, ... of the N/2 outputs and its
     // ring alternates between a pair's gate row and its up row, N/2 rows further on
     const bool pairs = PT::kFused && stream_epi(p) != 0;
@@ -199,10 +203,11 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
     // STAGE (whole-row waves, several to a workgroup): the workgroup fetches the activations once and its waves
     // take their operands from LDS; every wave loading the row for itself costs a CU's vector cache eight times
     // the bytes (16 KB per wave and token, twice that with norm weights: 1 to 3 us of a launch).
-    constexpr bool STAGE = KW == 1 && NW > 1;
-    __shared__ float4 xstage[STAGE ? MT * P * 8 * 64 : 1];
-    __shared__ float ssq_part[STAGE ? NW : 1][MT];
-    const bool idle = gw0 >= n_walk_all;   // KW > 1: the whole workgroup
+    constexpr bool STAGE = NW > 1;
+    extern __shared__ float4 xstage_all[];   // STAGE: [slice][token][8 * P slots][64 lanes], sized by the launch
+    float4* xstage = xstage_all + slice * (MT * P * 8 * 64);
+    __shared__ float ssq_part[STAGE ? NW * KW : 1][MT];
+    const bool idle = gw0 >= n_walk_all;   // NW == 1: the whole workgroup
     if (!STAGE && idle) return;
     const uint32_t gw = idle ? 0u : gw0;   // (a staged workgroup's idle waves help fetch the activations, then leave)
     const uint32_t n_walk = (n_walk_all - gw + stride - 1u) / stride;
@@ -232,7 +237,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
         for (int t = 0; t < MT; ++t) ssq[t] = 0.0f;
 #pragma unroll
         for (int pass = 0; pass < P; ++pass) {
-            uint32_t b = ((KW > 1 ? wave * P : 0u) + pass) * 8u + bl;
+            uint32_t b = (slice * P + pass) * 8u + bl;
             const bool valid = b < p.n_blocks;
             const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;   // activations of superblocks beyond K read as zero
             b = valid ? b : p.n_blocks - 1u;
@@ -273,7 +278,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
             for (int t = 0; t < MT; ++t) {
                 float ss = wave_sum(ssq[t]);   // the wave holds the whole row, or a K slice of it
                 if (KW > 1) {                  // the slices' sums of squares meet in LDS
-                    if (lane == 0) part[wave][t][0] = ss;
+                    if (lane == 0) part[slice][t][0] = ss;
                     __syncthreads();
                     ss = part[0][t][0];
 #pragma unroll
@@ -306,15 +311,16 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
         const int pro_rt = stream_pro(p);
 #pragma unroll
         for (int k = 0; k < XL; ++k) {
-            const uint32_t sl = wave + (uint32_t)k * NW, q = sl & 7u;
-            uint32_t b = (sl >> 3) * 8u + bl;
+            const uint32_t sl = walker + (uint32_t)k * NW, q = sl & 7u;
+            uint32_t b = (slice * P + (sl >> 3)) * 8u + bl;
             const bool valid = b < p.n_blocks;
             keep[k] = valid ? 0xFFFFFFFFu : 0u;   // activations of superblocks beyond K read as zero
             b = valid ? b : p.n_blocks - 1u;
             const size_t at = (size_t)b * KQ_QK + 64u * g + 16u * h + 32u * (q >> 2) + 4u * (q & 3u);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                const float* xp = p.X + (size_t)t * ldx + at;
+                const uint32_t xt = MT > 2 ? min((uint32_t)t, p.M - 1u) : (uint32_t)t;   // a masked token re-reads the last one
+                const float* xp = p.X + (size_t)xt * ldx + at;
                 ring_load16(xr[t][k], (const uint8_t*)xp);
                 if constexpr (EXTRA) {
                     const float* ep = pro_rt == STREAM_PRO_NORM ? stream_norm_w(p) + at
@@ -324,7 +330,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
             }
         }
 #pragma unroll
-        for (int pass = 0; pass < P; ++pass) hoff[pass] = min((uint32_t)pass * 8u + bl, p.n_blocks - 1u) * BLOCK;
+        for (int pass = 0; pass < P; ++pass) hoff[pass] = min((slice * P + (uint32_t)pass) * 8u + bl, p.n_blocks - 1u) * BLOCK;
 #pragma unroll
         for (int d = 0; d < D; ++d)
             ring[d].fill(p.W + row_of((uint32_t)d) * p.row_stride_bytes, hoff, j);
@@ -346,7 +352,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
                 float ssq = 0.0f;
 #pragma unroll
                 for (int k = 0; k < XL; ++k) {
-                    const uint32_t sl = wave + (uint32_t)k * NW;
+                    const uint32_t sl = walker + (uint32_t)k * NW;
                     float4 v = __builtin_bit_cast(float4, xr[t][k]);
                     if constexpr (PRO == STREAM_PRO_SILU || PRO == STREAM_PRO_GELU) {
                         const float4 u = __builtin_bit_cast(float4, er[EXTRA ? t : 0][EXTRA ? k : 0]);
@@ -365,7 +371,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
                 }
                 if constexpr (NORM) {
                     const float ss = wave_sum(ssq);
-                    if (lane == 0) ssq_part[wave][t] = ss;
+                    if (lane == 0) ssq_part[wave][t] = ss;   // (every element of x is fetched by exactly one wave)
                 }
             }
         };
@@ -399,7 +405,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
             for (int t = 0; t < MT; ++t) {
                 float ss = ssq_part[0][t];
 #pragma unroll
-                for (int w = 1; w < NW; ++w) ss += ssq_part[w][t];
+                for (int w = 1; w < NW * KW; ++w) ss += ssq_part[w][t];
                 const float r = 1.0f / sqrtf(ss / (float)p.K + stream_eps(p));
                 if (t == 0) rstd0 = r; else rstd1 = r;
             }
@@ -446,23 +452,25 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
                 }
             }
         }
+        // (the slices' barriers wait for LDS only: a full fence would drain the ring.  Walkers of a workgroup may
+        // differ by a chunk; a wave that has ended no longer counts at a barrier.)
         if (KW > 1) {
 #pragma unroll
-            for (int t = 0; t < MT; ++t) part[wave][t][lane] = res[t];
-            __syncthreads();
+            for (int t = 0; t < MT; ++t) part[slice * NW + walker][t][lane] = res[t];
+            lds_barrier();
         }
         // (the lane guard stays outside: with it inside, the gate|up launch measured 3 us slower.  In pair
         // mode cnt is even, so a lane inside the guard finds its partner there too.)
-        if ((KW == 1 || wave == 0) && lane < cnt) {
+        if ((KW == 1 || slice == 0) && lane < cnt) {
             const uint32_t r = (uint32_t)row_of(c0 + lane);
             const float bias = p.bias ? p.bias[r] : 0.0f;
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 float y = res[t];
                 if (KW > 1) {
-                    y = part[0][t][lane];
+                    y = part[walker][t][lane];
 #pragma unroll
-                    for (int w = 1; w < KW; ++w) y += part[w][t][lane];
+                    for (int w = 1; w < KW; ++w) y += part[w * NW + walker][t][lane];
                 }
                 if constexpr (PT::kFused) y *= t == 0 ? rstd0 : rstd1;
                 y += bias;
@@ -480,7 +488,7 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
                 p.Y[at] = y;
             }
         }
-        if (KW > 1) __syncthreads();
+        if (KW > 1) lds_barrier();
     }
     asm volatile("s_waitcnt vmcnt(0)");   // the ring's last refills land before the wave ends
 }
@@ -674,12 +682,12 @@ static uint32_t cu_count() { return device_cu_count(); }
         (p).M, (p).y_offset, (p).ldy, (p).bias, (p).residual
 
 template <int P, int NW, int D, int MT, typename PT, bool Q5 = false, int KW = 1>
-__global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_kernel(PT p)
+__global__ __launch_bounds__(64 * NW * KW) void q4k_stream_kernel(PT p)
 {
     q4k_stream_body<P, NW, D, MT, PT, Q5, KW>(p);
 }
 template <int P, int NW, int D, int MT, bool Q5 = false, int KW = 1>
-__global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_fused_kernel(KQ_FUSED_PARAMS)
+__global__ __launch_bounds__(64 * NW * KW) void q4k_stream_fused_kernel(KQ_FUSED_PARAMS)
 {
     q4k_stream_body<P, NW, D, MT, StreamFused, Q5, KW>(KQ_FUSED_STRUCT);
 }
@@ -689,7 +697,7 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_fused_kernel(KQ_FUSED_PARA
     q6k_stream_body<P, KW, D, MT, StreamFused>(KQ_FUSED_STRUCT);
 }
 template <int P, int NW, int D, int MT, bool Q5 = false, int KW = 1>
-__global__ __launch_bounds__(64 * (KW > 1 ? KW : NW)) void q4k_stream_dense_kernel(KQ_DENSE_PARAMS)
+__global__ __launch_bounds__(64 * NW * KW) void q4k_stream_dense_kernel(KQ_DENSE_PARAMS)
 {
     q4k_stream_body<P, NW, D, MT, StreamDense, Q5, KW>(KQ_DENSE_STRUCT);
 }
@@ -708,12 +716,22 @@ __global__ __launch_bounds__(64 * KW) void q6k_stream_dense_kernel(KQ_DENSE_PARA
 template <int P, int NW, int D, int MT, bool Q5, int KW, typename PT>
 static void launch_q4k_entry(dim3 grid, dim3 block, hipStream_t s, const PT& p)
 {
-    if constexpr (std::is_same<PT, StreamDense>::value)
-        hipLaunchKernelGGL((q4k_stream_dense_kernel<P, NW, D, MT, Q5, KW>), grid, block, 0, s, KQ_DENSE_ARGS(p, grid.x));
-    else if constexpr (std::is_same<PT, StreamFused>::value)
-        hipLaunchKernelGGL((q4k_stream_fused_kernel<P, NW, D, MT, Q5, KW>), grid, block, 0, s, KQ_FUSED_ARGS(p, grid.x));
-    else
-        hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT, Q5, KW>), grid, block, 0, s, p);
+    // the staging area of the activations (workgroups of several walkers): 16 bytes per lane and slot
+    constexpr size_t shmem = NW > 1 ? (size_t)KW * MT * P * 8 * 64 * 16 : 0;
+    auto raise = [](const void* kern) {
+        if (shmem > 32768) (void)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    };
+    static bool raised = false;   // per instantiation
+    if constexpr (std::is_same<PT, StreamDense>::value) {
+        if (!raised) { raise((const void*)q4k_stream_dense_kernel<P, NW, D, MT, Q5, KW>); raised = true; }
+        hipLaunchKernelGGL((q4k_stream_dense_kernel<P, NW, D, MT, Q5, KW>), grid, block, shmem, s, KQ_DENSE_ARGS(p, grid.x));
+    } else if constexpr (std::is_same<PT, StreamFused>::value) {
+        if (!raised) { raise((const void*)q4k_stream_fused_kernel<P, NW, D, MT, Q5, KW>); raised = true; }
+        hipLaunchKernelGGL((q4k_stream_fused_kernel<P, NW, D, MT, Q5, KW>), grid, block, shmem, s, KQ_FUSED_ARGS(p, grid.x));
+    } else {
+        if (!raised) { raise((const void*)q4k_stream_kernel<P, NW, D, MT, PT, Q5, KW>); raised = true; }
+        hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT, Q5, KW>), grid, block, shmem, s, p);
+    }
 }
 template <int P, int KW, int D, int MT, typename PT>
 static void launch_q6k_entry(dim3 grid, dim3 block, hipStream_t s, const PT& p)
@@ -801,6 +819,22 @@ static hipError_t launch_stream_four(const MatmulArgs& a, hipStream_t s, const P
 {
     const uint32_t nb = a.n_blocks;
     const int kw = nb <= 8u ? 1 : nb <= 16u ? 2 : nb <= 32u ? 4 : 7;
+    if (a.type != KQ_TYPE_Q6_K && kw <= 2) {
+        // rows of up to 16 superblocks: four walkers per K slice share the slice's activations through LDS
+        // (32 KB per slice; every wave loading its 128 activations per lane for itself moved 64 MB through
+        // the vector caches for the 9.4 MB of a 4096 x 4096 matrix)
+        const uint32_t wgs4 = stream_workgroups((a.N + 3u) / 4u, 1u, 0);
+        const dim3 grid4(wgs4, 1, 1);
+        const bool q5 = a.type == KQ_TYPE_Q5_K;
+        if (kw == 1) {
+            if (q5) launch_q4k_entry<1, 4, 2, 4, true, 1>(grid4, dim3(256), s, p);
+            else launch_q4k_entry<1, 4, 2, 4, false, 1>(grid4, dim3(256), s, p);
+        } else {
+            if (q5) launch_q4k_entry<1, 4, 2, 4, true, 2>(grid4, dim3(512), s, p);
+            else launch_q4k_entry<1, 4, 2, 4, false, 2>(grid4, dim3(512), s, p);
+        }
+        return hipGetLastError();
+    }
     const uint32_t wgs = stream_workgroups(a.N, kw >= 7 ? 1u : 8u / (uint32_t)kw, 0);
     const dim3 grid(wgs, 1, 1);
     if (a.type == KQ_TYPE_Q6_K) {
@@ -809,14 +843,10 @@ static hipError_t launch_stream_four(const MatmulArgs& a, hipStream_t s, const P
         else if (kw == 4) launch_q6k_entry<1, 4, 2, 4>(grid, dim3(256), s, p);
         else launch_q6k_entry<1, 7, 2, 4>(grid, dim3(448), s, p);
     } else if (a.type == KQ_TYPE_Q5_K) {
-        if (kw == 1) launch_q4k_entry<1, 1, 2, 4, true, 1>(grid, dim3(64), s, p);
-        else if (kw == 2) launch_q4k_entry<1, 1, 2, 4, true, 2>(grid, dim3(128), s, p);
-        else if (kw == 4) launch_q4k_entry<1, 1, 2, 4, true, 4>(grid, dim3(256), s, p);
+        if (kw == 4) launch_q4k_entry<1, 1, 2, 4, true, 4>(grid, dim3(256), s, p);
         else launch_q4k_entry<1, 1, 2, 4, true, 7>(grid, dim3(448), s, p);
     } else {
-        if (kw == 1) launch_q4k_entry<1, 1, 2, 4, false, 1>(grid, dim3(64), s, p);
-        else if (kw == 2) launch_q4k_entry<1, 1, 2, 4, false, 2>(grid, dim3(128), s, p);
-        else if (kw == 4) launch_q4k_entry<1, 1, 2, 4, false, 4>(grid, dim3(256), s, p);
+        if (kw == 4) launch_q4k_entry<1, 1, 2, 4, false, 4>(grid, dim3(256), s, p);
         else launch_q4k_entry<1, 1, 2, 4, false, 7>(grid, dim3(448), s, p);
     }
     return hipGetLastError();

@@ -34,7 +34,14 @@ static CheckResult assertClose(const float* a, const float* e, int n, float atol
     float worst = 0;
     int bad = kqo_assert_close(a, e, n, atol, rtol, &worst);
     if (!bad) return {true, ""};
-    char buf[128]; snprintf(buf, sizeof buf, "%d elements outside tolerance, worst excess %g", bad, worst);
+    int at = 0; float ex = -1.0f;
+    for (int i = 0; i < n; i++) {
+        const float x = std::fabs(a[i] - e[i]) - (atol + rtol * std::fabs(e[i]));
+        if (x > ex) { ex = x; at = i; }
+    }
+    char buf[192];
+    snprintf(buf, sizeof buf, "%d elements outside tolerance, worst excess %g (element %d: got %.9g, expected %.9g)", bad, worst,
+             at, a[at], e[at]);
     return {false, buf};
 }
 
@@ -323,8 +330,15 @@ TEST(chain_of_a_decoder_layer_tail) {
     readBuffer(bX, sep.data(), H * 4);
     releaseBuffer(bAttn); releaseBuffer(bX); releaseBuffer(bNw); releaseBuffer(bAct); releaseBuffer(wo); releaseBuffer(wg); releaseBuffer(wd);
     CheckResult r = assertClose(got.data(), expected.data(), H, 2e-4f, 2e-4f);
-    if (!r.ok) return r;
-    return assertClose(sep.data(), got.data(), H, 2e-5f, 2e-5f);
+    if (!r.ok) return {false, "chain against the oracle: " + r.msg};
+    // (the two forms apply the norm's 1/rms at different places — to the activations in the chain, to the outputs in
+    // the fused dispatch — and down's sums cancel heavily with these weights: a rounding's worth of difference in
+    // act shows as a few 1e-5 relative in single elements)
+    r = assertClose(sep.data(), expected.data(), H, 2e-4f, 2e-4f);
+    if (!r.ok) return {false, "separate fused dispatches against the oracle: " + r.msg};
+    r = assertClose(sep.data(), got.data(), H, 1e-4f, 1e-4f);
+    if (!r.ok) return {false, "separate fused dispatches against the chain: " + r.msg};
+    return r;
 }
 TEST(model_config_from_gguf) {
     // a metadata-only file of a Gemma-3-shaped model, read through the GGUFFile mirror and extractModelConfig
