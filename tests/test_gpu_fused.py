@@ -198,6 +198,7 @@ def test_fused_argument_checks(gpu):
 EPI = [
     # type, M, N outputs, K, epilogue, prologue, bias, expected kernel
     (Q4_K, 1, 14336, 4096, SILU, NONE, False, "gemv_stream_fused"),     # the decode FFN head at its real shape
+    (Q4_K, 1, 14336, 4096, SILU, NORM, False, "gemv_stream_fused"),     # ... with ffn_norm folded in (eight-wave form)
     (Q4_K, 2, 300, 4096, GELU, NONE, True, "gemv_stream_fused"),
     (Q4_K, 1, 257, 2048, SILU, NORM, False, "gemv_stream_fused"),       # ffn_norm folded in as well
     (Q4_K, 1, 100, 8192, SILU, NONE, False, "gemv_stream_fused"),       # K slices over four waves

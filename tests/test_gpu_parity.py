@@ -165,6 +165,7 @@ SHAPES = [
     (Q4_K, 2, 200, 1024),
     (Q4_K, 3, 130, 2048),
     (Q4_K, 4, 65, 512),
+    (Q4_K, 4, 70, 4096),        # two K slices x four walkers that share the activations; some walkers idle
     (Q4_K, 5, 9, 512),
     (Q4_K, 16, 96, 1024),
     (Q6_K, 1, 512, 4096),
@@ -195,6 +196,7 @@ SHAPES = [
     (Q5_K, 2, 500, 14336),
     (Q5_K, 1, 90, 28672),
     (Q5_K, 3, 130, 2048),
+    (Q5_K, 3, 70, 4096),
     (Q5_K, 5, 9, 512),
     (Q5_K, 7, 300, 4096),
     (Q5_K, 16, 2000, 4096),     # one tile per workgroup, ragged last tile
