@@ -932,10 +932,11 @@ static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, h
         else launch_q4k_one<P, NW, D, 1, PT, false>(grid, s, p); \
     } while (0)
     if constexpr (!PT::kGrouped) {
-        // Matrices that give every wave eight rows or more (gate|up: 28672 x 4096) run faster as eight waves
-        // per workgroup with two rows in flight each than as four with four: 15.3 against 16.8 us there.
-        // Shorter walks lose with it (6144 x 4096: 7.8 against 7.3 us), so they keep the four-wave form.
-        const bool eight = t.waves == 8 || (t.waves == 0 && t.depth == 0 && t.splits == 0 && a.N >= 8u * 8u * cu_count());
+        // Matrices that give every wave six rows or more (gate|up: 28672 x 4096) run faster as eight waves
+        // per workgroup with two rows in flight each than as four with four: 15.3 against 16.8 us there,
+        // 14336 x 4096 9.1 against 9.4.  Shorter walks lose with it (8192 x 4096: 6.2 against 6.0 us,
+        // 6144 x 4096: 6.1 against 5.1), so they keep the four-wave form.
+        const bool eight = t.waves == 8 || (t.waves == 0 && t.depth == 0 && t.splits == 0 && a.N >= 6u * 8u * cu_count());
         if (eight && !q5 && !two && a.n_blocks > 8u) {
             const uint32_t wgs8 = stream_workgroups((a.N + 7u) / 8u, 1u, 0);
             launch_q4k_entry<2, 8, 2, 1, false, 1>(dim3(wgs8, 1, 1), dim3(512), s, p);

@@ -308,7 +308,7 @@ def test_gemv_stream_shapes(gpu, kqo, type_, N, K, depth, rows_per_wave, M):
 @pytest.mark.parametrize("N,K", [(1000, 4096), (70, 3072), (16500, 2304), (9, 4096)])
 def test_gemv_stream_eight_wave_form(gpu, kqo, N, K):
     """The lanes-along-K kernel as eight waves per workgroup, two rows in flight each (what matrices of
-    16384 rows and more get by default), forced on small and ragged shapes; with a y offset and bias."""
+    12288 rows and more get by default), forced on small and ragged shapes; with a y offset and bias."""
     import torch
     from backpack_amd import capi, kquant
     raw, packed, w = gpu.make_weight(Q4_K, N, K, seed=N + 1)
