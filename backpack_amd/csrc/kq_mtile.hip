@@ -1018,19 +1018,41 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
         __syncthreads();
         if (*ticket != p.n_splits - 1u) return;   // whole workgroup
         if (mine) {
+            // eight splits' partials are requested before the first is added (one round trip, not one per
+            // split); the sums still run in split order
             float t4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            for (uint32_t z = 0; z < p.n_splits; ++z)
+            for (uint32_t z0 = 0; z0 < p.n_splits; z0 += 8u) {
+                float v[8][4];
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    t4[r] += __hip_atomic_load(p.partial + ((size_t)z * 16u + 4u * kq + r) * plane + prow, __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT);
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t z = min(z0 + (uint32_t)j, p.n_splits - 1u);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        v[j][r] = __hip_atomic_load(p.partial + ((size_t)z * 16u + 4u * kq + r) * plane + prow, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (z0 + (uint32_t)j < p.n_splits) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) t4[r] += v[j][r];
+                    }
+            }
             tot = t_f32x4{t4[0], t4[1], t4[2], t4[3]};
         }
         if (normed) {
             if (threadIdx.x < 16u) {
                 float t = 0.0f;
-                for (uint32_t z = 0; z < p.n_splits; ++z)
-                    t += __hip_atomic_load(ssq + z * 16u + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (uint32_t z0 = 0; z0 < p.n_splits; z0 += 8u) {   // (as above: eight loads in flight, sums in split order)
+                    float v[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        v[j] = __hip_atomic_load(ssq + min(z0 + (uint32_t)j, p.n_splits - 1u) * 16u + threadIdx.x, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (z0 + (uint32_t)j < p.n_splits) t += v[j];
+                }
                 rinv[threadIdx.x] = t;
             }
             __syncthreads();
