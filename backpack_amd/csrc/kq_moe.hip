@@ -16,6 +16,11 @@ namespace kq {
 // One workgroup buckets all pairs.  tiles: records of (2 + cap) words
 // {expert, count, pair ids...}; experts appear in ascending order, the pairs
 // of an expert in arrival order (the per-pair results do not depend on it).
+// One pass over the pairs: the LDS counter's old value is the pair's place inside its expert, and the
+// first pairs of a thread stay in registers until the records' places are known; the first record of
+// every expert comes from a scan over the workgroup (eight experts per thread, a wave scan, the waves'
+// totals through LDS) instead of one thread walking all experts.
+constexpr int MOE_GROUP_KEEP = 4;   // pairs per thread kept in registers (more are read again)
 __global__ __launch_bounds__(1024) void moe_group_kernel(const uint32_t* __restrict__ expert_idx, uint32_t n_pairs,
                                                          uint32_t n_experts, uint32_t cap, uint32_t* __restrict__ tiles,
                                                          uint32_t* __restrict__ n_tiles)
@@ -23,37 +28,86 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const uint32_t* __restr
     extern __shared__ uint32_t sm[];
     uint32_t* count = sm;                  // [n_experts]
     uint32_t* base = sm + n_experts;       // [n_experts] first tile of the expert
-    uint32_t* fill = sm + 2 * n_experts;   // [n_experts]
-    for (uint32_t e = threadIdx.x; e < n_experts; e += blockDim.x) { count[e] = 0; fill[e] = 0; }
+    uint32_t* fill = sm + 2 * n_experts;   // [n_experts] places taken by the kept pairs (more than 4096 pairs only)
+    __shared__ uint32_t wave_total[16];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    for (uint32_t e = tid; e < n_experts; e += 1024u) count[e] = 0;
     __syncthreads();
-    for (uint32_t p = threadIdx.x; p < n_pairs; p += blockDim.x) {
-        const uint32_t e = expert_idx[p];
-        if (e < n_experts) atomicAdd(&count[e], 1u);
+    uint32_t my_e[MOE_GROUP_KEEP], my_pos[MOE_GROUP_KEEP];
+#pragma unroll
+    for (int i = 0; i < MOE_GROUP_KEEP; ++i) {
+        const uint32_t p = tid + (uint32_t)i * 1024u;
+        my_e[i] = p < n_pairs ? expert_idx[p] : 0xFFFFFFFFu;
+    }
+#pragma unroll
+    for (int i = 0; i < MOE_GROUP_KEEP; ++i) {
+        my_pos[i] = 0;
+        if (my_e[i] < n_experts) my_pos[i] = atomicAdd(&count[my_e[i]], 1u);   // out-of-range ids are dropped
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t t = 0;
-        for (uint32_t e = 0; e < n_experts; ++e) {
-            base[e] = t;
-            t += (count[e] + cap - 1u) / cap;
+    const bool more = n_pairs > MOE_GROUP_KEEP * 1024u;   // (uniform)
+    if (more) {
+        // pairs beyond the kept ones: counted now, placed behind the kept ones by a second read below
+        for (uint32_t e = tid; e < n_experts; e += 1024u) fill[e] = count[e];
+        __syncthreads();
+        for (uint32_t p = tid + MOE_GROUP_KEEP * 1024u; p < n_pairs; p += 1024u) {
+            const uint32_t e = expert_idx[p];
+            if (e < n_experts) atomicAdd(&count[e], 1u);
         }
-        *n_tiles = t;
+        __syncthreads();
     }
+    // exclusive scan of the experts' record counts: thread t owns experts 8t .. 8t+7
+    uint32_t nt[8], mine = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t e = tid * 8u + j;
+        nt[j] = e < n_experts ? (count[e] + cap - 1u) / cap : 0u;
+        mine += nt[j];
+    }
+    uint32_t incl = mine;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t v = __shfl_up(incl, o, 64);
+        if (lane >= (uint32_t)o) incl += v;
+    }
+    if (lane == 63u) wave_total[wave] = incl;
     __syncthreads();
+    uint32_t before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+        const uint32_t v = wave_total[w];
+        before += (uint32_t)w < wave ? v : 0u;
+        all += v;
+    }
+    uint32_t run = before + incl - mine;
     const uint32_t stride = 2u + cap;
-    for (uint32_t e = threadIdx.x; e < n_experts; e += blockDim.x) {
-        const uint32_t nt = (count[e] + cap - 1u) / cap;
-        for (uint32_t i = 0; i < nt; ++i) {
-            uint32_t* rec = tiles + (size_t)(base[e] + i) * stride;
-            rec[0] = e;
-            rec[1] = min(cap, count[e] - i * cap);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t e = tid * 8u + j;
+        if (e < n_experts) {
+            base[e] = run;
+            for (uint32_t i = 0; i < nt[j]; ++i) {
+                uint32_t* rec = tiles + (size_t)(run + i) * stride;
+                rec[0] = e;
+                rec[1] = min(cap, count[e] - i * cap);
+            }
+            run += nt[j];
         }
     }
-    for (uint32_t p = threadIdx.x; p < n_pairs; p += blockDim.x) {
-        const uint32_t e = expert_idx[p];
-        if (e >= n_experts) continue;   // out-of-range ids are dropped; their outputs stay untouched
-        const uint32_t pos = atomicAdd(&fill[e], 1u);
-        tiles[(size_t)(base[e] + pos / cap) * stride + 2u + pos % cap] = p;
+    if (tid == 0) *n_tiles = all;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MOE_GROUP_KEEP; ++i) {
+        const uint32_t e = my_e[i];
+        if (e < n_experts) tiles[(size_t)(base[e] + my_pos[i] / cap) * stride + 2u + my_pos[i] % cap] = tid + (uint32_t)i * 1024u;
+    }
+    if (more) {
+        for (uint32_t p = tid + MOE_GROUP_KEEP * 1024u; p < n_pairs; p += 1024u) {
+            const uint32_t e = expert_idx[p];
+            if (e >= n_experts) continue;
+            const uint32_t pos = atomicAdd(&fill[e], 1u);
+            tiles[(size_t)(base[e] + pos / cap) * stride + 2u + pos % cap] = p;
+        }
     }
 }
 
@@ -103,7 +157,7 @@ size_t moe_tiles_words(uint32_t n_pairs, uint32_t n_experts, int sets)
 hipError_t launch_moe_group(const uint32_t* expert_idx, uint32_t n_pairs, uint32_t n_experts, int sets, uint32_t* tiles,
                             uint32_t* n_tiles, hipStream_t s)
 {
-    if (n_experts > 8192u) return hipErrorInvalidValue;   // three LDS arrays of n_experts words
+    if (n_experts > 8192u) return hipErrorInvalidValue;   // three LDS arrays of n_experts words, eight experts per thread
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 3 * n_experts * sizeof(uint32_t), s, expert_idx, n_pairs,
                        n_experts, 2u * (uint32_t)sets, tiles, n_tiles);
     return hipGetLastError();

@@ -649,6 +649,25 @@ def test_moe_matmul_grouped_ragged(gpu, kqo, type_, N, K, per_slot, family, kern
     assert np.all(np.abs(got - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
 
 
+def test_moe_matmul_grouped_many_pairs(gpu, kqo):
+    """More pairs than the grouping pass keeps in registers (4 per thread of its one workgroup): the rest are
+    counted first and placed behind the kept ones by a second read."""
+    from backpack_amd import capi, kquant
+    type_, N, K = Q4_K, 128, 256
+    E, T, k = 20, 1100, 4
+    raw, packed, w = gpu.make_weight(type_, E * N, K, seed=71)
+    rng = np.random.default_rng(72)
+    eidx = rng.integers(0, E, size=(T, k)).astype(np.uint32)
+    eidx[::7, 0] = 3                                        # one crowded expert
+    X = rng.standard_normal((T, K)).astype(np.float32)
+    _say("moe grouped, many pairs", T * k)
+    got = kquant.moe_matmul(gpu.dev(X), w, gpu.dev(eidx.view(np.int32)), E, x_per_slot=False).cpu().numpy()
+    assert capi.last_kernel() == "mtile_grouped"
+    want = kqo.moe_matmul(type_, X, packed, eidx, N, K, x_per_slot=False)
+    rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    assert np.all(np.abs(got - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
+
+
 @pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True), (Q6_K, 300, 4096, False),
                                                  (Q5_K, 768, 2048, False), (Q5_K, 2048, 768, True), (Q5_K, 300, 4096, False)])
 def test_moe_matmul_few_pairs_stream(gpu, kqo, type_, N, K, per_slot):
