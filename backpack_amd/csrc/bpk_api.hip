@@ -79,7 +79,7 @@ struct DeviceState {
     kq::SplitScratch gemm_split{};   // of the bf16 GEMM's cut tiles (its own, so that it can run beside a GEMV)
     uint32_t* moe_tiles = nullptr;   // kMoeWords words
     uint32_t* argmax_scratch = nullptr;   // partial values | partial indices | tickets of bpk_argmax_rows
-    float* route_logits = nullptr;   // ROUTE_SPREAD_TOKENS x 1024 router logits of a small-T route call
+    float* route_logits = nullptr;   // ROUTE_SCRATCH_FLOATS router logits of a route call that does not return them
     uint32_t* argmax_static = nullptr;    // this device's copy of the scratch array in the code object (not allocated)
     UploadStage up{};                // created by the first upload on the device
 };
@@ -121,7 +121,7 @@ int ensure_device(int device, DeviceState** out)
         constexpr size_t kArgmaxWords = (size_t)kq::ARGMAX_MAX_ROWS * (2u * kq::ARGMAX_PARTS + 1u);
         if (e == hipSuccess) e = hipMalloc((void**)&st.argmax_scratch, kArgmaxWords * sizeof(uint32_t));
         if (e == hipSuccess) e = hipMemset(st.argmax_scratch, 0, kArgmaxWords * sizeof(uint32_t));
-        if (e == hipSuccess) e = hipMalloc((void**)&st.route_logits, kq::ROUTE_SPREAD_TOKENS * 1024u * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc((void**)&st.route_logits, kq::ROUTE_SCRATCH_FLOATS * sizeof(float));
         if (e == hipSuccess) e = kq::argmax_static_scratch(&st.argmax_static);   // with `device` current
         if (e != hipSuccess) {
             // nothing half-made stays behind: a later call starts from scratch

@@ -66,6 +66,7 @@ hipError_t launch_add_residual(const float* T, const float* R, float* Y, uint32_
 hipError_t launch_topk_softmax(const float* logits, uint32_t T, uint32_t n_experts, uint32_t k, int normalize,
                                uint32_t* idx, float* wt, hipStream_t s);
 constexpr uint32_t ROUTE_SPREAD_TOKENS = 64;   // fewer tokens: experts spread over workgroups, two launches
+constexpr uint32_t ROUTE_SCRATCH_FLOATS = 1u << 20;   // the library's own place for router logits (4 MB)
 hipError_t launch_route(const float* X, const float* router_w, uint32_t T, uint32_t hidden, uint32_t n_experts,
                         uint32_t k, int normalize, float* logits_out, float* logits_scratch, uint32_t* idx, float* wt,
                         hipStream_t s);

@@ -46,13 +46,16 @@ __device__ __forceinline__ void route_select(float (&vals)[PER_LANE], uint32_t l
         else if ((bi & 63u) == lane) taken |= 1u << (bi >> 6);
         if (lane == s) { my_v = bv; my_i = bi; }
     }
+    // (the picks sit in lanes 0 .. k-1 of the first row of 16, k <= 16: DPP moves inside that row, lane 0 has the result)
     float mx = lane < k ? my_v : ROUTE_NEG_INF;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    mx = fmaxf(mx, group_partner<1>(mx)); mx = fmaxf(mx, group_partner<2>(mx));
+    mx = fmaxf(mx, group_partner<4>(mx)); mx = fmaxf(mx, group_partner<8>(mx));
+    mx = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mx), 0));
     const float ex = lane < k ? expf(my_v - mx) : 0.0f;
     float sum = ex;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) sum += __shfl_xor(sum, o);
+    sum += group_partner<1>(sum); sum += group_partner<2>(sum);
+    sum += group_partner<4>(sum); sum += group_partner<8>(sum);
+    sum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sum), 0));
     const float inv = (normalize && sum > 0.0f) ? 1.0f / sum : 1.0f;
     if (lane < k) {
         idx_out[lane] = my_i;
@@ -115,9 +118,7 @@ __device__ __forceinline__ void route_dot4(const float* x, const float* router_w
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) acc[j] += __shfl_xor(acc[j], o);
-        out[j] = acc[j];
+        out[j] = wave_total(acc[j]);   // (DPP moves: an LDS-routed shuffle costs a hundred cycles)
     }
 }
 
@@ -153,20 +154,69 @@ __global__ __launch_bounds__(256) void route_kernel(const float* X, const float*
     route_select_any(vals, lane, n_experts, k, normalize, idx + (size_t)tok * k, wt + (size_t)tok * k);
 }
 
-// Few tokens: the experts are spread over workgroups (blockIdx.x takes 16 of them, blockIdx.y is the token)
-// and the selection is a launch of its own.
-__global__ __launch_bounds__(256) void route_logits_kernel(const float* X, const float* router_w, uint32_t hidden,
-                                                           uint32_t n_experts, float* logits_out)
+// A workgroup takes TB tokens x 4 experts (many tokens: 8, so a router row is fetched once per 8 tokens instead of
+// once per token); its four waves take every fourth step along hidden (lanes along hidden inside a step) and their
+// sums meet in LDS, in wave order.  The selection is a launch of its own.  Tokens and experts beyond the end
+// repeat the last one (their sums are dropped).
+template <int TB>   // tokens per workgroup: 8, or 1 for a few tokens
+__global__ __launch_bounds__(256) void route_logits_tiled_kernel(const float* X, const float* router_w, uint32_t T,
+                                                                 uint32_t hidden, uint32_t n_experts, float* logits_out)
 {
+    __shared__ float part[4][4 * TB];
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const uint32_t tok = blockIdx.y;
-    const uint32_t e0 = blockIdx.x * 16u + wave * 4u;
-    if (e0 >= n_experts) return;
-    float v[4];
-    route_dot4(X + (size_t)tok * hidden, router_w, hidden, n_experts, e0, lane, v);
+    const uint32_t t0 = blockIdx.y * TB, e0 = blockIdx.x * 4u;
+    const uint32_t h4 = hidden / 4u;
+    const float4* x4[TB];
+    const float4* w4[4];
+#pragma unroll
+    for (int t = 0; t < TB; ++t) x4[t] = (const float4*)(X + (size_t)min(t0 + t, T - 1u) * hidden);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w4[j] = (const float4*)(router_w + (size_t)min(e0 + j, n_experts - 1u) * hidden);
+    float acc[4][TB];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-        if (lane == (uint32_t)j && e0 + j < n_experts) logits_out[(size_t)tok * n_experts + e0 + j] = v[j];
+#pragma unroll
+        for (int t = 0; t < TB; ++t) acc[j][t] = 0.0f;
+    // (the next step's loads are in flight while this step is multiplied)
+    float4 a[TB], b[4];
+    auto fetch = [&](uint32_t i) {
+        const uint32_t ic = min(i, h4 - 1u);
+#pragma unroll
+        for (int t = 0; t < TB; ++t) a[t] = x4[t][ic];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = w4[j][ic];
+    };
+    fetch(wave * 64u + lane);
+    for (uint32_t i = wave * 64u + lane; i < h4; i += 256u) {
+        float4 ca[TB], cb[4];
+#pragma unroll
+        for (int t = 0; t < TB; ++t) ca[t] = a[t];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) cb[j] = b[j];
+        fetch(i + 256u);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < TB; ++t) {
+                acc[j][t] = fmaf(ca[t].x, cb[j].x, acc[j][t]);
+                acc[j][t] = fmaf(ca[t].y, cb[j].y, acc[j][t]);
+                acc[j][t] = fmaf(ca[t].z, cb[j].z, acc[j][t]);
+                acc[j][t] = fmaf(ca[t].w, cb[j].w, acc[j][t]);
+            }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+            const float v = wave_total(acc[j][t]);
+            if (lane == (uint32_t)(j * TB + t)) part[wave][j * TB + t] = v;
+        }
+    __syncthreads();
+    if (threadIdx.x < 4u * TB) {
+        const uint32_t j = threadIdx.x / TB, t = threadIdx.x % TB;
+        const float v = ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) + part[3][threadIdx.x];
+        if (e0 + j < n_experts && t0 + t < T) logits_out[(size_t)(t0 + t) * n_experts + e0 + j] = v;
+    }
 }
 
 hipError_t launch_topk_softmax(const float* logits, uint32_t T, uint32_t n_experts, uint32_t k, int normalize,
@@ -181,12 +231,19 @@ hipError_t launch_route(const float* X, const float* router_w, uint32_t T, uint3
                         uint32_t k, int normalize, float* logits_out, float* logits_scratch, uint32_t* idx, float* wt,
                         hipStream_t s)
 {
-    // logits_scratch holds ROUTE_SPREAD_TOKENS x 1024 floats: below that many tokens a workgroup per token
-    // would leave most of the machine idle
+    // logits_scratch holds ROUTE_SCRATCH_FLOATS floats (at least ROUTE_SPREAD_TOKENS x 1024): below that many
+    // tokens a workgroup per token would leave most of the machine idle
     if (T < ROUTE_SPREAD_TOKENS && logits_scratch) {
         float* lg = logits_out ? logits_out : logits_scratch;
-        hipLaunchKernelGGL(route_logits_kernel, dim3((n_experts + 15u) / 16u, T), dim3(256), 0, s, X, router_w, hidden,
-                           n_experts, lg);
+        hipLaunchKernelGGL(route_logits_tiled_kernel<1>, dim3((n_experts + 3u) / 4u, T), dim3(256), 0, s, X, router_w, T,
+                           hidden, n_experts, lg);
+        return launch_topk_softmax(lg, T, n_experts, k, normalize, idx, wt, s);
+    }
+    // many tokens: logits by 8-token tiles, then the selection, as long as the logits have a place to go
+    if (T >= ROUTE_SPREAD_TOKENS && (logits_out || (logits_scratch && (uint64_t)T * n_experts <= ROUTE_SCRATCH_FLOATS))) {
+        float* lg = logits_out ? logits_out : logits_scratch;
+        hipLaunchKernelGGL(route_logits_tiled_kernel<8>, dim3((n_experts + 3u) / 4u, (T + 7u) / 8u), dim3(256), 0, s, X,
+                           router_w, T, hidden, n_experts, lg);
         return launch_topk_softmax(lg, T, n_experts, k, normalize, idx, wt, s);
     }
     hipLaunchKernelGGL(route_kernel, dim3(T), dim3(256), 0, s, X, router_w, hidden, n_experts, k, normalize,

@@ -22,6 +22,20 @@ __device__ __forceinline__ float group_partner(float x)
     return __builtin_bit_cast(float, group_partner<OFF>(__builtin_bit_cast(int, x)));
 }
 
+// The sum over the wave, in every lane: four DPP steps inside the rows of 16, then the four rows' values.
+__device__ __forceinline__ float wave_total(float v)
+{
+    v += group_partner<1>(v);
+    v += group_partner<2>(v);
+    v += group_partner<4>(v);
+    v += group_partner<8>(v);
+    const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (a + b) + (c + d);
+}
+
 // The better of two (value, index) candidates: larger value, then lower index.
 __device__ __forceinline__ void best_of(float& v, uint32_t& i, float ov, uint32_t oi)
 {

@@ -457,7 +457,7 @@ BPK_API int bpk_moe_topk_softmax(const float *logits, uint32_t T,
                                  uint32_t n_experts, uint32_t k, int normalize,
                                  uint32_t *idx, float *wt, void *stream);
 
-/* The same behind the router matvec, one launch: logits[t, e] = sum_h X[t, h] *
+/* The same behind the router matvec, one call (two launches): logits[t, e] = sum_h X[t, h] *
  * router_w[e, h] in fp32 (GGUF keeps `ffn_gate_inp.weight` as F32 [hidden,
  * n_experts]; the reference requantises it to Q8 for its Q8 matmul,
  * model_runner.cpp:3532-3540).  `logits` may be NULL when the caller does not

@@ -61,7 +61,11 @@ def test_topk_ties_masks_and_degenerate_rows(gpu, kqo):
     assert np.all(both_nan | (np.abs(got_wt - want_wt) <= 2e-7))
 
 
-@pytest.mark.parametrize("T,H,E,k", [(1, 2048, 128, 8), (256, 2048, 128, 8), (3, 4096, 256, 8), (2, 36, 10, 3)])
+@pytest.mark.parametrize("T,H,E,k", [(1, 2048, 128, 8), (256, 2048, 128, 8), (3, 4096, 256, 8), (2, 36, 10, 3),
+                                     # many tokens: logits by tiles of 8 tokens x 16 experts (ragged in both), then the selection
+                                     (70, 1024, 60, 4), (100, 36, 10, 3),
+                                     # ... and more logits than the library's own buffer holds when none are asked for
+                                     (9000, 64, 128, 8)])
 def test_route_matvec_and_selection(gpu, kqo, T, H, E, k):
     """Logits against a float64 contraction; the selection must be the oracle's selection on the
     logits the GPU produced (a near-tie may legitimately order differently on other logits)."""
