@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include "kq_kernels.h"
+#include "kq_wave.h"
 
 namespace kq {
 
@@ -28,8 +29,7 @@ __global__ __launch_bounds__(256) void rms_norm_rows_kernel(const float* X, cons
     const float* x = X + (size_t)blockIdx.x * K;
     float ss = 0.0f;
     for (uint32_t k = threadIdx.x; k < K; k += 256u) ss = __builtin_fmaf(x[k], x[k], ss);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    ss = wave_total(ss);
     if ((threadIdx.x & 63u) == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
     const float rstd = 1.0f / sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)K + eps);

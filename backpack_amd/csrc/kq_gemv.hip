@@ -83,8 +83,11 @@ __device__ __forceinline__ void stage_x_sums(const float* __restrict__ X, uint32
                 const float4 v = x4[c];
                 s = (v.x + v.y) + (v.z + v.w);
             }
-#pragma unroll
-            for (int off = 1; off < LANES; off <<= 1) s += __shfl_xor(s, off, 64);
+            // (DPP moves inside the group of 4 or 8 lanes: an LDS-routed shuffle costs a hundred cycles)
+            static_assert(LANES == 4 || LANES == 8, "a run is held by 4 or 8 lanes");
+            s += group_partner<1>(s);
+            s += group_partner<2>(s);
+            if (LANES > 4) s += group_partner<4>(s);
             if (c < chunks && (threadIdx.x % LANES) == 0) xs[(size_t)m * nblk * (256 / SEG) + c / LANES] = s;
         }
     }

@@ -986,8 +986,9 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
         if (normed) {
             // thread t converted for token t / 32: the sums of this workgroup's part of K, per token
             float ss = stager.ss;
-            ss += __shfl_xor(ss, 16, 64); ss += __shfl_xor(ss, 8, 64); ss += __shfl_xor(ss, 4, 64);
-            ss += __shfl_xor(ss, 2, 64); ss += __shfl_xor(ss, 1, 64);
+            ss += group_partner<1>(ss); ss += group_partner<2>(ss); ss += group_partner<4>(ss);
+            ss += group_partner<8>(ss);          // (DPP moves inside the row of 16 ...
+            ss += __shfl_xor(ss, 16, 64);        //  ... and one exchange between the token's two rows)
             if ((threadIdx.x & 31u) == 0u) rinv[threadIdx.x >> 5] = ss;
             __syncthreads();
         }
