@@ -216,7 +216,7 @@ int bpk_set_option(const char* name, int value)
         return BPK_OK;
     }
     if (!strcmp(name, "chain_spin_us")) {
-        if (value < 0) return fail(BPK_ERR_SHAPE, "chain_spin_us must not be negative");
+        if (value < 0 || value > 10000000) return fail(BPK_ERR_SHAPE, "chain_spin_us must lie in 0 .. 10000000 (ten seconds)");
         t_chain_spin_us = value;
         return BPK_OK;
     }
@@ -778,7 +778,8 @@ int bpk_chain_create(const bpk_chain_op* ops, uint32_t n_ops, bpk_chain** out)
             }
         }
     }
-    if (kq::chain_lds_bytes(max_k) > kq::CHAIN_MAX_LDS) return fail(BPK_ERR_SHAPE, "K=%u exceeds what a workgroup can stage", max_k);
+    if (max_k > kq::CHAIN_MAX_K || kq::chain_lds_bytes(max_k) > kq::CHAIN_MAX_LDS)
+        return fail(BPK_ERR_SHAPE, "K=%u exceeds what a workgroup can stage (K <= %u)", max_k, kq::CHAIN_MAX_K);
     bpk_chain* c = new (std::nothrow) bpk_chain;
     if (!c) return fail(BPK_ERR_SHAPE, "out of host memory");
     (void)hipGetDevice(&c->device);
@@ -849,6 +850,10 @@ int bpk_chain_run(bpk_chain* c, uint32_t first, uint32_t count, void* stream)
         }
         if (c->checked.size() < 4096u) c->checked.push_back(key);
     }
+    // the hold hook exists for the tests of the give-up path: it is taken only with a short bound on the waits,
+    // so that a stray setting cannot make every launch spin for the default two seconds
+    if (t_chain_hold && (t_chain_spin_us <= 0 || t_chain_spin_us > 100000))
+        return fail(BPK_ERR_SHAPE, "chain_hold is a test hook and needs chain_spin_us set to 1 .. 100000 first");
     kq::ChainLaunch a{};
     a.ops = c->d_ops;
     a.parity = c->d_words;
@@ -875,8 +880,14 @@ int bpk_chain_trace(void* stamps)
 int bpk_chain_status(bpk_chain* c)
 {
     if (!c) return fail(BPK_ERR_NULL, "chain must be non-null");
+    int dev = -1;
+    (void)hipGetDevice(&dev);
+    if (dev != c->device) return fail(BPK_ERR_DEVICE, "the chain was created on device %d, current is %d", c->device, dev);
+    // every stream of the device, non-blocking ones included: a launch that is still waiting may yet give up
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return hip_fail(e, "waiting for the chain's launches");
     uint32_t word = 0;
-    const hipError_t e = hipMemcpy(&word, c->d_words + c->n_ops + 1u, sizeof word, hipMemcpyDeviceToHost);
+    e = hipMemcpy(&word, c->d_words + c->n_ops + 1u, sizeof word, hipMemcpyDeviceToHost);
     if (e != hipSuccess) return hip_fail(e, "reading the chain's error word");
     if (word == 0) return BPK_OK;
     return fail(BPK_ERR_TIMEOUT, "a launch of the chain gave up waiting for the inputs of op %u (the grid was not all "

@@ -72,13 +72,33 @@ void releaseBuffer(GPUBuffer& b)
 
 GPUBuffer uploadKQWeight(const std::string& name, const KQuantPacked& w)
 {
-    GPUBuffer b = createBuffer(name, w.data.size() * sizeof(uint32_t));
-    if (b.handle) writeBuffer(b, w.data.data(), w.data.size() * sizeof(uint32_t));
+    // the kernels fetch packed rows in 16-byte pieces: the allocation carries KQ_WEIGHT_TAIL_BYTES readable
+    // (zeroed) bytes behind the last row, as bpk_weight_create's does
+    const size_t bytes = w.data.size() * sizeof(uint32_t);
+    GPUBuffer b = createBuffer(name, bytes + KQ_WEIGHT_TAIL_BYTES);
+    if (!b.handle) return b;
+    if (bytes) writeBuffer(b, w.data.data(), bytes);
+    if (hipMemset((char*)b.handle + bytes, 0, KQ_WEIGHT_TAIL_BYTES) != hipSuccess) fprintf(stderr, "uploadKQWeight(%s): clearing the tail failed\n", name.c_str());
     return b;
+}
+
+int checkKQWeightView(GGUFType type, const GPUBuffer& W, uint32_t rows, uint32_t rowStrideWords, const std::string& name)
+{
+    if (!W.handle) return BPK_OK;   // the library reports the missing pointer
+    const size_t need = (size_t)rows * rowStrideWords * sizeof(uint32_t) + (type == GGUF_TYPE_Q6_K ? KQ_WEIGHT_TAIL_BYTES : 0);
+    if (W.offset > W.size || W.size - W.offset < need) {
+        fprintf(stderr, "[%s] weight view of %zu bytes at offset %zu is smaller than the %zu bytes its %u rows need%s\n",
+                name.c_str(), W.size, W.offset, need, rows,
+                type == GGUF_TYPE_Q6_K ? " (Q6_K rows are fetched in 16-byte pieces: 16 readable bytes must follow the last row; "
+                                         "uploadKQWeight allocates them)" : "");
+        return BPK_ERR_SHAPE;
+    }
+    return BPK_OK;
 }
 
 int KQDispatch::run(void* stream) const
 {
+    if (const int bad = checkKQWeightView(type, W, P.v[1], P.v[3], name)) return bad;
     const int rc = bpk_kq_matmul((int)type, (const float*)X.ptr(), W.ptr(), (const float*)Bias.ptr(), (float*)Y.ptr(), M,
                                  P.v[1], P.v[0], P.v[2], P.v[3], P.v[4], stream);
     if (rc != BPK_OK) fprintf(stderr, "[%s] %s\n", name.c_str(), bpk_last_error());
@@ -97,6 +117,8 @@ int gatherKQ(GGUFType type, const GPUBuffer& W, uint32_t rowStrideWords, const G
 int KQFusedDispatch::run(void* stream) const
 {
     const KQDispatch& d = base;
+    // with an epilogue W holds gate rows and up rows: twice the outputs
+    if (const int bad = checkKQWeightView(d.type, d.W, d.P.v[1] * (epilogue != BPK_EPI_NONE ? 2u : 1u), d.P.v[3], d.name)) return bad;
     bpk_kq_fusion f{prologue, (const float*)NormW.ptr(), eps, (const float*)Residual.ptr(), epilogue};
     const int rc = bpk_kq_matmul_fused((int)d.type, (const float*)d.X.ptr(), d.W.ptr(), (const float*)d.Bias.ptr(),
                                        (float*)d.Y.ptr(), d.M, d.P.v[1], d.P.v[0], d.P.v[2], d.P.v[3], d.P.v[4], &f,
@@ -119,6 +141,7 @@ int KQChain::build()
             fprintf(stderr, "%s: a chain takes one token per dispatch\n", d.name.c_str());
             return BPK_ERR_SHAPE;
         }
+        if (const int bad = checkKQWeightView(d.type, d.W, d.P.v[1] * (f.epilogue != BPK_EPI_NONE ? 2u : 1u), d.P.v[3], d.name)) return bad;
         ops[i] = bpk_chain_op{(int)d.type, (const float*)d.X.ptr(), d.W.ptr(), (const float*)d.Bias.ptr(), (float*)d.Y.ptr(),
                               d.P.v[1], d.P.v[0], d.P.v[2], d.P.v[3], d.P.v[4],
                               bpk_kq_fusion{f.prologue, (const float*)f.NormW.ptr(), f.eps, (const float*)f.Residual.ptr(),
@@ -219,7 +242,7 @@ bool GGUFFile::loadKQWeight(const std::vector<std::string>& names, GPUBuffer& W,
     }
     bpk_weight_desc d;
     bpk_weight_describe(*owner, &d);
-    W = GPUBuffer{d.data, d.bytes, 0};
+    W = GPUBuffer{d.data, d.bytes + KQ_WEIGHT_TAIL_BYTES, 0};   // the library's allocation carries the readable tail
     desc = KQuantPacked{};
     desc.N = d.N; desc.K = d.K; desc.rowStrideWords = d.row_stride_words; desc.nBlocks = d.n_blocks;
     desc.type = (GGUFType)d.type;

@@ -52,7 +52,14 @@ void writeBuffer(const GPUBuffer& b, const void* src, size_t bytes);
 void readBuffer(const GPUBuffer& b, void* dst, size_t bytes);   // synchronises the device
 void releaseBuffer(GPUBuffer& b);
 
+// Packed rows are fetched in 16-byte pieces and Q6_K blocks are 210 bytes, so a Q6_K weight must stay readable
+// for this many bytes behind its last row (include/bpk_kquant.h, bpk_kq_matmul).  uploadKQWeight allocates and
+// zeroes them; a buffer made some other way has to provide them itself.
+constexpr size_t KQ_WEIGHT_TAIL_BYTES = 16;
 GPUBuffer uploadKQWeight(const std::string& name, const KQuantPacked& w);
+// Host-side check every dispatch below runs before it launches: the view W must hold `rows` packed rows and,
+// for Q6_K, the readable tail.  Returns BPK_OK or BPK_ERR_SHAPE (message on stderr); touches no device.
+int checkKQWeightView(GGUFType type, const GPUBuffer& W, uint32_t rows, uint32_t rowStrideWords, const std::string& name);
 
 struct KQParams { uint32_t v[5]; };
 inline KQParams makeKQParams(uint32_t K, uint32_t N, uint32_t nBlocks, uint32_t rowStride, uint32_t yOffset = 0)

@@ -208,6 +208,7 @@ __device__ __forceinline__ bool chain_stage_x(const ChainOp& p, const float* mai
 {
     if (p.K <= 4096u) return chain_stage_x_n<4>(p, mail, par, pt, xs, red, gave_up, wave, lane);
     if (p.K <= 9216u) return chain_stage_x_n<9>(p, mail, par, pt, xs, red, gave_up, wave, lane);
+    static_assert(18u * 2u * CHAIN_THREADS >= CHAIN_MAX_K, "the widest staging form must cover the longest row a chain accepts");
     return chain_stage_x_n<18>(p, mail, par, pt, xs, red, gave_up, wave, lane);
 }
 
@@ -691,7 +692,7 @@ __global__ __launch_bounds__(CHAIN_THREADS) void chain_kernel(ChainLaunch a)
 
 int chain_mode_for(int type, uint32_t n_blocks, int epi)
 {
-    if (n_blocks == 0 || n_blocks > 16u * CW) return -1;
+    if (n_blocks == 0 || n_blocks > 16u * CW || n_blocks * KQ_QK > CHAIN_MAX_K) return -1;
     if (type != KQ_TYPE_Q4_K && type != KQ_TYPE_Q6_K) return -1;
     // rows of up to 16 superblocks are held whole by a wave, longer ones as K slices of 8 or 16 per wave
     uint32_t mode = type == KQ_TYPE_Q6_K ? CHAIN_MODE_Q6 : 0u;

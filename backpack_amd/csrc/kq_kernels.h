@@ -180,6 +180,9 @@ constexpr uint32_t CHAIN_MAX_OPS = 1024;
 constexpr uint32_t CHAIN_TRACE_POINTS = 8;
 constexpr uint32_t CHAIN_MAX_PER_LAUNCH = 64;   // ops one launch walks (their descriptors sit in LDS)
 constexpr size_t CHAIN_MAX_LDS = (size_t)156 << 10;   // dynamic LDS a chain launch may ask for
+// longest X row a chain op may have: what the widest staging form (18 pairs per thread of 512) covers, and what
+// fits the dynamic LDS beside the descriptors and the waves' staging windows
+constexpr uint32_t CHAIN_MAX_K = 18432;
 constexpr uint32_t CHAIN_ERR_TIMEOUT = 1u; // low byte of the error word; the op index sits above it
 struct ChainLaunch {
     const ChainOp* ops;

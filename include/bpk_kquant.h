@@ -94,7 +94,8 @@ typedef struct bpk_weight_desc {
     uint32_t n_blocks;         /* superblocks per row            */
     uint32_t row_stride_words; /* words per packed row           */
     void *data;                /* device address of row 0        */
-    size_t bytes;              /* size of the device allocation  */
+    size_t bytes;              /* N*row_stride_words*4, the packed rows; the allocation
+                                  holds 16 readable zero bytes more (see bpk_kq_matmul) */
 } bpk_weight_desc;
 
 /* parts[i] points at raw GGUF bytes (host) of an n_rows[i] x K matrix; the
@@ -289,6 +290,9 @@ BPK_API int bpk_kq_matmul_fused(int type, const float *X, const void *W,
                                 size_t workspace_bytes, void *stream);
 
 /* ---- chains of decode matvecs: replaces a recorded stretch of the dispatch list ----
+ * EXPERIMENTAL, not on the default path: measured slower per token than the same
+ * ops as separate bpk_kq_matmul_fused launches; what it buys is one launch per
+ * stretch.
  * The reference records one token's dispatches once (buildDecodePipeline) and
  * replays the list per token (runtime/model_runner.cpp:5725-5759).  Between two
  * attention blocks that list is k-quant matvecs and the elementwise dispatches
@@ -306,7 +310,8 @@ BPK_API int bpk_kq_matmul_fused(int type, const float *X, const void *W,
  * has its lowest mantissa bit cleared (a relative 2^-24; Y itself is exact).
  *
  * Each op: the arguments of bpk_kq_matmul_fused with M = 1 (N counts outputs; W
- * has 2N rows with an epilogue).  Served: Q4_K and Q6_K, K <= 32768, X and norm_w
+ * has 2N rows with an epilogue).  Served: Q4_K and Q6_K, K <= 18432 (the longest
+ * row a workgroup stages in LDS), X and norm_w
  * 16-byte aligned, Q4_K rows 16-byte aligned; the act(gate)*up epilogue for Q4_K
  * with K <= 4096.  An input must lie wholly inside one earlier op's outputs or
  * outside all of them; bpk_chain_create refuses anything else with
@@ -367,8 +372,8 @@ BPK_API int bpk_argmax_rows(const float *logits, uint32_t M, uint32_t N,
 
 /* bpk_argmax_rows for callers that cannot allocate device memory: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
- * has no counterpart in the reference (whose argmax dispatches bind buffers made
- * at load time, runtime/model_runner.cpp:2441-2453).  Same function and same
+ * has no counterpart in the reference (whose dispatches bind buffers made at
+ * load time).  Same function and same
  * kernel as bpk_argmax_rows; the per-row partial maxima and arrival tickets live
  * in an array inside the library's code object (132 096 bytes per GPU, held
  * until the process ends) instead of allocated scratch, and the call itself
@@ -507,10 +512,12 @@ BPK_API int bpk_force_kernel(int family);
  * through a per-device workspace and are added in the order of the walk, so
  * results repeat bit for bit); "fused_separate": 1 makes bpk_kq_matmul_fused run its prologue,
  * matmul and add as separate launches for every shape (needs the workspace);
- * "chain_spin_us": bound of a wait between the ops of a chain in microseconds;
- * "chain_hold": 1 keeps the ops of a chain from handing their outputs on, so
- * that every wait for them runs out (the way the tests reach the give-up path
- * with every workgroup exiting normally); "chain_ahead": 1 + the rows per wave
+ * "chain_spin_us": bound of a wait between the ops of a chain in microseconds
+ * (at most ten seconds);
+ * "chain_hold" (test hook, refused unless chain_spin_us is 1..100000): 1 keeps
+ * the ops of a chain from handing their outputs on, so that every wait for them
+ * runs out (the way the tests reach the give-up path with every workgroup
+ * exiting normally); "chain_ahead": 1 + the rows per wave
  * of the next op touched into L2 while an op finishes.  0 = automatic. */
 BPK_API int bpk_set_option(const char *name, int value);
 

@@ -383,8 +383,39 @@ TEST(model_config_from_gguf) {
     return {true, ""};
 }
 
-int main()
+// Host-only checks (no device is touched): a Q6_K weight view without the 16 readable bytes behind its last row
+// is refused before anything is launched; the same view with them passes the check.
+static int hostOnlyChecks()
 {
+    int failed = 0;
+    auto expect = [&](const char* what, bool ok) { printf("%-60s %s\n", what, ok ? "PASS" : "FAIL"); failed += !ok; };
+    const uint32_t N = 4096, K = 14336;
+    uint32_t nb = 0, rs = 0;
+    expect("layout of a Q6_K row", bpk_kq_layout(BPK_TYPE_Q6_K, K, &nb, &rs) == BPK_OK && nb == 56 && rs == 2940);
+    const size_t rows = (size_t)N * rs * 4;   // 11760 * 4096 bytes: a whole number of allocation granules
+    GPUBuffer exact{(void*)0x1000, rows, 0}, tailed{(void*)0x1000, rows + KQ_WEIGHT_TAIL_BYTES, 0};
+    expect("Q6_K view without the tail is refused", checkKQWeightView(GGUF_TYPE_Q6_K, exact, N, rs, "down") == BPK_ERR_SHAPE);
+    expect("Q6_K view with the tail passes", checkKQWeightView(GGUF_TYPE_Q6_K, tailed, N, rs, "down") == BPK_OK);
+    GPUBuffer sub{(void*)0x1000, rows + KQ_WEIGHT_TAIL_BYTES, rows / 2};
+    expect("Q6_K sub-view of the second half of the rows passes", checkKQWeightView(GGUF_TYPE_Q6_K, sub, N / 2, rs, "down") == BPK_OK);
+    expect("Q6_K sub-view that runs past the allocation is refused",
+           checkKQWeightView(GGUF_TYPE_Q6_K, sub, N / 2 + 1, rs, "down") == BPK_ERR_SHAPE);
+    expect("Q4_K needs no tail", checkKQWeightView(GGUF_TYPE_Q4_K, GPUBuffer{(void*)0x1000, (size_t)N * 576 * 4, 0}, N, 576, "o") == BPK_OK);
+    // the dispatches run the check before they launch: a refused view returns without a device call
+    KQDispatch d{GGUF_TYPE_Q6_K, GPUBuffer{(void*)0x2000, (size_t)K * 4, 0}, exact, GPUBuffer{}, GPUBuffer{(void*)0x3000, (size_t)N * 4, 0},
+                 makeKQParams(K, N, nb, rs), 1, "down"};
+    expect("KQDispatch::run refuses it", d.run() == BPK_ERR_SHAPE);
+    KQFusedDispatch f; f.base = d;
+    expect("KQFusedDispatch::run refuses it", f.run() == BPK_ERR_SHAPE);
+    KQChain c; c.add(f);
+    expect("KQChain::build refuses it", c.build() == BPK_ERR_SHAPE);
+    printf("%d host-only checks failed\n", failed);
+    return failed ? 1 : 0;
+}
+
+int main(int argc, char** argv)
+{
+    if (argc > 1 && !strcmp(argv[1], "--host-only")) return hostOnlyChecks();
     if (bpk_init(0) != BPK_OK) { fprintf(stderr, "bpk_init: %s\n", bpk_last_error()); return 2; }
     int failed = 0;
     for (auto& t : registry()) {

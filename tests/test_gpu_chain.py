@@ -230,6 +230,38 @@ def test_chain_wait_gives_up_and_recovers(gpu, kqo):
     assert torch.equal(d["qkv"], good)
 
 
+def test_chain_status_waits_for_launches_on_side_streams(gpu, kqo):
+    """bpk_chain_status synchronises with the device itself: a launch issued on a non-blocking side stream that is
+    still inside its bounded wait when status is called must be waited for and reported, without the caller
+    synchronising first."""
+    import torch
+    from backpack_amd import capi
+    ch, d, host, W = _layer(gpu, kqo, 1024, 2816, 256, seed=6, in_place=False)
+    ch.run()
+    torch.cuda.synchronize()
+    ch.status()
+    side = torch.cuda.Stream()
+    capi.set_option("chain_hold", 1)
+    with pytest.raises(capi.BpkError) as e:        # the hook is refused without a short bound on the waits
+        ch.run()
+    assert e.value.code == -2 and "chain_spin_us" in str(e.value)
+    capi.set_option("chain_spin_us", 50000)        # 50 ms: far longer than the host needs to reach status()
+    try:
+        with torch.cuda.stream(side):
+            ch.run()
+    finally:
+        capi.set_option("chain_hold", 0)
+        capi.set_option("chain_spin_us", 0)
+    with pytest.raises(capi.BpkError) as e:
+        ch.status()                                # no synchronize in between
+    assert e.value.code == -11
+    ch.reset()
+    ch.run()
+    ch.status()
+    with pytest.raises(capi.BpkError):
+        capi.set_option("chain_spin_us", 20000000)
+
+
 def test_chain_create_refusals(gpu):
     import torch
     from backpack_amd import capi, kquant
