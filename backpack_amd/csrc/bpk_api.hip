@@ -36,6 +36,7 @@ thread_local int t_chain_spin_us = 0;    // 0 = default
 thread_local int t_chain_ahead = 0;      // 1 + rows touched ahead; 0 = default
 thread_local void* t_chain_trace = nullptr;   // device buffer for the chain kernel's time stamps (diagnostics)
 thread_local int t_chain_hold = 0;
+thread_local int t_mgemv_auto = 1;       // option "mgemv": 0 keeps one-token Q4_K matvecs on the lanes-along-K kernel
 
 int fail(int code, const char* fmt, ...)
 {
@@ -181,7 +182,7 @@ const char* bpk_last_kernel(void) { return t_kernel; }
 
 int bpk_force_kernel(int family)
 {
-    if (family < 0 || family > 6) return fail(BPK_ERR_SHAPE, "kernel family %d unknown", family);
+    if (family < 0 || family > 7) return fail(BPK_ERR_SHAPE, "kernel family %d unknown", family);
     t_family = family;
     return BPK_OK;
 }
@@ -218,6 +219,10 @@ int bpk_set_option(const char* name, int value)
     if (!strcmp(name, "chain_spin_us")) {
         if (value < 0 || value > 10000000) return fail(BPK_ERR_SHAPE, "chain_spin_us must lie in 0 .. 10000000 (ten seconds)");
         t_chain_spin_us = value;
+        return BPK_OK;
+    }
+    if (!strcmp(name, "mgemv")) {
+        t_mgemv_auto = value != 0;
         return BPK_OK;
     }
     if (!strcmp(name, "chain_hold")) {
@@ -448,6 +453,17 @@ static int matmul_impl(int type, const float* X, const void* W, const float* bia
     if (t_family == 6 || (t_family == 0 && mtile_ok && ((M >= 3 && M <= 255 && !stream_four) || tile_two))) {
         t_kernel = "mtile";
         e = kq::launch_mtile(a, st->split, s);
+        return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+    }
+    // One token on a Q4_K matrix of many rows (gate|up): the contraction on the matrix cores.  The lanes-along-K
+    // kernel is bound by its vector arithmetic there and follows the part's clock: 28672 x 4096 took it 13.7 to
+    // 16.4 us from box to box, this kernel 13.6 to 14.4 (same runs; steady state 6.5 against 5.7-6.0 TB/s).
+    // Matrices of a few thousand rows have a tile or two per workgroup and stay (6144 x 4096: 6.7 against 5.7 us).
+    const bool mgemv_ok = kq::mgemv_supported(a);
+    if (t_family == 7 && !mgemv_ok) return fail(BPK_ERR_SHAPE, "matrix-core GEMV cannot serve this call");
+    if (t_family == 7 || (t_family == 0 && mgemv_ok && t_mgemv_auto && N >= 16384u)) {
+        t_kernel = "mgemv";
+        e = kq::launch_mgemv(a, kq::device_cu_count(), t_gemv.splits, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
     }
     if (t_family == 5 && !stream_ok) return fail(BPK_ERR_SHAPE, "lanes-along-K GEMV cannot serve this call");

@@ -114,6 +114,11 @@ hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const G
 bool gemv_stream_supported(const MatmulArgs& a);
 hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStream_t s);
 
+// One token on the matrix cores: Q4_K rows of up to 16 superblocks, 16-byte aligned (kq_mgemv.hip).
+bool mgemv_supported(const MatmulArgs& a);
+// form 1: sixteen waves of one superblock each (four waves per SIMD); otherwise eight waves of two
+hipError_t launch_mgemv(const MatmulArgs& a, uint32_t cus, int form, hipStream_t s);
+
 // 16-row x 16-token MFMA tiles for M = 2..16 (dense): weights read once for all tokens.
 bool mtile_supported(const MatmulArgs& a);
 hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s);

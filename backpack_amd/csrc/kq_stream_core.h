@@ -151,16 +151,12 @@ __device__ __forceinline__ void q4k_piece_dot(const s_u32x4 hdr, const s_u32x4 q
         for (int t = 0; t < MT; ++t) {
             alo[t] = s_fma_h(a.x, xlo[t][4 * m + 0], alo[t]);
             ahi[t] = s_fma_h(b.x, xhi[t][4 * m + 0], ahi[t]);
-#ifndef KQ_EXP_LESS_VALU
             alo[t] = s_fma_h(c.x, xlo[t][4 * m + 1], alo[t]);
             ahi[t] = s_fma_h(d.x, xhi[t][4 * m + 1], ahi[t]);
-#endif
             alo[t] = s_fma_h(a.y, xlo[t][4 * m + 2], alo[t]);
             ahi[t] = s_fma_h(b.y, xhi[t][4 * m + 2], ahi[t]);
-#ifndef KQ_EXP_LESS_VALU
             alo[t] = s_fma_h(c.y, xlo[t][4 * m + 3], alo[t]);
             ahi[t] = s_fma_h(d.y, xhi[t][4 * m + 3], ahi[t]);
-#endif
         }
     }
     // 6-bit scale and min of sub-blocks 2g and 2g+1: two adjacent bytes of each

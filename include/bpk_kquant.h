@@ -497,7 +497,8 @@ BPK_API const char *bpk_last_kernel(void);
  * 0 = automatic, 1 = generic, 2 = row-per-lane GEMV (M <= 4), 3 = row-per-lane
  * kernel on the 4x4x4 matrix-core op (M <= 16), 4 = matrix-core tiled GEMM
  * (bf16 X only), 5 = lanes-along-K GEMV (M = 1), 6 = 16-row x 16-token
- * matrix-core tiles (M <= 16).  A forced family that cannot serve the call's
+ * matrix-core tiles (M <= 16), 7 = one token on the matrix cores (Q4_K rows of
+ * up to 16 superblocks).  A forced family that cannot serve the call's
  * shape fails with BPK_ERR_SHAPE instead of falling back. */
 BPK_API int bpk_force_kernel(int family);
 
@@ -512,6 +513,8 @@ BPK_API int bpk_force_kernel(int family);
  * through a per-device workspace and are added in the order of the walk, so
  * results repeat bit for bit); "fused_separate": 1 makes bpk_kq_matmul_fused run its prologue,
  * matmul and add as separate launches for every shape (needs the workspace);
+ * "mgemv": 0 keeps one-token Q4_K matvecs of many rows on the lanes-along-K
+ * kernel (1, the default, takes them to the matrix-core kernel);
  * "chain_spin_us": bound of a wait between the ops of a chain in microseconds
  * (at most ten seconds);
  * "chain_hold" (test hook, refused unless chain_spin_us is 1..100000): 1 keeps

@@ -29,7 +29,7 @@ LAYER_SET = {
     "gate_up_q5": (Q5_K, 28672, 4096),
     "down_q5": (Q5_K, 4096, 14336),
 }
-SLACK = {"mrow": 1e-5, "mtile": 2e-5}
+SLACK = {"mrow": 1e-5, "mtile": 2e-5, "mgemv": 2e-5}
 
 
 def _say(*a):

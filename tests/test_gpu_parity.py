@@ -146,7 +146,7 @@ def test_q5k_matmul_vs_oracle(gpu, kqo, M, N, K, kernel):
 # units of the output rms: VALU kernels accumulate like the CPU; the matrix-core kernels feed
 # activations as fp16 hi + lo (22 bits relative to the largest element of the token's
 # superblock) and the MFMA adds its products with about 2^-19 relative alignment loss.
-SLACK = {"mrow": 1e-5, "mrow_grouped": 1e-5, "mtile": 2e-5}
+SLACK = {"mrow": 1e-5, "mrow_grouped": 1e-5, "mtile": 2e-5, "mgemv": 2e-5}
 
 SHAPES = [
     # type, M, N, K
@@ -209,7 +209,7 @@ SHAPES = [
 
 
 @pytest.mark.parametrize("type_,M,N,K", SHAPES)
-@pytest.mark.parametrize("family", [0, 1, 2, 3, 5, 6])
+@pytest.mark.parametrize("family", [0, 1, 2, 3, 5, 6, 7])
 def test_matmul_vs_oracle(gpu, kqo, type_, M, N, K, family):
     from backpack_amd import capi, kquant
     raw, packed, w = gpu.make_weight(type_, N, K, seed=N + K)
@@ -303,6 +303,70 @@ def test_gemv_stream_shapes(gpu, kqo, type_, N, K, depth, rows_per_wave, M):
         got = got[:, 7:]
     gpu.check_matmul(kqo, type_, got, X, packed, N, K, bias=bias,
                      label=f"stream {type_} {N}x{K} d{depth} r{rows_per_wave}")
+
+
+@pytest.mark.parametrize("form", [0, 1])
+@pytest.mark.parametrize("N,K", [(16, 256), (17, 512), (100, 4096), (1000, 2048), (333, 3840), (4099, 4096), (16400, 1792),
+                                 (40000, 768)])
+def test_matrix_core_gemv_shapes(gpu, kqo, N, K, form):
+    """One token on the matrix cores (what Q4_K matrices of 16384 rows and more get by default), forced on small
+    and ragged shapes: a last tile moved up to end at row N - 1, K slices that do not exist (fewer than 16
+    superblocks, odd counts), more than eight tiles per workgroup (two rounds of the waves' meeting), both forms
+    (eight waves of two superblocks, sixteen of one); with a y offset and bias, unit vectors, twice in a row."""
+    import torch
+    from backpack_amd import capi, kquant
+    raw, packed, w = gpu.make_weight(Q4_K, N, K, seed=N + 2)
+    rng = np.random.default_rng(N + form)
+    bias = rng.standard_normal(N).astype(np.float32)
+    out = torch.full((1, N + 3), 4.5, device="cuda")
+    capi.set_option("gemv_splits", form)
+    capi.force_kernel(7)
+    try:
+        for case in ("randn", "unit", "outlier"):
+            X = rng.standard_normal((1, K)).astype(np.float32)
+            if case == "unit":
+                X[:] = 0.0
+                X[0, int(rng.integers(K))] = 1.0
+            elif case == "outlier":
+                X[0, int(rng.integers(K))] = 3.0e4      # one huge activation: its superblock's other elements keep 22 bits of IT
+            _say("mgemv", N, K, form, case)
+            xd, bd = gpu.dev(X), gpu.dev(bias)
+            got = []
+            for _ in range(2):
+                out.fill_(4.5)
+                capi.check(capi.lib().bpk_kq_matmul(Q4_K, xd.data_ptr(), w.data.data_ptr(), bd.data_ptr(), out.data_ptr(), 1, N, K,
+                                                    w.n_blocks, w.row_stride_words, 3, None))
+                assert capi.last_kernel() == "mgemv"
+                got.append(out.cpu().numpy())
+            assert np.array_equal(got[0], got[1]), "two launches on the same inputs differ"
+            assert np.all(got[0][:, :3] == 4.5)
+            # (the outlier's products dominate the matrix instruction's running sums, whose additions lose alignment
+            # bits at about 2^-19 of the LARGEST addend: every output carries a few 1e-5 of the outlier's product)
+            gpu.check_matmul(kqo, Q4_K, got[0][:, 3:], X, packed, N, K, bias=bias, label=f"mgemv {N}x{K} form {form} {case}",
+                             slack=1e-4 if case == "outlier" else 2e-5)
+    finally:
+        capi.force_kernel(0)
+        capi.set_option("gemv_splits", 0)
+
+
+def test_matrix_core_gemv_is_the_choice_for_gate_up(gpu, kqo):
+    """The library's own choice: Q4_K, one token, 16384 rows or more -> the matrix-core kernel; the option switches it off."""
+    from backpack_amd import capi, kquant
+    N, K = 16384, 512
+    raw, packed, w = gpu.make_weight(Q4_K, N, K, seed=5)
+    X = np.random.default_rng(5).standard_normal((1, K)).astype(np.float32)
+    got = kquant.matmul(gpu.dev(X), w).cpu().numpy()
+    assert capi.last_kernel() == "mgemv"
+    gpu.check_matmul(kqo, Q4_K, got, X, packed, N, K, label="mgemv by choice", slack=2e-5)
+    capi.set_option("mgemv", 0)
+    try:
+        got2 = kquant.matmul(gpu.dev(X), w).cpu().numpy()
+        assert capi.last_kernel() == "gemv_stream"
+    finally:
+        capi.set_option("mgemv", 1)
+    gpu.check_matmul(kqo, Q4_K, got2, X, packed, N, K, label="stream with the option off")
+    two = kquant.matmul(gpu.dev(np.repeat(X, 2, axis=0)), w)
+    assert capi.last_kernel() != "mgemv"       # two tokens: not this kernel
 
 
 @pytest.mark.parametrize("N,K", [(1000, 4096), (70, 3072), (16500, 2304), (9, 4096)])
