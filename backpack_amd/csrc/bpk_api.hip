@@ -36,7 +36,7 @@ thread_local int t_chain_spin_us = 0;    // 0 = default
 thread_local int t_chain_ahead = 0;      // 1 + rows touched ahead; 0 = default
 thread_local void* t_chain_trace = nullptr;   // device buffer for the chain kernel's time stamps (diagnostics)
 thread_local int t_chain_hold = 0;
-thread_local int t_mgemv_auto = 1;       // option "mgemv": 0 keeps one-token Q4_K matvecs on the lanes-along-K kernel
+thread_local int t_mgemv_auto = 1;       // option "mgemv": 0 never, 1 from 49152 rows on, 2 from 16384 rows on
 
 int fail(int code, const char* fmt, ...)
 {
@@ -222,7 +222,8 @@ int bpk_set_option(const char* name, int value)
         return BPK_OK;
     }
     if (!strcmp(name, "mgemv")) {
-        t_mgemv_auto = value != 0;
+        if (value < 0 || value > 2) return fail(BPK_ERR_SHAPE, "mgemv must be 0, 1 or 2");
+        t_mgemv_auto = value;
         return BPK_OK;
     }
     if (!strcmp(name, "chain_hold")) {
@@ -455,13 +456,16 @@ static int matmul_impl(int type, const float* X, const void* W, const float* bia
         e = kq::launch_mtile(a, st->split, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
     }
-    // One token on a Q4_K matrix of many rows (gate|up): the contraction on the matrix cores.  The lanes-along-K
-    // kernel is bound by its vector arithmetic there and follows the part's clock: 28672 x 4096 took it 13.7 to
-    // 16.4 us from box to box, this kernel 13.6 to 14.4 (same runs; steady state 6.5 against 5.7-6.0 TB/s).
-    // Matrices of a few thousand rows have a tile or two per workgroup and stay (6144 x 4096: 6.7 against 5.7 us).
+    // One token on a Q4_K matrix of very many rows: the contraction on the matrix cores.  Its steady state is
+    // faster than the lanes-along-K kernel's (6.5 against 5.7-6.0 TB/s: 114688 x 4096 takes 44.3 against 48.7 us,
+    // 57344 x 4096 23.9 against 25.3), its start and end are not (x is split and laid out as operands before the
+    // first product, the waves meet before the stores), and on gate|up's 28672 x 4096 the two are level — 13.9
+    // against 13.9-14.0 us alone; inside the decode step the lanes-along-K kernel is 0.3 us ahead per launch, and
+    // every other kernel of the step ran 1 % slower next to this one (1.219 against 1.210 ms on four boxes).  On
+    // parts whose clock runs low the order flips (14.4 against 15.8-16.4 us).  So: from 49152 rows on.
     const bool mgemv_ok = kq::mgemv_supported(a);
     if (t_family == 7 && !mgemv_ok) return fail(BPK_ERR_SHAPE, "matrix-core GEMV cannot serve this call");
-    if (t_family == 7 || (t_family == 0 && mgemv_ok && t_mgemv_auto && N >= 16384u)) {
+    if (t_family == 7 || (t_family == 0 && mgemv_ok && N >= (t_mgemv_auto == 2 ? 16384u : 49152u) && t_mgemv_auto)) {
         t_kernel = "mgemv";
         e = kq::launch_mgemv(a, kq::device_cu_count(), t_gemv.splits, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);

@@ -24,8 +24,8 @@
 // Three tiles of weights are in flight per wave; their loads are issued from inline asm and waited for by hand
 // (the compiler's own placement drains the whole queue at every refill inside a loop), under the rules written
 // out in kq_stream_core.h: KQ_REQUIRES_NO_SPILL, every register a load fills passes through the wait that
-// names it, the number of loads in flight is the same at every wait (past its last tile a wave fetches the
-// last tile again and drops it).
+// names it, the number of loads in flight is the same at every wait (past its last tile a wave issues its
+// requests with no lane active).
 //
 // Results differ from the lanes-along-K kernel's by the hi + lo split of x: 22 bits relative to the largest
 // |x| of a superblock.
@@ -68,6 +68,49 @@ __device__ __forceinline__ void mg_load16(g_u32x4& v, uint32_t off, const uint8_
     v = *(const g_u32x4*)(base + off);
 #else
     asm volatile("global_load_dwordx4 %0, %1, %2 ; ringld" : "+v"(v) : "v"(off), "s"(base));
+#endif
+}
+
+// The loads of one tile as one statement, issued with no lane active when `on` is zero: such a load moves nothing
+// but keeps its place in the memory counter, so the number of loads in flight is the same at every wait and a
+// wave past its last tile requests nothing real.  (One statement: the compiler must not place an instruction of
+// its own between the change of EXEC and its restoration.)
+__device__ __forceinline__ void mg_request(g_u32x4 (&d)[5], const uint32_t (&o)[5], const uint8_t* base, uint32_t on)
+{
+#ifdef KQ_TRACKED_LOADS
+    if (on)
+        for (int k = 0; k < 5; ++k) d[k] = *(const g_u32x4*)(base + o[k]);
+#else
+    uint64_t saved;
+    asm volatile("s_mov_b64 %[sv], exec\n\t"
+                 "s_and_b32 exec_lo, exec_lo, %[on]\n\t"
+                 "s_and_b32 exec_hi, exec_hi, %[on]\n\t"
+                 "global_load_dwordx4 %0, %6, %[b] ; ringld\n\t"
+                 "global_load_dwordx4 %1, %7, %[b] ; ringld\n\t"
+                 "global_load_dwordx4 %2, %8, %[b] ; ringld\n\t"
+                 "global_load_dwordx4 %3, %9, %[b] ; ringld\n\t"
+                 "global_load_dwordx4 %4, %10, %[b] ; ringld\n\t"
+                 "s_mov_b64 exec, %[sv]"
+                 : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]), "+v"(d[4]), [sv] "=&s"(saved)
+                 : "v"(o[0]), "v"(o[1]), "v"(o[2]), "v"(o[3]), "v"(o[4]), [b] "s"(base), [on] "s"(on));
+#endif
+}
+__device__ __forceinline__ void mg_request(g_u32x4 (&d)[3], const uint32_t (&o)[3], const uint8_t* base, uint32_t on)
+{
+#ifdef KQ_TRACKED_LOADS
+    if (on)
+        for (int k = 0; k < 3; ++k) d[k] = *(const g_u32x4*)(base + o[k]);
+#else
+    uint64_t saved;
+    asm volatile("s_mov_b64 %[sv], exec\n\t"
+                 "s_and_b32 exec_lo, exec_lo, %[on]\n\t"
+                 "s_and_b32 exec_hi, exec_hi, %[on]\n\t"
+                 "global_load_dwordx4 %0, %4, %[b] ; ringld\n\t"
+                 "global_load_dwordx4 %1, %5, %[b] ; ringld\n\t"
+                 "global_load_dwordx4 %2, %6, %[b] ; ringld\n\t"
+                 "s_mov_b64 exec, %[sv]"
+                 : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), [sv] "=&s"(saved)
+                 : "v"(o[0]), "v"(o[1]), "v"(o[2]), [b] "s"(base), [on] "s"(on));
 #endif
 }
 
@@ -166,8 +209,8 @@ __global__ __launch_bounds__(64 * WAVES) void q4k_mgemv_kernel(const uint8_t* __
     g_u32x4 raw[MG_DEPTH][NU] = {};
     auto request = [&](uint32_t i, g_u32x4 (&dst)[NU]) {
         const uint8_t* base = W + (size_t)tile_row0(i) * row_stride;
-#pragma unroll
-        for (int k = 0; k < NU; ++k) mg_load16(dst[k], u_src[k], base);
+        // past the last tile: a request of no lanes
+        mg_request(dst, u_src, base, (uint32_t)__builtin_amdgcn_readfirstlane(i < n_i ? -1 : 0));
     };
 #pragma unroll
     for (int d = 0; d < MG_DEPTH; ++d) request((uint32_t)d, raw[d]);
@@ -227,7 +270,7 @@ __global__ __launch_bounds__(64 * WAVES) void q4k_mgemv_kernel(const uint8_t* __
         mg_wait<(MG_DEPTH - 1) * NU>(buf);   // the other buffers' loads stay in flight
 #pragma unroll
         for (int k = 0; k < NU; ++k) *(g_u32x4*)(win + u_dst[k]) = buf[k];
-        request(i + MG_DEPTH, buf);  // (past the last tile: the last tile again, dropped)
+        request(i + MG_DEPTH, buf);
         mg_window_fence();
         float tot = 0.0f;
         const uint8_t* rowp = win + n * PITCH;
@@ -313,7 +356,7 @@ __global__ __launch_bounds__(64 * WAVES) void q4k_mgemv_kernel(const uint8_t* __
         }
     }
 #ifndef KQ_TRACKED_LOADS
-    asm volatile("s_waitcnt vmcnt(0)");   // the last refills land before the wave ends
+    asm volatile("s_waitcnt vmcnt(0)");   // nothing is in flight when the wave ends
 #endif
 }
 

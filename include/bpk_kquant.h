@@ -513,8 +513,9 @@ BPK_API int bpk_force_kernel(int family);
  * through a per-device workspace and are added in the order of the walk, so
  * results repeat bit for bit); "fused_separate": 1 makes bpk_kq_matmul_fused run its prologue,
  * matmul and add as separate launches for every shape (needs the workspace);
- * "mgemv": 0 keeps one-token Q4_K matvecs of many rows on the lanes-along-K
- * kernel (1, the default, takes them to the matrix-core kernel);
+ * "mgemv": which one-token Q4_K matvecs go to the matrix-core kernel instead of
+ * the lanes-along-K kernel: 0 none, 1 (default) matrices of 49152 rows and more,
+ * 2 from 16384 rows on (gate|up: level on most parts, ahead where the clock runs low);
  * "chain_spin_us": bound of a wait between the ops of a chain in microseconds
  * (at most ten seconds);
  * "chain_hold" (test hook, refused unless chain_spin_us is 1..100000): 1 keeps

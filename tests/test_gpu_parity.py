@@ -349,10 +349,11 @@ def test_matrix_core_gemv_shapes(gpu, kqo, N, K, form):
         capi.set_option("gemv_splits", 0)
 
 
-def test_matrix_core_gemv_is_the_choice_for_gate_up(gpu, kqo):
-    """The library's own choice: Q4_K, one token, 16384 rows or more -> the matrix-core kernel; the option switches it off."""
+def test_matrix_core_gemv_by_choice(gpu, kqo):
+    """The library's own choice: Q4_K, one token, 49152 rows or more -> the matrix-core kernel; the option moves the
+    threshold or switches it off."""
     from backpack_amd import capi, kquant
-    N, K = 16384, 512
+    N, K = 49152, 256
     raw, packed, w = gpu.make_weight(Q4_K, N, K, seed=5)
     X = np.random.default_rng(5).standard_normal((1, K)).astype(np.float32)
     got = kquant.matmul(gpu.dev(X), w).cpu().numpy()
@@ -362,6 +363,11 @@ def test_matrix_core_gemv_is_the_choice_for_gate_up(gpu, kqo):
     try:
         got2 = kquant.matmul(gpu.dev(X), w).cpu().numpy()
         assert capi.last_kernel() == "gemv_stream"
+        capi.set_option("mgemv", 2)
+        raw3, packed3, w3 = gpu.make_weight(Q4_K, 16384, 256, seed=6)
+        got3 = kquant.matmul(gpu.dev(X), w3).cpu().numpy()
+        assert capi.last_kernel() == "mgemv"
+        gpu.check_matmul(kqo, Q4_K, got3, X, packed3, 16384, 256, label="mgemv from 16384 rows", slack=2e-5)
     finally:
         capi.set_option("mgemv", 1)
     gpu.check_matmul(kqo, Q4_K, got2, X, packed, N, K, label="stream with the option off")
