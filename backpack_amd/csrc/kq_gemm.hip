@@ -370,24 +370,32 @@ __device__ __forceinline__ void il_scales(const RawQ4& r, uint32_t kc, uint32_t 
     const float dmin = half_bits_to_float(r.h.x >> 16);
     uint32_t sc, mn;
     q4k_scale_min(r.h.y, r.h.z, r.h.w, (int)((kc & 3u) * 2u + hf), sc, mn);
-    // the high nibble is converted in place (16 q), so its scale carries the 1/16
-    s0 = d * (float)sc * (hf ? 0.0625f : 1.0f);
+    // a masked nibble is left where it is and read as an fp16 subnormal, q * 2^-24 (low nibble) or q * 2^-20 (high
+    // nibble): the scale carries the matching power of two (an exact scaling, so fma(q_h, s0, nb) rounds the same
+    // exact value as fma(d * sc, q, nb) does)
+    s0 = d * (float)sc * (hf ? 1048576.0f : 16777216.0f);
     s1 = s0;
     nb = -(dmin * (float)mn);
 }
-// 8 weights (piece v of the thread's run of 32) -> 16 bytes of bf16
+typedef _Float16 gm_half2 __attribute__((ext_vector_type(2)));
+// 8 weights (piece v of the thread's run of 32) -> 16 bytes of bf16.  No integer-to-float conversion: the nibbles
+// enter v_fma_mix_f32 as fp16 subnormals (two masks and a shift per four weights instead of a mask and four
+// conversions).
 __device__ __forceinline__ u32x4 il_expand(const RawQ4& r, uint32_t, uint32_t hf, int v, float s0, float, float nb)
 {
     const u32x4 src = v < 2 ? r.q0 : r.q1;
-    const uint32_t mask = hf ? 0xF0F0F0F0u : 0x0F0F0F0Fu;
+    const uint32_t mask = hf ? 0x00F000F0u : 0x000F000Fu;
     u32x4 out;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const uint32_t w = src[(v & 1) * 2 + j] & mask;
-        const float f0 = fmaf(s0, (float)(w & 255u), nb);
-        const float f1 = fmaf(s0, (float)((w >> 8) & 255u), nb);
-        const float f2 = fmaf(s0, (float)((w >> 16) & 255u), nb);
-        const float f3 = fmaf(s0, (float)(w >> 24), nb);
+        const uint32_t w = src[(v & 1) * 2 + j];
+        const gm_half2 a = __builtin_bit_cast(gm_half2, w & mask);          // bytes 0 and 2
+        const gm_half2 b = __builtin_bit_cast(gm_half2, (w >> 8) & mask);   // bytes 1 and 3
+        const _Float16 a0 = a.x, a1 = a.y, b0 = b.x, b1 = b.y;
+        const float f0 = fmaf((float)a0, s0, nb);
+        const float f1 = fmaf((float)b0, s0, nb);
+        const float f2 = fmaf((float)a1, s0, nb);
+        const float f3 = fmaf((float)b1, s0, nb);
         out[j * 2] = pack_bf16(f0, f1);
         out[j * 2 + 1] = pack_bf16(f2, f3);
     }

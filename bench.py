@@ -32,11 +32,23 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 COPY_RATE_GBS = 6350.0          # what a plain streaming read reaches on this pool's MI355X (6.0-6.7 TB/s measured)
 METRIC = "Q4_K M=1 matvec HBM GB/s (% of peak); M=2048 dequant-GEMM TFLOPS (% MFMA)"
 
-# HBM bytes per launch of the dominant kernel.  NOT measured in this run: copied from the rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE summary named below (FETCH_SIZE x 2.000 KiB + WRITE_SIZE x 1.000 KiB, the factors
-# being what the same counters read for a 256 MiB copy kernel); regenerate that file when the kernel changes.
+# HBM bytes per launch of the dominant kernel are NOT measured in this run: they are read from the committed
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary named below (FETCH_SIZE x 2.000 KiB + WRITE_SIZE x 1.000 KiB, the
+# factors being what the same counters read for a 256 MiB copy kernel), from its line
+# "traffic_bytes <kernel family> <shape> <bytes>"; no such line for the kernel that ran -> null.
 TRAFFIC_PROFILE = "profiles/decode_gemv_hbm_traffic_pmc.txt"
-MEASURED_TRAFFIC_BYTES = 66436321
+
+
+def profiled_traffic(kernel, shape):
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+            for line in f:
+                t = line.split()
+                if len(t) == 4 and t[0] == "traffic_bytes" and t[1] == kernel and t[2] == shape:
+                    return int(t[3])
+    except OSError:
+        pass
+    return None
 
 
 def parse():
@@ -56,7 +68,8 @@ def parse():
                     help="skip the layer set at M = 2, 4, 8, 16 (speculative-decode verify batches)")
     ap.add_argument("--no-moe", action="store_true",
                     help="skip the Qwen3-30B-A3B-shaped routed-expert FFN at T = 1 and T = 256")
-    ap.add_argument("--all", action="store_true", help="also the single-matvec leg (config 0), --fused")
+    ap.add_argument("--all", action="store_true", help="also --fused")
+    ap.add_argument("--no-config0", action="store_true", help="skip the single 4096x4096 matvec (cold / hot)")
     ap.add_argument("--fused", action="store_true",
                     help="also time the layer set with RMSNorm folded into qkv and act*mul + residual into down")
     ap.add_argument("--load", action="store_true",
@@ -247,11 +260,12 @@ def main():
         capi.set_option("gemm_tile", args.gemm_tile)
     if args.gemm_split:
         capi.set_option("gemm_split", args.gemm_split)
+    mats = build_layer_set(args.layers)
     if args.prefill_only:
-        print(json.dumps({"prefill": prefill_leg()}))
+        torch.cuda.synchronize()
+        print(json.dumps({"prefill": prefill_leg(mats, 2048)}))
         return
 
-    mats = build_layer_set(args.layers)
     torch.cuda.synchronize()
     wb, act = algorithmic_bytes(mats)
     use_graph = not args.no_graph
@@ -272,8 +286,11 @@ def main():
     dom_w = dom[0][1]
     dom_bytes = synth.weight_bytes(dom_w.type, dom_w.N, dom_w.K) + (dom_w.K + dom_w.N) * 4
     dom_gbs = dom_bytes / (dsec / launches) / 1e9
+    dom_kernel = capi.last_kernel()     # the library's name of the kernel family that served these launches
+    dom_shape = f"{dom_w.N}x{dom_w.K}"
+    traffic = profiled_traffic(dom_kernel, dom_shape)
     roofline = {
-        "kernel": f"kq::q4k_stream_dense_kernel<2, 8, 2, 1, false, 1> ({capi.last_kernel()}; gate|up 28672x4096 Q4_K, M=1)",
+        "kernel": f"{dom_kernel} (gate|up {dom_shape} Q4_K, M=1; instantiation: see profiles/decode_layer_set_kernel_trace.txt)",
         "bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
         "bytes_per_launch": dom_bytes, "us_per_launch": round(dsec / launches * 1e6, 3),
@@ -281,8 +298,8 @@ def main():
         "us_per_launch_min": round(dom_pass[0] / len(dom) * 1e6, 3),
         "us_per_launch_median": round(dom_pass[len(dom_pass) // 2] / len(dom) * 1e6, 3),
         "launches_timed": launches,
-        "traffic": MEASURED_TRAFFIC_BYTES,
-        "traffic_source": f"not measured in this run: rocprofv3 --pmc summary {TRAFFIC_PROFILE}",
+        "traffic": traffic,
+        "traffic_source": f"not measured in this run: rocprofv3 --pmc summary {TRAFFIC_PROFILE}, line for {dom_kernel} {dom_shape}",
         "frac_of_measured_copy_rate": round(dom_gbs / COPY_RATE_GBS, 4),
     }
 
@@ -316,7 +333,7 @@ def main():
         "roofline": roofline,
         "per_shape": shapes,
     }
-    if args.all:
+    if not args.no_config0:
         out["config0"] = config0_leg()
     if not args.no_verify:
         out["verify"] = verify_leg(mats, wb, use_graph)
@@ -328,10 +345,11 @@ def main():
         out["gguf_load"] = load_leg()
     if not args.no_prefill:
         # the second half of the metric: M=2048 dequant-GEMM TFLOP/s and its fraction of the bf16 MFMA peak
-        out["prefill"] = prefill_leg()
-        out["prefill_m512"] = prefill_leg(512)
+        out["prefill"] = prefill_leg(mats, 2048)
+        out["prefill_m512"] = prefill_leg(mats, 512)
         out["gemm_tflops_m2048"] = out["prefill"]["layer_set"]["TFLOPs"]
         out["gemm_pct_of_mfma_peak"] = out["prefill"]["layer_set"]["pct_of_bf16_mfma_peak"]
+        out["gemm_accuracy"] = out["prefill"]["accuracy"]
     if not args.no_cpu:
         del mats, dom
         torch.cuda.empty_cache()
@@ -630,41 +648,79 @@ def moe_leg():
     return res
 
 
-def prefill_leg(M=2048):
-    """M=2048 bf16 dequant-GEMM over one layer's four matrices + lm_head."""
+def prefill_leg(mats, M=2048):
+    """The bf16 dequant-GEMM over the layer set at M tokens: ONE PASS = every one of the set's distinct matrices
+    (32 layers x [qkv, o, gate_up, down] + lm_head, the weights the decode leg holds) multiplied once, in layer
+    order, on one stream; timed over whole passes.  Per-shape figures come from passes over one shape's 32
+    matrices.  `accuracy`: the output of one gate|up launch against fp64 contractions of (a) the exactly
+    dequantised weights (bpk_kq_dequant_rows, bit-identical to the reference's dequant) and (b) those weights
+    rounded to bf16, on sampled rows, computed with torch on the GPU."""
     import torch
-    from backpack_amd import kquant, synth
-    spec = synth.LLAMA3_8B
+    from backpack_amd import kquant
+    xs, ys = {}, {}
+    for _, w, _, _ in mats:
+        if w.K not in xs:
+            xs[w.K] = torch.randn(M, w.K, device="cuda", generator=torch.Generator(device="cuda").manual_seed(w.K)).to(torch.bfloat16)
+        if w.N not in ys:
+            ys[w.N] = torch.empty(M, w.N, device="cuda")
+
+    def run(sel, passes, warm):
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            for _ in range(warm):
+                for _, w, _, _ in sel:
+                    kquant.matmul(xs[w.K], w, out=ys[w.N])
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(passes):
+                for _, w, _, _ in sel:
+                    kquant.matmul(xs[w.K], w, out=ys[w.N])
+            e1.record(stream)
+            stream.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / passes
+
     res = {}
-    flops_total, sec_total = 0.0, 0.0
-    for name, type_, N, K in list(spec["layer"]) + [spec["lm_head"]]:
-        data = synth.make_packed_device(type_, N, K, seed=77)
-        w = kquant.KQuantPacked(data, type_, N, K, synth.row_stride_words(type_, K), synth.n_blocks(K))
-        x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
-        y = torch.empty(M, N, device="cuda")
-        for _ in range(2):
-            kquant.matmul(x, w, out=y)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        reps = 20
-        e0.record()
-        for _ in range(reps):
-            kquant.matmul(x, w, out=y)
-        e1.record()
-        torch.cuda.synchronize()
-        s = e0.elapsed_time(e1) * 1e-3 / reps
-        fl = 2.0 * M * N * K
-        res[name] = {"ms": round(s * 1e3, 3), "TFLOPs": round(fl / s / 1e12, 1)}
-        weight = 32 if name != "lm_head" else 1
-        flops_total += fl * weight
-        sec_total += s * weight
-        del data, w, x, y
-    tf = flops_total / sec_total / 1e12
+    for name in ("qkv", "o", "gate_up", "down", "lm_head"):
+        sel = [m for m in mats if m[0] == name]
+        s = run(sel, 2 if name != "lm_head" else 6, 1) / len(sel)
+        w = sel[0][1]
+        res[name] = {"ms": round(s * 1e3, 3), "TFLOPs": round(2.0 * M * w.N * w.K / s / 1e12, 1)}
+    passes = 3
+    sec = run(mats, passes, 1)
+    flops = sum(2.0 * M * w.N * w.K for _, w, _, _ in mats)
+    tf = flops / sec / 1e12
     res["layer_set"] = {"TFLOPs": round(tf, 1), "pct_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS * 100, 2),
-                        "M": M, "ms_extrapolated": round(sec_total * 1e3, 2),
-                        "how": "one layer's four matrices x 32 + lm_head, extrapolated: each matrix timed as 20 launches "
-                               "back to back on the same weights (cache-warm; the kernel is bound by the matrix cores)"}
+                        "M": M, "ms_per_pass": round(sec * 1e3, 2), "launches_per_pass": len(mats), "passes_timed": passes,
+                        "how": f"full pass: each of the set's {len(mats)} distinct matrices once per pass, in layer order, "
+                               f"{passes} passes timed after one of warm-up"}
+    if M == 2048:
+        res["accuracy"] = gemm_accuracy(next(m for m in mats if m[0] == "gate_up")[1], xs, ys, M)
     return res
+
+
+def gemm_accuracy(w, xs, ys, M):
+    """Largest error of one bf16 GEMM launch on sampled weight rows, relative to the rms and to the largest |y| of
+    the sample: against the exact weights (the error the bf16 rounding of W brings: unit roundoff 2^-9 per weight)
+    and against the bf16-rounded weights (what the kernel itself adds: accumulation order only)."""
+    import torch
+    from backpack_amd import kquant
+    x, y = xs[w.K], ys[w.N]
+    kquant.matmul(x, w, out=y)
+    rows = torch.randperm(w.N, device="cuda", generator=torch.Generator(device="cuda").manual_seed(3))[:256].to(torch.int32)
+    deq = kquant.dequant_rows(w, rows)                    # fp32 [256, K], bit-exact weights
+    got = y[:, rows.long()].double()
+    x64 = x.double()
+    exact = x64 @ deq.double().T
+    rounded = x64 @ deq.to(torch.bfloat16).double().T
+    rms, peak = float(exact.pow(2).mean().sqrt()), float(exact.abs().max())
+    e1, e2 = float((got - exact).abs().max()), float((got - rounded).abs().max())
+    return {"matrix": f"gate_up {w.N}x{w.K}, M={M}, 256 sampled weight rows",
+            "max_err_over_rms": round(e1 / rms, 5), "max_err_over_peak": round(e1 / peak, 6),
+            "frobenius_rel": round(float((got - exact).pow(2).sum().sqrt() / exact.pow(2).sum().sqrt()), 6),
+            "vs_bf16_rounded_weights_over_peak": float(f"{e2 / peak:.3g}"),
+            "note": "errors against the exact weights are the bf16 rounding of W that the workload prescribes "
+                    "(tolerance 1e-2 of the largest |y|); against the rounded weights only the summation order is left"}
 
 
 if __name__ == "__main__":
