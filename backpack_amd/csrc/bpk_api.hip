@@ -451,7 +451,7 @@ static int matmul_impl(int type, const float* X, const void* W, const float* bia
     // parts as token slots) beats two tokens on the vector units there (28672x4096: 19.6 against 22.7 us; 6144x4096:
     // 11.1 against 8.5, so smaller matrices stay)
     const bool tile_two = M == 2 && type != BPK_TYPE_Q6_K && weights >= (64ull << 20);
-    if (t_family == 6 || (t_family == 0 && mtile_ok && ((M >= 3 && M <= 255 && !stream_four) || tile_two))) {
+    if (t_family == 6 || (t_family == 0 && mtile_ok && ((M >= 3 && !stream_four) || tile_two))) {
         t_kernel = "mtile";
         e = kq::launch_mtile(a, st->split, s);
         return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);

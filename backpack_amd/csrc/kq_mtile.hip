@@ -1131,8 +1131,9 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1)
 bool mtile_supported(const MatmulArgs& a)
 {
     // dense calls of more than 16 tokens run as groups of 16 (8 for Q6_K), each reading the weights again:
-    // meant for the few dozen tokens between a verify batch and a prefill, not for prefill itself
-    if (!a.expert_idx && (a.M < 1 || a.M > 255)) return false;   // grouped calls bring their tokens in records
+    // meant for the few dozen tokens between a verify batch and a prefill, not for prefill itself (whose entry
+    // point is the bf16 GEMM); any fp32 token count is served this way rather than by the generic kernel
+    if (!a.expert_idx && (a.M < 1 || a.M > 65536u)) return false;   // grouped calls bring their tokens in records
     if (((uintptr_t)a.X & 15u)) return false;
     if (a.type == KQ_TYPE_Q4_K || a.type == KQ_TYPE_Q5_K) return !(((uintptr_t)a.W & 15u) || (a.row_stride_bytes & 15u));
     if (a.type == KQ_TYPE_Q6_K) return !(((uintptr_t)a.W & 1u) || (a.row_stride_bytes & 1u));

@@ -226,7 +226,10 @@ BPK_API int bpk_gguf_weight_create(const bpk_gguf *g, const char *const *names,
  * aligned rows take the fast kernels).  Q6_K blocks are 210 bytes and are
  * fetched in 16-byte pieces: the buffer must stay readable for 16 bytes past
  * the end of the last row (bpk_weight_create allocates them).  bias: f32 [N] or NULL (= zeros).
- * Y: f32, caller-owned, not cleared.  fp32 accumulation throughout. */
+ * Y: f32, caller-owned, not cleared.  fp32 accumulation throughout.  Up to 16
+ * tokens (8 on Q6_K matrices) every weight byte is read once per call; more
+ * tokens run in groups of that size, each reading the weights again (prefill
+ * chunks belong on bpk_prefill_rows_bf16 + bpk_kq_matmul_bf16). */
 BPK_API int bpk_kq_matmul(int type, const float *X, const void *W,
                           const float *bias, float *Y, uint32_t M, uint32_t N,
                           uint32_t K, uint32_t n_blocks,

@@ -166,8 +166,11 @@ def test_chain_in_place_equals_separate_calls(gpu, kqo):
     h0 = gpu.dev(host["h0"])
 
     def close(a, b):
+        # the bound of the C++ host layer's chain test (tests/cpp/kernel_test.cpp, chain_of_a_decoder_layer_tail:
+        # separate fused dispatches against the chain, atol = rtol = 1e-4 per element), and 2e-5 of the largest element
         scale = float(b.abs().max())
-        return float((a - b).abs().max()) <= 2e-5 * scale
+        elementwise = bool(((a - b).abs() <= 1e-4 + 1e-4 * b.abs()).all())
+        return elementwise and float((a - b).abs().max()) <= 2e-5 * scale
     ch.run()
     torch.cuda.synchronize()
     ch.status()

@@ -184,6 +184,9 @@ SHAPES = [
     (Q6_K, 13, 1800, 1536),     # Q6_K beyond 8 tokens: two groups; 6 blocks
     (Q4_K, 37, 300, 1024),      # fp32 X beyond 16 tokens: groups of 16 (Q4_K) / 8 (Q6_K) on the tile kernel
     (Q6_K, 21, 200, 1024),
+    (Q4_K, 64, 1024, 4096),     # ... a prefill-sized chunk through the fp32 entry point: four groups
+    (Q4_K, 128, 512, 4096),
+    (Q6_K, 300, 96, 1024),      # ... beyond 255 tokens (the tile kernel, not the generic one)
     (Q4_K, 16, 22500, 512),     # tile kernel, a wave per tile (7 or 8 tiles per workgroup), ragged last tile
     (Q6_K, 5, 23001, 768),
     (Q4_K, 16, 6144, 4096),     # tile kernel with K cut over workgroups (4 runs of one chunk), partials folded by the last
@@ -347,6 +350,18 @@ def test_matrix_core_gemv_shapes(gpu, kqo, N, K, form):
     finally:
         capi.force_kernel(0)
         capi.set_option("gemv_splits", 0)
+
+
+def test_fp32_chunks_of_any_size_stay_off_the_generic_kernel(gpu, kqo):
+    """fp32 X with more than 255 tokens: the tile kernel in groups of 16 tokens, as for 17 .. 255 (the generic
+    kernel, one wave per output row, is the fallback for shapes no other kernel takes, not for token counts)."""
+    from backpack_amd import capi, kquant
+    M, N, K = 260, 128, 512
+    raw, packed, w = gpu.make_weight(Q4_K, N, K, seed=9)
+    X = np.random.default_rng(9).standard_normal((M, K)).astype(np.float32)
+    got = kquant.matmul(gpu.dev(X), w).cpu().numpy()
+    assert capi.last_kernel() == "mtile"
+    gpu.check_matmul(kqo, Q4_K, got, X, packed, N, K, label="mtile 260 tokens", slack=2e-5)
 
 
 def test_matrix_core_gemv_by_choice(gpu, kqo):
