@@ -167,9 +167,11 @@ def test_chain_in_place_equals_separate_calls(gpu, kqo):
 
     def close(a, b):
         # the bound of the C++ host layer's chain test (tests/cpp/kernel_test.cpp, chain_of_a_decoder_layer_tail:
-        # separate fused dispatches against the chain, atol = rtol = 1e-4 per element), and 2e-5 of the largest element
+        # separate fused dispatches against the chain, atol = rtol = 1e-4 per element on outputs of unit scale; here
+        # the outputs are not of unit scale, so the absolute part is 1e-4 of their rms), and 2e-5 of the largest element
         scale = float(b.abs().max())
-        elementwise = bool(((a - b).abs() <= 1e-4 + 1e-4 * b.abs()).all())
+        rms = float(b.double().pow(2).mean().sqrt())
+        elementwise = bool(((a - b).abs() <= 1e-4 * rms + 1e-4 * b.abs()).all())
         return elementwise and float((a - b).abs().max()) <= 2e-5 * scale
     ch.run()
     torch.cuda.synchronize()

@@ -119,7 +119,7 @@ def test_four_token_stream_kernels(gpu, kqo, type_, M, N, K):
                                           (1, 4096, 4096, "gemv_stream"), (2, 6144, 4096, "gemv_stream"),
                                           (1, 77, 256, "gemv_stream"), (1, 500, 3072, "gemv_stream"),
                                           (5, 130, 2048, "mtile"), (17, 40, 512, "mtile"), (4, 64, 768, "gemv_stream"),
-                                          (13, 700, 4096, "mtile"), (70, 40, 512, "mtile"), (300, 40, 512, "generic"),
+                                          (13, 700, 4096, "mtile"), (70, 40, 512, "mtile"), (300, 40, 512, "mtile"),
                                           (1, 1000, 14336, "gemv_stream"), (2, 300, 8192, "gemv_stream"),
                                           (1, 200, 28672, "gemv_stream"), (2, 200, 28672, "generic"),
                                           (1, 50, 32768, "generic")])
@@ -131,7 +131,7 @@ def test_q5k_matmul_vs_oracle(gpu, kqo, M, N, K, kernel):
     bias = np.random.default_rng(1).standard_normal(N).astype(np.float32)
     y = kquant.matmul(gpu.dev(X), w, bias=gpu.dev(bias)).cpu().numpy()
     assert capi.last_kernel() == kernel
-    gpu.check_matmul(kqo, Q5_K, y, X, packed, N, K, bias=bias, label=f"q5k {M}x{N}x{K}")
+    gpu.check_matmul(kqo, Q5_K, y, X, packed, N, K, bias=bias, label=f"q5k {M}x{N}x{K}", slack=2e-5 if kernel == "mtile" else 1e-6)
     if kernel != "generic":      # and the generic kernel on the same inputs
         capi.force_kernel(1)
         try:
