@@ -31,6 +31,7 @@ thread_local int t_family = 0;
 thread_local kq::GemvTuning t_gemv;
 thread_local int t_gemm_tile = 0;
 thread_local int t_gemm_split = 0;
+thread_local bool t_moe_fold = true;    // option "moe_fold": the slots' weighted sum inside the last matvec where its kernel can
 thread_local int t_fused_separate = 0;
 thread_local int t_chain_spin_us = 0;    // 0 = default
 thread_local int t_chain_ahead = 0;      // 1 + rows touched ahead; 0 = default
@@ -228,6 +229,10 @@ int bpk_set_option(const char* name, int value)
     }
     if (!strcmp(name, "chain_hold")) {
         t_chain_hold = value != 0;
+        return BPK_OK;
+    }
+    if (!strcmp(name, "moe_fold")) {
+        t_moe_fold = value != 0;
         return BPK_OK;
     }
     if (!strcmp(name, "gemm_split")) {
@@ -1095,6 +1100,11 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
         a.W2 = (const uint8_t*)up; a.Y2 = U;
         e = kq::launch_gemv_stream(a, t_gemv, s);
         d.X2 = U;
+        if (e == hipSuccess && t_moe_fold && kq::stream_combine_supported(d, T)) {
+            // ... and the weighted sum over the slots into down's launch: its waves are a token's slots
+            e = kq::launch_stream_combine(d, expert_wt, out, T, t_gemv, s);
+            return e == hipSuccess ? BPK_OK : hip_fail(e, t_kernel);
+        }
         if (e == hipSuccess) e = kq::launch_gemv_stream(d, t_gemv, s);
     } else if (tile_path) {
         // two or more pairs per expert on average: records of 8 pairs (16 from four pairs per expert on),

@@ -113,6 +113,11 @@ hipError_t launch_gemv_rows(const MatmulArgs& a, const SplitScratch& sc, const G
 // in registers.  t.splits, when set, overrides the rows per wave.
 bool gemv_stream_supported(const MatmulArgs& a);
 hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStream_t s);
+// The grouped call `a` (Q6_K, up to 8 slots per token) with the weighted sum over each token's slots folded into
+// the launch: out[token, r] = sum over slots, in slot order, of wt[pair] * (W[expert_idx[pair]] x[pair])[r].
+bool stream_combine_supported(const MatmulArgs& a, uint32_t tokens);
+hipError_t launch_stream_combine(const MatmulArgs& a, const float* wt, float* out, uint32_t tokens, const GemvTuning& t,
+                                 hipStream_t s);
 
 // One token on the matrix cores: Q4_K rows of up to 16 superblocks, 16-byte aligned (kq_mgemv.hip).
 bool mgemv_supported(const MatmulArgs& a);

@@ -39,7 +39,7 @@ struct StreamDense {          // 64 bytes = the 16 dwords that kernel-argument p
     uint32_t N, K, n_blocks, row_stride_bytes, y_offset, ldy;
     uint32_t M;   // tokens; read only by the four-token kernels (three tokens run as four, the last one masked)
     uint32_t grid_x;   // workgroups of the launch along x (as an argument: the hidden one would be a fetch of its own)
-    static constexpr bool kGrouped = false, kFused = false;
+    static constexpr bool kGrouped = false, kFused = false, kCombine = false;
 };
 
 // Dense matvec with a prologue on the activations (STREAM_PRO_*; for the act forms the X rows are
@@ -59,7 +59,7 @@ struct StreamFused {
     // Y[n] = act(gate_n . x) * (up_n . x): a wave takes both rows of a pair, one after the other
     int epi;
     uint32_t grid_x;   // workgroups of the launch along x
-    static constexpr bool kGrouped = false, kFused = true;
+    static constexpr bool kGrouped = false, kFused = true, kCombine = false;
 };
 
 // Expert indirection: blockIdx.y is a (token, slot) pair that uses weight rows expert_idx[pair]*N ..
@@ -79,7 +79,16 @@ struct StreamGrouped {
     const uint8_t* W2;
     float* Y2;
     const float* X2;
-    static constexpr bool kGrouped = true, kFused = false;
+    static constexpr bool kGrouped = true, kFused = false, kCombine = false;
+};
+
+// The last matvec of an expert FFN with the weighted sum over a token's slots folded in (Q6_K kernel): blockIdx.y
+// is a token, wave w of the workgroup serves the token's slot w (pair token * k_slots + w) over the same rows as
+// the other waves, and where the K slices of a long row would meet, the slots' results meet instead:
+// Y[token, r] = sum over slots, in slot order, of wt[pair] * (W[expert_idx[pair]] x[pair])[r].
+struct StreamCombine : StreamGrouped {
+    const float* wt;
+    static constexpr bool kCombine = true;
 };
 
 
@@ -94,6 +103,20 @@ __device__ __forceinline__ void stream_select_pair(StreamGrouped& p)
     if (p.X2) p.X2 += xrow;
     p.Y += (size_t)pair * p.ldy;
 }
+// The pair of wave `wave` in a slot-combining launch; returns the pair's weight.  Waves beyond the token's
+// slots repeat the last slot and are left out of the sum.
+__device__ __forceinline__ float stream_select_slot(StreamCombine& p, uint32_t wave)
+{
+    const uint32_t tok = blockIdx.y;
+    const uint32_t pair = tok * p.k_slots + min(wave, p.k_slots - 1u);
+    p.W += (size_t)p.expert_idx[pair] * p.N * p.row_stride_bytes;
+    const size_t xrow = (size_t)(p.x_per_slot ? pair : tok) * p.K;
+    p.X += xrow;
+    if (p.X2) p.X2 += xrow;
+    p.Y += (size_t)tok * p.ldy;
+    return p.wt[pair];
+}
+template <typename PT> __device__ __forceinline__ float stream_select_slot(PT&, uint32_t) { return 1.0f; }
 __device__ __forceinline__ void stream_select_pair(StreamDense&) {}
 __device__ __forceinline__ void stream_touch_late_args(const StreamFused& p)
 {
@@ -509,10 +532,15 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
 template <int P, int KW, int D, int MT, typename PT>
 __device__ __forceinline__ void q6k_stream_body(PT p)
 {
-    stream_select_pair(p);
+    constexpr bool COMBINE = PT::kCombine;   // the waves are a token's slots, not K slices
     __shared__ float part[KW > 1 ? KW : 1][MT][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t slots = COMBINE ? min(p.M, (uint32_t)KW) : (uint32_t)KW;   // (a combining launch passes its slots per token in M)
+    float slot_wt = 1.0f;
+    if constexpr (COMBINE) slot_wt = stream_select_slot(p, wave);
+    else stream_select_pair(p);
+    const uint32_t kslice = COMBINE ? 0u : wave;
     const uint32_t g = blockIdx.x, stride = stream_grid_x(p);
     const uint32_t n_rows = g < p.N ? (p.N - g + stride - 1u) / stride : 0u;
     const uint32_t bl = lane >> 3, t = lane & 7u, n = t >> 2, lg = t & 3u;
@@ -532,7 +560,7 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
         for (int tk = 0; tk < MT; ++tk) ssq[tk] = 0.0f;
 #pragma unroll
         for (int pass = 0; pass < P; ++pass) {
-            uint32_t b = (wave * P + pass) * 8u + bl;
+            uint32_t b = (kslice * P + pass) * 8u + bl;
             const bool valid = b < p.n_blocks;
             const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;   // activations of superblocks beyond K read as zero
             b = valid ? b : p.n_blocks - 1u;
@@ -631,7 +659,7 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
         }
         if (KW > 1) {
 #pragma unroll
-            for (int tk = 0; tk < MT; ++tk) part[wave][tk][lane] = res[tk];
+            for (int tk = 0; tk < MT; ++tk) part[wave][tk][lane] = COMBINE ? slot_wt * res[tk] : res[tk];
             __syncthreads();
         }
         if (wave == 0 && lane < cnt) {
@@ -643,9 +671,10 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
                 if (KW > 1) {
                     y = part[0][tk][lane];
 #pragma unroll
-                    for (int w = 1; w < KW; ++w) y += part[w][tk][lane];
+                    for (int w = 1; w < KW; ++w)
+                        if (!COMBINE || (uint32_t)w < slots) y += part[w][tk][lane];
                 }
-                if (MT > 2 && (uint32_t)tk >= p.M) continue;
+                if (!COMBINE && MT > 2 && (uint32_t)tk >= p.M) continue;
                 const size_t at = (size_t)tk * p.ldy + p.y_offset + r;
                 if constexpr (PT::kFused) y *= tk == 0 ? rstd0 : rstd1;
                 y += bias;
@@ -969,6 +998,40 @@ static void stream_fill_common(PT& p, const MatmulArgs& a)
     p.y_offset = a.y_offset;
     p.ldy = a.ldy;
     p.M = a.M;
+}
+
+bool stream_combine_supported(const MatmulArgs& a, uint32_t tokens)
+{
+    return a.type == KQ_TYPE_Q6_K && a.expert_idx && a.k_slots >= 1u && a.k_slots <= 8u && a.n_blocks <= 16u && tokens >= 1u &&
+           tokens <= 65535u && a.M == tokens * a.k_slots && gemv_stream_supported(a) && !a.W2 && !a.bias;
+}
+
+// a = the grouped call of the last matvec (pairs, X per pair); out[token, r] = sum over slots of wt * result
+hipError_t launch_stream_combine(const MatmulArgs& a, const float* wt, float* out, uint32_t tokens, const GemvTuning& t,
+                                 hipStream_t s)
+{
+    StreamCombine p;
+    stream_fill_common(p, a);
+    p.expert_idx = a.expert_idx;
+    p.k_slots = a.k_slots;
+    p.x_per_slot = a.x_per_slot;
+    p.W2 = nullptr;
+    p.Y2 = nullptr;
+    p.X2 = a.X2;
+    p.wt = wt;
+    p.Y = out;
+    p.M = a.k_slots;
+    // as many waves as the grouped launch would start: the workgroups of one token share the machine with the
+    // other tokens', twice over.  (Measured on a 128-expert layer, 8 slots, 2048 x 768, one token: 18.5-19.0 us for
+    // the layer against 18.9-19.5 with the sum as a launch of its own; four rows in flight, or fewer rows per
+    // workgroup, are slower.)
+    uint32_t wgs = stream_workgroups(a.N, 1u, t.splits);
+    wgs = (wgs + tokens - 1u) / tokens;
+    if (t.splits == 0) wgs *= 2u;
+    const dim3 grid(wgs, tokens, 1);
+    if (a.n_blocks <= 8u) launch_q6k_entry<1, 8, 2, 1>(grid, dim3(512), s, p);
+    else launch_q6k_entry<2, 8, 2, 1>(grid, dim3(512), s, p);
+    return hipGetLastError();
 }
 
 hipError_t launch_gemv_stream(const MatmulArgs& a, const GemvTuning& t, hipStream_t s)

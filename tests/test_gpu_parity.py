@@ -707,6 +707,34 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo, tgu, tdn):
             assert np.all(np.abs(rowk - ref) <= 1e-3 * rms + 1e-3 * np.abs(ref))
 
 
+@pytest.mark.parametrize("T,E,k,H,I", [(1, 16, 8, 512, 768), (3, 8, 2, 512, 256), (5, 64, 7, 768, 2304), (2, 16, 9, 512, 512)])
+def test_moe_ffn_slot_sum_inside_the_last_matvec(gpu, kqo, T, E, k, H, I):
+    """A few pairs with a Q6_K down projection: the weighted sum over a token's slots rides in down's launch
+    (up to 8 slots; option moe_fold 0 keeps it a launch of its own).  Both against the oracle and each other."""
+    from backpack_amd import capi, kquant
+    _say("moe slot sum", T, E, k, H, I)
+    _, gp, gw = gpu.make_weight(Q4_K, E * I, H, seed=61)
+    _, up, uw = gpu.make_weight(Q4_K, E * I, H, seed=62)
+    _, dp, dw = gpu.make_weight(Q6_K, E * H, I, seed=63)
+    rng = np.random.default_rng(T * 7 + k)
+    eidx, ew = _routing(rng, T, E, k)
+    X = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
+    got = {}
+    try:
+        for fold in (1, 0):
+            capi.set_option("moe_fold", fold)
+            got[fold] = kquant.moe_ffn(gpu.dev(X), gw, uw, dw, gpu.dev(eidx.view(np.int32)), gpu.dev(ew), E).cpu().numpy()
+            assert capi.last_kernel() == "moe_ffn_stream"
+    finally:
+        capi.set_option("moe_fold", 1)
+    want = kqo.moe_ffn(Q4_K, Q6_K, X, gp, up, dp, eidx, ew, H, I)
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    for fold in (1, 0):
+        assert np.all(np.abs(got[fold] - want) <= 1e-3 * rms + 1e-3 * np.abs(want)), fold
+    # the same products summed in the same slot order: only the rounding of wt * y may differ
+    assert np.abs(got[1] - got[0]).max() <= 1e-5 * rms
+
+
 @pytest.mark.parametrize("family,kernel", [(0, "mtile_grouped"), (3, "mrow_grouped")])
 @pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True),
                                                  # K of one chunk: waves walk several tiles per staged X; ragged last tile
