@@ -60,7 +60,7 @@ def check_compiler() -> None:
         raise RuntimeError(msg)
 
 
-_REG = re.compile(r"v\[(\d+):(\d+)\]|v(\d+)")
+_REG = re.compile(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b")
 
 
 def _regs(text: str) -> set[int]:
@@ -99,6 +99,49 @@ def check_ring_registers(asm_path: str) -> list[str]:
             elif "; ringwait" in line:
                 waits |= _regs(line.split("; ringwait", 1)[1])
     close()
+    return problems
+
+
+# A source that carries this marker keeps its hand-waited loads in straight-line code: every kernel's listing, read top
+# to bottom, is the order of execution as far as the ring is concerned (loads ahead of the loop, then wait, use and
+# refill of one slot after another in the loop's body).  Its generated code also passes check_ring_order.
+STRAIGHT_LINE_MARKER = "KQ_RING_STRAIGHT_LINE"
+
+
+def check_ring_order(asm_path: str) -> list[str]:
+    """Reads every function top to bottom with the set of registers that have a marked load in flight: a marked
+    wait may only name registers of that set (and takes them out), a marked load may not write a register still
+    in it, and no other instruction may mention one (a copy, a spill, a reuse as a temporary).  Stricter than
+    check_ring_registers, which compares sets per function; only meaningful for listings whose text order is
+    the order of execution."""
+    problems = []
+    func, flying, n = None, set(), 0
+    with open(asm_path) as f:
+        for line in f:
+            n += 1
+            m = re.match(r"^([A-Za-z_][\w.$]*):\s*(;.*)?$", line)
+            if m and not m.group(1).startswith(".L"):
+                func, flying = m.group(1), set()
+                continue
+            if not line.startswith("\t") or line.lstrip().startswith((".", ";")):
+                continue
+            code = line.split(";", 1)[0]
+            if "; ringld" in line:
+                parts = code.split(",")
+                dest = _regs(parts[0].split(None, 1)[1] if len(parts[0].split(None, 1)) > 1 else "")
+                if dest & flying:
+                    problems.append(f"{func}, line {n}: v{sorted(dest & flying)} loaded again before its wait")
+                addr = _regs(",".join(parts[1:]))
+                if addr & flying:
+                    problems.append(f"{func}, line {n}: a load's address uses v{sorted(addr & flying)}, which is in flight")
+                flying |= dest
+            elif "; ringwait" in line:
+                named = _regs(line.split("; ringwait", 1)[1])
+                if named - flying:
+                    problems.append(f"{func}, line {n}: a wait names v{sorted(named - flying)}, which no load in flight writes")
+                flying -= named
+            elif _regs(code) & flying:
+                problems.append(f"{func}, line {n}: '{code.strip()[:60]}' touches v{sorted(_regs(code) & flying)} with a load in flight")
     return problems
 
 
@@ -144,6 +187,8 @@ def _compile(src: str) -> str:
         if ra.returncode:
             raise RuntimeError(f"hipcc -S failed on {src}:\n{ra.stderr}")
         problems = check_ring_registers(asm)
+        if STRAIGHT_LINE_MARKER in text:
+            problems += check_ring_order(asm)
         if problems:
             raise RuntimeError(f"{src}: registers of hand-waited loads were moved between load and wait:\n" +
                                "\n".join(problems[:8]))

@@ -25,7 +25,9 @@
 // (the compiler's own placement drains the whole queue at every refill inside a loop), under the rules written
 // out in kq_stream_core.h: KQ_REQUIRES_NO_SPILL, every register a load fills passes through the wait that
 // names it, the number of loads in flight is the same at every wait (past its last tile a wave issues its
-// requests with no lane active).
+// requests with no lane active).  The ring lives in straight-line code here (KQ_RING_STRAIGHT_LINE), so the
+// build also reads the listing top to bottom and refuses any instruction that mentions a register between its
+// load and its wait.
 //
 // Results differ from the lanes-along-K kernel's by the hi + lo split of x: 22 bits relative to the largest
 // |x| of a superblock.

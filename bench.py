@@ -696,7 +696,31 @@ def prefill_leg(mats, M=2048):
                                f"{passes} passes timed after one of warm-up"}
     if M == 2048:
         res["accuracy"] = gemm_accuracy(next(m for m in mats if m[0] == "gate_up")[1], xs, ys, M)
+        res["vendor_bf16_gemm"] = vendor_gemm({n: next(m for m in mats if m[0] == n)[1] for n in ("gate_up", "down")}, xs, M)
     return res
+
+
+def vendor_gemm(shapes, xs, M):
+    """For scale only: the vendor library's plain bf16 GEMM (torch.matmul) on the same shapes, with the weights
+    already expanded to bf16 in HBM and a bf16 output, ten launches back to back."""
+    import torch
+    out = {"what": "torch.matmul, bf16 weights resident in HBM (3.5x the packed bytes), bf16 output; not part of the product"}
+    for name, w in shapes.items():
+        wb = torch.randn(w.N, w.K, device="cuda").to(torch.bfloat16)
+        yb = torch.empty(M, w.N, device="cuda", dtype=torch.bfloat16)
+        for _ in range(3):
+            torch.matmul(xs[w.K], wb.t(), out=yb)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            torch.matmul(xs[w.K], wb.t(), out=yb)
+        e1.record()
+        torch.cuda.synchronize()
+        sec = e0.elapsed_time(e1) * 1e-3 / 10
+        out[name] = {"ms": round(sec * 1e3, 3), "TFLOPs": round(2.0 * M * w.N * w.K / sec / 1e12, 1)}
+        del wb, yb
+    return out
 
 
 def gemm_accuracy(w, xs, ys, M):
