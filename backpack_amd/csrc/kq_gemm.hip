@@ -671,6 +671,158 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
     }
 }
 
+// The thread's 16 quant bytes of a k step when four threads share a weight row (quarter = 2 * hf + wq: the
+// sub-block pair's half hf, the first or second 16 of its 32 bytes): they go where the loaders above put the
+// FIRST 16 bytes, so that il_expand serves pieces 0 and 1 of them.
+__device__ __forceinline__ void il1_load_q(const uint8_t* row, uint32_t kc, uint32_t, uint32_t wq, RawQ4& r, bool = true)
+{
+    const u32x4* q = (const u32x4*)(row + (size_t)(kc >> 2) * KQ_Q4K_BYTES + 16 + (kc & 3u) * 32u);
+    r.q0 = q[wq];
+}
+__device__ __forceinline__ void il1_load_q(const uint8_t* row, uint32_t kc, uint32_t, uint32_t wq, RawQ5& r, bool extra = true)
+{
+    const uint8_t* blk = row + (size_t)(kc >> 2) * KQ_Q5K_BYTES;
+    r.q0 = ((const u32x4*)(blk + 48 + (kc & 3u) * 32u))[wq];
+    if (extra) r.b0 = ((const u32x4*)(blk + 16))[wq];
+}
+__device__ __forceinline__ void il1_load_q(const uint8_t* row, uint32_t kc, uint32_t hf, uint32_t wq, RawQ6& r, bool = true)
+{
+    const uint32_t c = kc & 3u, h = c >> 1, t = (c & 1u) * 2u + hf;
+    const uint8_t* blk = row + (size_t)(kc >> 2) * KQ_Q6K_BYTES;
+    __builtin_memcpy(&r.a0, blk + 64u * h + 32u * (t & 1u) + 16u * wq, 16);
+    __builtin_memcpy(&r.b0, blk + 128u + 32u * h + 16u * wq, 16);
+}
+
+// 256 tokens x 128 weight rows per workgroup, whole tiles, one per workgroup: for matrices of few rows at many
+// tokens (N = 4096 at M = 2048 is 256 such tiles, one per CU over the full K, where 256 x 256 tiles fill half the
+// CUs or need their K cut in two and a second kernel to add the halves).  Eight waves as 4 x 2, 64 x 64 each; four
+// threads share a weight row of a k step (16 weights each), the X tile and the schedule are those of the kernel
+// above.
+template <int TYPE>
+__global__ __launch_bounds__(512) void gemm_bf16_n128_kernel(GemmParams p)
+{
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int BM = 256, BN = 128, WAVES_N = 2, WM = 64, WN = 64, TM = 2, TN = 2;
+    constexpr int A_BYTES = BM * GEMM_LD, B_BYTES = BN * GEMM_LD;
+    constexpr int XROWS = 64;
+    using Raw = typename std::conditional<TYPE == KQ_TYPE_Q4_K, RawQ4,
+                                          typename std::conditional<TYPE == KQ_TYPE_Q5_K, RawQ5, RawQ6>::type>::type;
+    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
+    uint8_t* As = smem;
+    uint8_t* Bs = smem + 2 * A_BYTES;
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const uint32_t nk = p.K / GEMM_BK;
+    const uint32_t x_dst = (tid >> 3) * GEMM_LD + (tid & 7u) * 16u;
+    const uint32_t wrow = tid >> 2, whf = (tid >> 1) & 1u, wq = tid & 1u;
+    const uint32_t w_dst = wrow * GEMM_LD + (tid & 3u) * 32u;
+    const uint32_t a_src = (wm * WM + (lane & 31u)) * GEMM_LD + (lane >> 5) * 16u;
+    const uint32_t b_src = (wn * WN + (lane & 31u)) * GEMM_LD + (lane >> 5) * 16u;
+    const uint32_t tile = blockIdx.x;
+    const uint32_t m0 = (tile / p.tiles_n) * BM, n0 = (tile % p.tiles_n) * BN;
+
+    const uint8_t* xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t m = min(m0 + i * XROWS + (tid >> 3), p.M - 1u);
+        xsrc[i] = (const uint8_t*)p.X + (size_t)m * p.K * 2u + (tid & 7u) * 16u;
+    }
+    const uint8_t* wsrc = p.W + (size_t)min(n0 + wrow, p.N - 1u) * p.row_stride_bytes;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    u32x4 xr[4];
+    Raw w;
+    float s0, s1, nb;
+    auto tile_at = [&](uint32_t t) { return min(t, nk - 1u); };
+    auto load_x = [&](uint32_t t, int i) { xr[i] = *(const u32x4*)(xsrc[i] + (size_t)tile_at(t) * (GEMM_BK * 2)); };
+    auto scales = [&](uint32_t t) {
+        il_scales(w, tile_at(t), whf, s0, s1, nb);
+        if (Q6 && wq) s0 = s1;   // Q6_K: the second 16 of a run of 32 have a scale of their own
+    };
+    auto read_ops = [&](uint32_t buf, int s, bf16x8 (&af)[TM], bf16x8 (&bfr)[TN]) {
+        const uint8_t* a = As + buf * A_BYTES + a_src + s * 32;
+        const uint8_t* b = Bs + buf * B_BYTES + b_src + s * 32;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[i] = *(const bf16x8*)(a + i * 32 * GEMM_LD);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bfr[j] = *(const bf16x8*)(b + j * 32 * GEMM_LD);
+    };
+    auto mfma_ops = [&](const bf16x8 (&af)[TM], const bf16x8 (&bfr)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    };
+    // piece v of tile t: the X copy, and for v < 2 eight of the thread's sixteen weights, into LDS buffer t&1; the
+    // piece's registers are then refilled from tile t+1
+    auto convert_piece = [&](uint32_t t, int v, bool refill = true, bool extra = true) {
+        const uint32_t buf = t & 1u;
+        *(u32x4*)(As + buf * A_BYTES + x_dst + v * XROWS * GEMM_LD) = xr[v];
+        if (v < 2) *(u32x4*)(Bs + buf * B_BYTES + w_dst + v * 16) = il_expand(w, tile_at(t), whf, v, s0, s1, nb);
+        load_x(t + 1u, v);
+        if (v == 1 && refill) il1_load_q(wsrc, tile_at(t + 1u), whf, wq, w, extra);
+    };
+    auto slice_schedule = [&]() {
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+#pragma unroll
+        for (int g = 0; g < TM * TN; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_x(0, i);
+    il_load_head(wsrc, tile_at(0), whf, w);
+    il1_load_q(wsrc, tile_at(0), whf, wq, w);
+    scales(0);
+    il_load_head(wsrc, tile_at(1), whf, w);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) convert_piece(0, v);
+    scales(1);
+    il_load_head(wsrc, tile_at(2), whf, w);
+    convert_piece(1, 0);
+    __syncthreads();
+
+    bf16x8 af[2][TM], bfr[2][TN];
+    read_ops(0, 0, af[0], bfr[0]);
+    auto k_step = [&](uint32_t kt, bool refill, bool new_block, bool opens) {
+        const uint32_t buf = kt & 1u;
+#pragma unroll
+        for (int s = 0; s < 3; ++s) {
+            read_ops(buf, s + 1, af[(s + 1) & 1], bfr[(s + 1) & 1]);
+            mfma_ops(af[s & 1], bfr[s & 1]);
+            convert_piece(kt + 1u, s + 1, refill, opens);
+            slice_schedule();
+        }
+        __syncthreads();
+        read_ops(buf ^ 1u, 0, af[0], bfr[0]);
+        mfma_ops(af[1], bfr[1]);
+        scales(kt + 2u);
+        il_load_head(wsrc, tile_at(kt + 3u), whf, w, new_block);
+        convert_piece(kt + 2u, 0);
+        slice_schedule();
+    };
+    for (uint32_t kt = 0; kt < nk; kt += 4u) {
+        k_step(kt, true, false, false);
+        k_step(kt + 1u, !Q6, true, false);
+        k_step(kt + 2u, true, false, true);
+        k_step(kt + 3u, !Q6, false, false);
+    }
+    store_acc<TM, TN>(p, acc, m0 + wm * WM, n0 + wn * WN, lane);
+}
+
 // Sums the runs of the tiles that the persistent kernel's cut points split, adds the bias and stores Y.
 // blockIdx.x = cut point (between workgroups b and b+1 of the walk), blockIdx.y = which of the 8
 // accumulator blocks of every wave's 128 x 64 share; thread = (wave, lane) of the persistent kernel.  The
@@ -764,6 +916,23 @@ static hipError_t launch_gemm_persistent(GemmParams p, uint32_t share, const Spl
     return hipGetLastError();
 }
 
+template <int TYPE>
+static hipError_t launch_gemm_n128(GemmParams p, hipStream_t s)
+{
+    constexpr size_t shmem = 2 * (size_t)(256 + 128) * GEMM_LD;
+    auto kern = gemm_bf16_n128_kernel<TYPE>;
+    static bool raised = false;   // per instantiation
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    p.tiles_n = (p.N + 127u) / 128u;
+    const uint32_t tiles = ((p.M + 255u) / 256u) * p.tiles_n;
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(512), shmem, s, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const SplitScratch& sc, hipStream_t s)
 {
     GemmParams p{};
@@ -776,7 +945,7 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const Spli
     p.row_stride_bytes = a.row_stride_bytes;
     p.ldy = a.ldy;
     const bool q4 = a.type == KQ_TYPE_Q4_K, q5 = a.type == KQ_TYPE_Q5_K;
-    // Three ways to run a shape, priced in microseconds with figures measured on the Llama-3-8B matrices at
+    // Four ways to run a shape, priced in microseconds with figures measured on the Llama-3-8B matrices at
     // M = 256 .. 2048: (a) 256-tiles, one workgroup per tile, in rounds over the CUs; (b) the walk over all
     // (tile, k step) units of the 256-tiles cut into equal shares, one per CU, where every run over part of a
     // tile costs a workspace slot (256 KB written, read back by the sum kernel); (c) 128-tiles, two workgroups
@@ -793,8 +962,23 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const Spli
     const float t_small = (float)((small + 2u * cus - 1u) / (2u * cus)) * ((float)nk * tk128 + 0.25f * te);
     bool use_big = t_small > (t_whole < t_shares ? t_whole : t_shares);
     uint32_t share = t_shares < t_whole ? one_per_cu : nk;
-    if (tile == 256) use_big = true;
-    if (tile == 128) use_big = false;
+    // (d) 256 x 128 tiles, whole, in rounds over the CUs: a k step 1.08 us (Q4_K) / 1.3 us (Q6_K), an epilogue
+    // 8 us, and three quarters of that while half of the CUs or more have no tile.  Measured: 4096 x 4096 Q4_K at
+    // M = 2048 87 against 106 us for the cheapest of (a)..(c) inside a pass over a layer set (77 against 96-100 us
+    // launched back to back), at M = 1024 57 against 62 us; 4096 x 14336 Q6_K at M = 2048 269 against 267 us for
+    // equal shares inside the pass (259 against 270 back to back), at M = 1024 183 against 147 us: priced so that
+    // the Q6_K matrix keeps its equal shares.
+    const uint64_t half = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 127u) / 128u);
+    const float tk_h = q4 ? 1.08f : q5 ? 1.15f : 1.3f;
+    const float t_half = (float)((half + cus - 1u) / cus) * ((float)nk * tk_h + 8.0f) * (2u * half <= cus ? 0.75f : 1.0f);
+    const float t_best = t_small < (t_whole < t_shares ? t_whole : t_shares) ? t_small : (t_whole < t_shares ? t_whole : t_shares);
+    bool use_half = t_half < t_best;
+    if (tile == 256) { use_big = true; use_half = false; }
+    if (tile == 128) { use_big = false; use_half = false; }
+    if (tile == 129) use_half = true;
+    if (split != 0) use_half = use_half && tile == 129;   // a forced split means the 256-tile walk
+    if (use_half)
+        return q4 ? launch_gemm_n128<KQ_TYPE_Q4_K>(p, s) : q5 ? launch_gemm_n128<KQ_TYPE_Q5_K>(p, s) : launch_gemm_n128<KQ_TYPE_Q6_K>(p, s);
     if (split == 1) share = nk;
     if (split == 2) share = one_per_cu;              // forced: any number of runs per tile
     if (use_big)

@@ -509,8 +509,8 @@ BPK_API int bpk_force_kernel(int family);
  * K-range splits of the row-per-lane GEMV, or rows per wave of the
  * lanes-along-K GEMV; "gemv_waves": waves per workgroup of the row-per-lane
  * kernels (2, 4 or 8); "gemv_depth": rows a wave of the lanes-along-K GEMV
- * keeps in flight (1, 2 or 4); "gemm_tile": square workgroup tile of the bf16
- * GEMM (128 or 256); "gemm_split": how the 256-tile GEMM hands out work
+ * keeps in flight (1, 2 or 4); "gemm_tile": workgroup tile of the bf16
+ * GEMM (128 or 256: square; 129: 256 tokens x 128 weight rows); "gemm_split": how the 256-tile GEMM hands out work
  * (1 = one tile per workgroup, 2 = the walk over tiles and k steps cut into
  * equal shares per compute unit; the runs of a tile cut between workgroups go
  * through a per-device workspace and are added in the order of the walk, so

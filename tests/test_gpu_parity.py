@@ -526,6 +526,14 @@ GEMM_SHAPES = [
     # 256-tile, one tile per workgroup
     (Q4_K, 512, 1024, 4096, 257),
     (Q6_K, 300, 520, 768, 257),
+    # 256 tokens x 128 rows per workgroup (option value 129)
+    (Q4_K, 300, 520, 768, 129),
+    (Q4_K, 512, 1024, 4096, 129),
+    (Q4_K, 33, 70, 2048, 129),
+    (Q5_K, 300, 520, 1024, 129),
+    (Q6_K, 190, 260, 1024, 129),
+    (Q6_K, 256, 256, 768, 129),      # odd block count
+    (Q6_K, 512, 512, 4096, 129),
 ]
 
 
