@@ -364,12 +364,33 @@ __device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint3
     const u32x4* q = (const u32x4*)(row + (size_t)(kc >> 2) * KQ_Q4K_BYTES + 16 + (kc & 3u) * 32u);
     if (half == 0) r.q0 = q[0]; else r.q1 = q[1];
 }
-__device__ __forceinline__ void il_scales(const RawQ4& r, uint32_t kc, uint32_t hf, float& s0, float& s1, float& nb)
+// Scale and minimum of sub-block 2 * c + hf of a Q4_K / Q5_K header, c = the k step's place in its superblock.  The
+// k loop knows c at compile time (cpos >= 0): the choice between the two 6-bit layouts is then no branch, which
+// q4k_scale_min's is (it cut every k step of the loop into three basic blocks).
+__device__ __forceinline__ void il_scale_min(uint32_t u0, uint32_t u1, uint32_t u2, uint32_t kc, uint32_t hf, int cpos,
+                                             uint32_t& sc, uint32_t& mn)
+{
+    if (cpos < 0) {
+        q4k_scale_min(u0, u1, u2, (int)((kc & 3u) * 2u + hf), sc, mn);
+        return;
+    }
+    const uint32_t sh = 8u * ((2u * (uint32_t)cpos + hf) & 3u);
+    const uint32_t a = (u0 >> sh) & 255u, b = (u1 >> sh) & 255u;
+    if (cpos < 2) {
+        sc = a & 63u;
+        mn = b & 63u;
+    } else {
+        const uint32_t c = (u2 >> sh) & 255u;
+        sc = (c & 15u) | ((a >> 6) << 4);
+        mn = (c >> 4) | ((b >> 6) << 4);
+    }
+}
+__device__ __forceinline__ void il_scales(const RawQ4& r, uint32_t kc, uint32_t hf, float& s0, float& s1, float& nb, int cpos = -1)
 {
     const float d = half_bits_to_float(r.h.x & 0xFFFFu);
     const float dmin = half_bits_to_float(r.h.x >> 16);
     uint32_t sc, mn;
-    q4k_scale_min(r.h.y, r.h.z, r.h.w, (int)((kc & 3u) * 2u + hf), sc, mn);
+    il_scale_min(r.h.y, r.h.z, r.h.w, kc, hf, cpos, sc, mn);
     // a masked nibble is left where it is and read as an fp16 subnormal, q * 2^-24 (low nibble) or q * 2^-20 (high
     // nibble): the scale carries the matching power of two (an exact scaling, so fma(q_h, s0, nb) rounds the same
     // exact value as fma(d * sc, q, nb) does)
@@ -418,12 +439,12 @@ __device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint3
     if (half == 0) { r.q0 = q[0]; if (extra) r.b0 = b[0]; }
     else { r.q1 = q[1]; if (extra) r.b1 = b[1]; }
 }
-__device__ __forceinline__ void il_scales(const RawQ5& r, uint32_t kc, uint32_t hf, float& s0, float& s1, float& nb)
+__device__ __forceinline__ void il_scales(const RawQ5& r, uint32_t kc, uint32_t hf, float& s0, float& s1, float& nb, int cpos = -1)
 {
     const float d = half_bits_to_float(r.h.x & 0xFFFFu);
     const float dmin = half_bits_to_float(r.h.x >> 16);
     uint32_t sc, mn;
-    q4k_scale_min(r.h.y, r.h.z, r.h.w, (int)((kc & 3u) * 2u + hf), sc, mn);
+    il_scale_min(r.h.y, r.h.z, r.h.w, kc, hf, cpos, sc, mn);
     s0 = d * (float)sc;
     s1 = s0;
     nb = -(dmin * (float)mn);
@@ -471,7 +492,7 @@ __device__ __forceinline__ void il_load_q(const uint8_t* row, uint32_t kc, uint3
         __builtin_memcpy(&r.b1, blk + 128u + 32u * h + 16u, 16);
     }
 }
-__device__ __forceinline__ void il_scales(const RawQ6& r, uint32_t, uint32_t, float& s0, float& s1, float& nb)
+__device__ __forceinline__ void il_scales(const RawQ6& r, uint32_t, uint32_t, float& s0, float& s1, float& nb, int = -1)
 {
     const float d = half_bits_to_float(r.d16);
     s0 = d * (float)(int)(int8_t)(r.sc2 & 255u);
@@ -600,11 +621,11 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
     il_load_head(wsrc, tile_at(0), whf, w);
     il_load_q(wsrc, tile_at(0), whf, 0, w);
     il_load_q(wsrc, tile_at(0), whf, 1, w);
-    il_scales(w, tile_at(0), whf, s0, s1, nb);
+    il_scales(w, tile_at(0), whf, s0, s1, nb, 0);
     il_load_head(wsrc, tile_at(1), whf, w);
 #pragma unroll
     for (int v = 0; v < 4; ++v) convert_piece(0, v);
-    il_scales(w, tile_at(1), whf, s0, s1, nb);
+    il_scales(w, tile_at(1), whf, s0, s1, nb, 1);
     il_load_head(wsrc, tile_at(2), whf, w);
     convert_piece(1, 0);
     __syncthreads();
@@ -613,8 +634,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
     read_ops(0, 0, af[0], bfr[0]);
     // one k step; refill = whether the quant registers freed by tile kt+1 are loaded with tile kt+2,
     // new_block = whether tile kt+3 opens a superblock (else its header is the one already in registers)
-    // (opens = whether tile kt+2 opens a superblock)
-    auto k_step = [&](uint32_t kt, bool refill, bool new_block, bool opens) {
+    // (opens = whether tile kt+2 opens a superblock; pos2 = the place of tile kt+2 in its superblock: runs start on
+    // a superblock, and the tiles past a run's end, clamped to its last, are never multiplied)
+    auto k_step = [&](uint32_t kt, bool refill, bool new_block, bool opens, int pos2) {
         const uint32_t buf = kt & 1u;
         // slices 0..2 of tile kt; pieces 1..3 of tile kt+1 go to the other buffer
 #pragma unroll
@@ -630,7 +652,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
         // tile kt+1 are fetched and piece 0 of tile kt+2 replaces tile kt in LDS.
         read_ops(buf ^ 1u, 0, af[0], bfr[0]);
         mfma_ops(af[1], bfr[1]);
-        il_scales(w, tile_at(kt + 2u), whf, s0, s1, nb);
+        il_scales(w, tile_at(kt + 2u), whf, s0, s1, nb, pos2);
         il_load_head(wsrc, tile_at(kt + 3u), whf, w, new_block);
         convert_piece(kt + 2u, 0);
         slice_schedule();
@@ -643,10 +665,10 @@ __global__ __launch_bounds__(512) void gemm_bf16_sk_kernel(GemmParams p)
     // odd tile after it.
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
     for (uint32_t kt = 0; kt < nk; kt += 4u) {
-        k_step(kt, true, false, false);
-        k_step(kt + 1u, !Q6, true, false);
-        k_step(kt + 2u, true, false, true);
-        k_step(kt + 3u, !Q6, false, false);
+        k_step(kt, true, false, false, 2);
+        k_step(kt + 1u, !Q6, true, false, 3);
+        k_step(kt + 2u, true, false, true, 0);
+        k_step(kt + 3u, !Q6, false, false, 1);
     }
 
     // A tile walked in one piece is stored.  A run over part of a tile leaves its sums in the workspace, in
@@ -744,8 +766,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_n128_kernel(GemmParams p)
     float s0, s1, nb;
     auto tile_at = [&](uint32_t t) { return min(t, nk - 1u); };
     auto load_x = [&](uint32_t t, int i) { xr[i] = *(const u32x4*)(xsrc[i] + (size_t)tile_at(t) * (GEMM_BK * 2)); };
-    auto scales = [&](uint32_t t) {
-        il_scales(w, tile_at(t), whf, s0, s1, nb);
+    auto scales = [&](uint32_t t, int pos) {
+        il_scales(w, tile_at(t), whf, s0, s1, nb, pos);
         if (Q6 && wq) s0 = s1;   // Q6_K: the second 16 of a run of 32 have a scale of their own
     };
     auto read_ops = [&](uint32_t buf, int s, bf16x8 (&af)[TM], bf16x8 (&bfr)[TN]) {
@@ -786,18 +808,18 @@ __global__ __launch_bounds__(512) void gemm_bf16_n128_kernel(GemmParams p)
     for (int i = 0; i < 4; ++i) load_x(0, i);
     il_load_head(wsrc, tile_at(0), whf, w);
     il1_load_q(wsrc, tile_at(0), whf, wq, w);
-    scales(0);
+    scales(0, 0);
     il_load_head(wsrc, tile_at(1), whf, w);
 #pragma unroll
     for (int v = 0; v < 4; ++v) convert_piece(0, v);
-    scales(1);
+    scales(1, 1);
     il_load_head(wsrc, tile_at(2), whf, w);
     convert_piece(1, 0);
     __syncthreads();
 
     bf16x8 af[2][TM], bfr[2][TN];
     read_ops(0, 0, af[0], bfr[0]);
-    auto k_step = [&](uint32_t kt, bool refill, bool new_block, bool opens) {
+    auto k_step = [&](uint32_t kt, bool refill, bool new_block, bool opens, int pos2) {
         const uint32_t buf = kt & 1u;
 #pragma unroll
         for (int s = 0; s < 3; ++s) {
@@ -809,16 +831,16 @@ __global__ __launch_bounds__(512) void gemm_bf16_n128_kernel(GemmParams p)
         __syncthreads();
         read_ops(buf ^ 1u, 0, af[0], bfr[0]);
         mfma_ops(af[1], bfr[1]);
-        scales(kt + 2u);
+        scales(kt + 2u, pos2);
         il_load_head(wsrc, tile_at(kt + 3u), whf, w, new_block);
         convert_piece(kt + 2u, 0);
         slice_schedule();
     };
     for (uint32_t kt = 0; kt < nk; kt += 4u) {
-        k_step(kt, true, false, false);
-        k_step(kt + 1u, !Q6, true, false);
-        k_step(kt + 2u, true, false, true);
-        k_step(kt + 3u, !Q6, false, false);
+        k_step(kt, true, false, false, 2);
+        k_step(kt + 1u, !Q6, true, false, 3);
+        k_step(kt + 2u, true, false, true, 0);
+        k_step(kt + 3u, !Q6, false, false, 1);
     }
     store_acc<TM, TN>(p, acc, m0 + wm * WM, n0 + wn * WN, lane);
 }
