@@ -42,17 +42,14 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h16)
 __device__ __forceinline__ void q4k_scale_min(uint32_t u0, uint32_t u1, uint32_t u2, int sb,
                                               uint32_t& sc, uint32_t& mn)
 {
+    // (both layouts are computed and one is selected: a branch here cuts the caller's loop body into basic blocks)
     const int j = sb & 3;
     const uint32_t a = (u0 >> (8 * j)) & 255u;
     const uint32_t b = (u1 >> (8 * j)) & 255u;
-    if (sb < 4) {
-        sc = a & 63u;
-        mn = b & 63u;
-    } else {
-        const uint32_t c = (u2 >> (8 * j)) & 255u;
-        sc = (c & 15u) | ((a >> 6) << 4);
-        mn = (c >> 4) | ((b >> 6) << 4);
-    }
+    const uint32_t c = (u2 >> (8 * j)) & 255u;
+    const bool low = sb < 4;
+    sc = low ? (a & 63u) : ((c & 15u) | ((a >> 6) << 4));
+    mn = low ? (b & 63u) : ((c >> 4) | ((b >> 6) << 4));
 }
 
 // Byte-granular read through the word array (any alignment of the block).

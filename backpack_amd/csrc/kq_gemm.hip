@@ -1003,6 +1003,31 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const Spli
         return q4 ? launch_gemm_n128<KQ_TYPE_Q4_K>(p, s) : q5 ? launch_gemm_n128<KQ_TYPE_Q5_K>(p, s) : launch_gemm_n128<KQ_TYPE_Q6_K>(p, s);
     if (split == 1) share = nk;
     if (split == 2) share = one_per_cu;              // forced: any number of runs per tile
+    // Whole 256-tiles whose last round over the CUs is at most half full (gate|up at M = 2048: 896 tiles = 3.5
+    // rounds): the last round's tiles, a block of weight rows over all tokens, run as 256 x 128 tiles in a second
+    // launch — twice as many, so they fill the CUs — behind the full rounds.
+    if (use_big && share == nk && tile == 0 && split == 0) {
+        const uint32_t m_tiles = (a.M + 255u) / 256u, n_tiles = (a.N + 255u) / 256u;
+        const uint32_t rounds = (uint32_t)(big / cus), rest = (uint32_t)(big % cus);
+        if (rounds >= 1u && rest > 0u && 2u * rest <= cus && rest % m_tiles == 0u) {
+            const float t_two = (float)rounds * ((float)nk * tk + te) + ((float)nk * tk_h + 8.0f) + 3.0f;
+            if (t_two < t_whole) {
+                const uint32_t n1 = (n_tiles - rest / m_tiles) * 256u;   // weight rows of the full rounds
+                GemmParams p1 = p, p2 = p;
+                p1.N = n1;
+                p2.N = a.N - n1;
+                p2.W = p.W + (size_t)n1 * p.row_stride_bytes;
+                p2.Y = p.Y + n1;
+                p2.bias = p.bias ? p.bias + n1 : nullptr;
+                hipError_t e = q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p1, nk, sc, s)
+                                  : q5 ? launch_gemm_persistent<KQ_TYPE_Q5_K>(p1, nk, sc, s)
+                                       : launch_gemm_persistent<KQ_TYPE_Q6_K>(p1, nk, sc, s);
+                if (e != hipSuccess) return e;
+                return q4 ? launch_gemm_n128<KQ_TYPE_Q4_K>(p2, s)
+                          : q5 ? launch_gemm_n128<KQ_TYPE_Q5_K>(p2, s) : launch_gemm_n128<KQ_TYPE_Q6_K>(p2, s);
+            }
+        }
+    }
     if (use_big)
         return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, share, sc, s)
                   : q5 ? launch_gemm_persistent<KQ_TYPE_Q5_K>(p, share, sc, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, share, sc, s);
