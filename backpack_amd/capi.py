@@ -69,6 +69,8 @@ class ModelConfig(C.Structure):
 
 _SIGS = {
     "bpk_version": (C.c_int, []),
+    "bpk_gemm_plan": (C.c_int, [C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(C.c_int),
+                                C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "bpk_last_error": (C.c_char_p, []),
     "bpk_last_kernel": (C.c_char_p, []),
     "bpk_force_kernel": (C.c_int, [C.c_int]),
@@ -178,3 +180,10 @@ def force_kernel(family: int) -> None:
 
 def set_option(name: str, value: int) -> None:
     check(lib().bpk_set_option(name.encode(), value))
+
+
+def gemm_plan(type_: int, M: int, N: int, K: int, compute_units: int = 256):
+    """(form, share, rows_first) of the bf16 dequant-GEMM for a shape: host arithmetic, no device needed."""
+    form, share, first = C.c_int(), C.c_uint32(), C.c_uint32()
+    check(lib().bpk_gemm_plan(type_, M, N, K, compute_units, C.byref(form), C.byref(share), C.byref(first)))
+    return form.value, share.value, first.value

@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "kq_format.h"
+#include "kq_gemm_plan.h"
 #include "kq_kernels.h"
 
 namespace {
@@ -241,6 +242,20 @@ int bpk_set_option(const char* name, int value)
         return BPK_OK;
     }
     return fail(BPK_ERR_SHAPE, "unknown option '%s'", name);
+}
+
+int bpk_gemm_plan(int type, uint32_t M, uint32_t N, uint32_t K, uint32_t compute_units, int* form, uint32_t* share,
+                  uint32_t* rows_first)
+{
+    if (!known_type(type)) return fail(BPK_ERR_TYPE, "unsupported GGUF type (Q4_K=12, Q5_K=13, Q6_K=14)");
+    if (!form || !share || !rows_first) return fail(BPK_ERR_NULL, "form, share and rows_first must be non-null");
+    if (M == 0 || N == 0 || K == 0 || K % KQ_QK || compute_units == 0)
+        return fail(BPK_ERR_SHAPE, "M, N, compute_units must be positive and K a positive multiple of 256");
+    const kq::GemmPlan pl = kq::plan_gemm_bf16(type, M, N, K, compute_units, t_gemm_tile, t_gemm_split);
+    *form = pl.form;
+    *share = pl.share;
+    *rows_first = pl.rows_first;
+    return BPK_OK;
 }
 
 int bpk_init(int device) { return ensure_device(device, nullptr); }

@@ -30,6 +30,7 @@
 // 32 consecutive floats of one Y row.
 #include "kq_format.h"
 #include "kq_kernels.h"
+#include "kq_gemm_plan.h"
 #include <type_traits>
 
 namespace kq {
@@ -967,72 +968,31 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const Spli
     p.row_stride_bytes = a.row_stride_bytes;
     p.ldy = a.ldy;
     const bool q4 = a.type == KQ_TYPE_Q4_K, q5 = a.type == KQ_TYPE_Q5_K;
-    // Four ways to run a shape, priced in microseconds with figures measured on the Llama-3-8B matrices at
-    // M = 256 .. 2048: (a) 256-tiles, one workgroup per tile, in rounds over the CUs; (b) the walk over all
-    // (tile, k step) units of the 256-tiles cut into equal shares, one per CU, where every run over part of a
-    // tile costs a workspace slot (256 KB written, read back by the sum kernel); (c) 128-tiles, two workgroups
-    // per CU.  A k step of a 256-tile takes tk, of a 128-tile tk128; a tile's epilogue te.
-    const uint32_t cus = device_cu_count(), nk = a.K / GEMM_BK;
-    const uint64_t big = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 255u) / 256u);
-    const uint64_t small = (uint64_t)((a.M + 127u) / 128u) * ((a.N + 127u) / 128u);
-    const float tk = q4 ? 1.7f : q5 ? 1.9f : 2.2f, tk128 = q4 ? 1.4f : q5 ? 1.6f : 2.0f, te = 12.0f, t_slot = 0.1f, t_sum = 5.0f;
-    const uint32_t one_per_cu = (uint32_t)((big * nk + cus - 1u) / cus);   // equal shares over all CUs
-    const uint64_t runs = (big * nk + one_per_cu - 1u) / one_per_cu;
-    const float t_whole = (float)((big + cus - 1u) / cus) * ((float)nk * tk + te);
-    const float t_shares = (float)one_per_cu * tk + te * (1.0f + (float)one_per_cu / (float)nk)
-                           + t_slot * (float)(one_per_cu < nk ? runs : 2u * (runs - 1u)) + t_sum;
-    const float t_small = (float)((small + 2u * cus - 1u) / (2u * cus)) * ((float)nk * tk128 + 0.25f * te);
-    bool use_big = t_small > (t_whole < t_shares ? t_whole : t_shares);
-    uint32_t share = t_shares < t_whole ? one_per_cu : nk;
-    // (d) 256 x 128 tiles, whole, in rounds over the CUs: a k step 1.08 us (Q4_K) / 1.3 us (Q6_K), an epilogue
-    // 8 us, and three quarters of that while half of the CUs or more have no tile.  Measured: 4096 x 4096 Q4_K at
-    // M = 2048 87 against 106 us for the cheapest of (a)..(c) inside a pass over a layer set (77 against 96-100 us
-    // launched back to back), at M = 1024 57 against 62 us; 4096 x 14336 Q6_K at M = 2048 269 against 267 us for
-    // equal shares inside the pass (259 against 270 back to back), at M = 1024 183 against 147 us: priced so that
-    // the Q6_K matrix keeps its equal shares.
-    const uint64_t half = (uint64_t)((a.M + 255u) / 256u) * ((a.N + 127u) / 128u);
-    const float tk_h = q4 ? 1.08f : q5 ? 1.15f : 1.3f;
-    const float t_half = (float)((half + cus - 1u) / cus) * ((float)nk * tk_h + 8.0f) * (2u * half <= cus ? 0.75f : 1.0f);
-    const float t_best = t_small < (t_whole < t_shares ? t_whole : t_shares) ? t_small : (t_whole < t_shares ? t_whole : t_shares);
-    bool use_half = t_half < t_best;
-    if (tile == 256) { use_big = true; use_half = false; }
-    if (tile == 128) { use_big = false; use_half = false; }
-    if (tile == 129) use_half = true;
-    if (split != 0) use_half = use_half && tile == 129;   // a forced split means the 256-tile walk
-    if (use_half)
+    const GemmPlan plan = plan_gemm_bf16(a.type, a.M, a.N, a.K, device_cu_count(), tile, split);
+    switch (plan.form) {
+    case GEMM_FORM_HALF:
         return q4 ? launch_gemm_n128<KQ_TYPE_Q4_K>(p, s) : q5 ? launch_gemm_n128<KQ_TYPE_Q5_K>(p, s) : launch_gemm_n128<KQ_TYPE_Q6_K>(p, s);
-    if (split == 1) share = nk;
-    if (split == 2) share = one_per_cu;              // forced: any number of runs per tile
-    // Whole 256-tiles whose last round over the CUs is at most half full (gate|up at M = 2048: 896 tiles = 3.5
-    // rounds): the last round's tiles, a block of weight rows over all tokens, run as 256 x 128 tiles in a second
-    // launch — twice as many, so they fill the CUs — behind the full rounds.
-    if (use_big && share == nk && tile == 0 && split == 0) {
-        const uint32_t m_tiles = (a.M + 255u) / 256u, n_tiles = (a.N + 255u) / 256u;
-        const uint32_t rounds = (uint32_t)(big / cus), rest = (uint32_t)(big % cus);
-        if (rounds >= 1u && rest > 0u && 2u * rest <= cus && rest % m_tiles == 0u) {
-            const float t_two = (float)rounds * ((float)nk * tk + te) + ((float)nk * tk_h + 8.0f) + 3.0f;
-            if (t_two < t_whole) {
-                const uint32_t n1 = (n_tiles - rest / m_tiles) * 256u;   // weight rows of the full rounds
-                GemmParams p1 = p, p2 = p;
-                p1.N = n1;
-                p2.N = a.N - n1;
-                p2.W = p.W + (size_t)n1 * p.row_stride_bytes;
-                p2.Y = p.Y + n1;
-                p2.bias = p.bias ? p.bias + n1 : nullptr;
-                hipError_t e = q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p1, nk, sc, s)
-                                  : q5 ? launch_gemm_persistent<KQ_TYPE_Q5_K>(p1, nk, sc, s)
-                                       : launch_gemm_persistent<KQ_TYPE_Q6_K>(p1, nk, sc, s);
-                if (e != hipSuccess) return e;
-                return q4 ? launch_gemm_n128<KQ_TYPE_Q4_K>(p2, s)
-                          : q5 ? launch_gemm_n128<KQ_TYPE_Q5_K>(p2, s) : launch_gemm_n128<KQ_TYPE_Q6_K>(p2, s);
-            }
-        }
+    case GEMM_FORM_ROUNDS_THEN_HALF: {
+        GemmParams p1 = p, p2 = p;
+        p1.N = plan.rows_first;
+        p2.N = a.N - plan.rows_first;
+        p2.W = p.W + (size_t)plan.rows_first * p.row_stride_bytes;
+        p2.Y = p.Y + plan.rows_first;
+        p2.bias = p.bias ? p.bias + plan.rows_first : nullptr;
+        hipError_t e = q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p1, plan.share, sc, s)
+                          : q5 ? launch_gemm_persistent<KQ_TYPE_Q5_K>(p1, plan.share, sc, s)
+                               : launch_gemm_persistent<KQ_TYPE_Q6_K>(p1, plan.share, sc, s);
+        if (e != hipSuccess) return e;
+        return q4 ? launch_gemm_n128<KQ_TYPE_Q4_K>(p2, s) : q5 ? launch_gemm_n128<KQ_TYPE_Q5_K>(p2, s) : launch_gemm_n128<KQ_TYPE_Q6_K>(p2, s);
     }
-    if (use_big)
-        return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, share, sc, s)
-                  : q5 ? launch_gemm_persistent<KQ_TYPE_Q5_K>(p, share, sc, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, share, sc, s);
-    return q4 ? launch_gemm<KQ_TYPE_Q4_K, 128, 128, 4>(p, s)
-              : q5 ? launch_gemm<KQ_TYPE_Q5_K, 128, 128, 4>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 128, 128, 4>(p, s);
+    case GEMM_FORM_WHOLE:
+    case GEMM_FORM_SHARES:
+        return q4 ? launch_gemm_persistent<KQ_TYPE_Q4_K>(p, plan.share, sc, s)
+                  : q5 ? launch_gemm_persistent<KQ_TYPE_Q5_K>(p, plan.share, sc, s) : launch_gemm_persistent<KQ_TYPE_Q6_K>(p, plan.share, sc, s);
+    default:
+        return q4 ? launch_gemm<KQ_TYPE_Q4_K, 128, 128, 4>(p, s)
+                  : q5 ? launch_gemm<KQ_TYPE_Q5_K, 128, 128, 4>(p, s) : launch_gemm<KQ_TYPE_Q6_K, 128, 128, 4>(p, s);
+    }
 }
 
 }  // namespace kq

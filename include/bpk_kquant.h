@@ -531,6 +531,17 @@ BPK_API int bpk_force_kernel(int family);
  * of the next op touched into L2 while an op finishes.  0 = automatic. */
 BPK_API int bpk_set_option(const char *name, int value);
 
+/* Which form of the bf16 dequant-GEMM bpk_kq_matmul_bf16 takes for a shape on a
+ * part of `compute_units` CUs, with this thread's "gemm_tile" / "gemm_split"
+ * options: host arithmetic only, no device is touched (diagnostic; the reference
+ * has no such kernel, its prefill loops M = 1, runtime/model_runner.cpp:6148-6158).
+ * *form: 0 = 128 x 128 tiles; 1 = 256 x 256 tiles, one workgroup each; 2 = the
+ * walk over the 256-tiles' k steps cut into equal shares (*share k steps each);
+ * 3 = tiles of 256 tokens x 128 weight rows; 4 = the full rounds of 256-tiles
+ * over the first *rows_first weight rows, then the rest as in 3. */
+BPK_API int bpk_gemm_plan(int type, uint32_t M, uint32_t N, uint32_t K, uint32_t compute_units,
+                          int *form, uint32_t *share, uint32_t *rows_first);
+
 #ifdef __cplusplus
 }
 #endif

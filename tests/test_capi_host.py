@@ -65,3 +65,60 @@ def test_matmul_argument_validation_needs_no_gpu():
     assert L.bpk_kq_matmul(Q4_K, one, C.c_void_p(18), None, one, 1, 8, 256, 1, 36, 0, None) == -4
     # n_blocks inconsistent with K
     assert L.bpk_kq_matmul(Q4_K, one, one, None, one, 1, 8, 512, 1, 72, 0, None) == -2
+
+
+# ---- which form of the bf16 dequant-GEMM serves a shape: host arithmetic, pinned on the shapes it was priced on ----
+SMALL, WHOLE, SHARES, HALF, ROUNDS_THEN_HALF = range(5)
+
+
+@pytest.mark.parametrize("name,type_,N,K,M,want", [
+    # the Llama-3-8B matrices at 2048 tokens on 256 CUs
+    ("gate_up", Q4_K, 28672, 4096, 2048, ROUNDS_THEN_HALF),   # 896 tiles = 3.5 rounds: 3 rounds, then 4096 rows as 256 x 128 tiles
+    ("qkv", Q4_K, 6144, 4096, 2048, WHOLE),                    # 192 tiles, under one round
+    ("o", Q4_K, 4096, 4096, 2048, HALF),                       # 256 tiles of 256 x 128: one per CU
+    ("down", Q6_K, 4096, 14336, 2048, SHARES),                 # 128 tiles of long K: every tile cut in two
+    ("lm_head", Q6_K, 128256, 4096, 2048, WHOLE),              # 4008 tiles; the last round is more than half full
+    # ... and at 512 tokens
+    ("gate_up", Q4_K, 28672, 4096, 512, WHOLE),
+    ("down", Q6_K, 4096, 14336, 512, SHARES),
+    ("o", Q4_K, 4096, 4096, 512, SHARES),
+    # one small tile's worth of work
+    ("tiny", Q4_K, 128, 256, 128, SMALL),
+])
+def test_gemm_plan_on_the_shapes_it_was_priced_on(name, type_, N, K, M, want):
+    form, share, first = capi.gemm_plan(type_, M, N, K, 256)
+    assert form == want, (name, form, share, first)
+    nk = K // 64
+    if form == ROUNDS_THEN_HALF:
+        # the first launch is whole rounds of whole tiles, the second at most one round of half tiles
+        m_tiles = -(-M // 256)
+        assert share == nk and first % 256 == 0 and 0 < first < N
+        assert (m_tiles * (first // 256)) % 256 == 0
+        assert m_tiles * -(-(N - first) // 128) <= 256
+    if form == WHOLE:
+        assert share == nk
+    if form == SHARES:
+        assert share % 4 == 0 and share != nk
+
+
+def test_gemm_plan_follows_the_options_and_refuses_bad_arguments():
+    try:
+        capi.set_option("gemm_tile", 128)
+        assert capi.gemm_plan(Q4_K, 2048, 28672, 4096)[0] == SMALL
+        capi.set_option("gemm_tile", 129)
+        assert capi.gemm_plan(Q4_K, 2048, 28672, 4096)[0] == HALF
+        capi.set_option("gemm_tile", 256)
+        capi.set_option("gemm_split", 1)
+        assert capi.gemm_plan(Q6_K, 2048, 4096, 14336)[:2] == (WHOLE, 14336 // 64)
+        capi.set_option("gemm_split", 2)
+        form, share, _ = capi.gemm_plan(Q4_K, 2048, 28672, 4096)
+        assert form == SHARES and share == 224    # 896 tiles x 64 steps over 256 CUs
+    finally:
+        capi.set_option("gemm_tile", 0)
+        capi.set_option("gemm_split", 0)
+    with pytest.raises(capi.BpkError):
+        capi.gemm_plan(Q4_K, 2048, 4096, 100)     # K not a multiple of 256
+    with pytest.raises(capi.BpkError):
+        capi.gemm_plan(11, 2048, 4096, 4096)      # unknown type
+    # a part with fewer CUs: o no longer fits one round of half tiles and the answer changes with the count
+    assert capi.gemm_plan(Q4_K, 2048, 4096, 4096, 128)[0] in (WHOLE, SHARES, HALF, SMALL)
