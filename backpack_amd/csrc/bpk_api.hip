@@ -205,7 +205,8 @@ int bpk_set_option(const char* name, int value)
         return BPK_OK;
     }
     if (!strcmp(name, "gemm_tile")) {
-        if (value != 0 && value != 128 && value != 129 && value != 256) return fail(BPK_ERR_SHAPE, "gemm_tile must be 0, 128, 129 or 256");
+        if (value != 0 && value != 128 && value != 129 && value != 192 && value != 256)
+            return fail(BPK_ERR_SHAPE, "gemm_tile must be 0, 128, 129, 192 or 256");
         t_gemm_tile = value;
         return BPK_OK;
     }

@@ -846,6 +846,157 @@ __global__ __launch_bounds__(512) void gemm_bf16_n128_kernel(GemmParams p)
     store_acc<TM, TN>(p, acc, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
+#ifndef KQ_N192_VALU
+#define KQ_N192_VALU 5
+#endif
+// 256 tokens x 192 weight rows per workgroup, whole tiles: N = 6144 at M = 2048 is 256 such tiles, one per CU, where
+// 256 x 256 tiles leave a quarter of the CUs without one.  The kernel above with waves of 64 x 96 and two items
+// per thread: a quarter row of rows 0..127 (as above) and one of rows 128..191 — those 64 rows are taken twice,
+// by threads t and t + 256, which store the same bytes: no wave has a path of its own, so the k loop stays one
+// basic block.  Item A's two pieces are expanded in the slice behind the barrier and the first slice of the next
+// step, item B's in the two slices after that: the places of pieces 0..3 in the 256-tile kernel.
+template <int TYPE>
+__global__ __launch_bounds__(512) void gemm_bf16_n192_kernel(GemmParams p)
+{
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int BM = 256, BN = 192, WAVES_N = 2, WM = 64, WN = 96, TM = 2, TN = 3;
+    constexpr int A_BYTES = BM * GEMM_LD, B_BYTES = BN * GEMM_LD;
+    constexpr int XROWS = 64;
+    using Raw = typename std::conditional<TYPE == KQ_TYPE_Q4_K, RawQ4,
+                                          typename std::conditional<TYPE == KQ_TYPE_Q5_K, RawQ5, RawQ6>::type>::type;
+    constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K;
+    uint8_t* As = smem;
+    uint8_t* Bs = smem + 2 * A_BYTES;
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const uint32_t nk = p.K / GEMM_BK;
+    const uint32_t x_dst = (tid >> 3) * GEMM_LD + (tid & 7u) * 16u;
+    const uint32_t wrow = tid >> 2, whf = (tid >> 1) & 1u, wq = tid & 1u;
+    const uint32_t wrow_b = 128u + ((tid >> 2) & 63u);
+    const uint32_t w_dst = wrow * GEMM_LD + (tid & 3u) * 32u;
+    const uint32_t w_dst_b = wrow_b * GEMM_LD + (tid & 3u) * 32u;
+    const uint32_t a_src = (wm * WM + (lane & 31u)) * GEMM_LD + (lane >> 5) * 16u;
+    const uint32_t b_src = (wn * WN + (lane & 31u)) * GEMM_LD + (lane >> 5) * 16u;
+    const uint32_t tile = blockIdx.x;
+    const uint32_t m0 = (tile / p.tiles_n) * BM, n0 = (tile % p.tiles_n) * BN;
+
+    const uint8_t* xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t m = min(m0 + i * XROWS + (tid >> 3), p.M - 1u);
+        xsrc[i] = (const uint8_t*)p.X + (size_t)m * p.K * 2u + (tid & 7u) * 16u;
+    }
+    const uint8_t* wsrc = p.W + (size_t)min(n0 + wrow, p.N - 1u) * p.row_stride_bytes;
+    const uint8_t* wsrc_b = p.W + (size_t)min(n0 + wrow_b, p.N - 1u) * p.row_stride_bytes;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    u32x4 xr[4];
+    Raw w, wb;
+    float s0, s1, nb, s0b, s1b, nbb;
+    auto tile_at = [&](uint32_t t) { return min(t, nk - 1u); };
+    auto load_x = [&](uint32_t t, int i) { xr[i] = *(const u32x4*)(xsrc[i] + (size_t)tile_at(t) * (GEMM_BK * 2)); };
+    auto scales_a = [&](uint32_t t, int pos) {
+        il_scales(w, tile_at(t), whf, s0, s1, nb, pos);
+        if (Q6 && wq) s0 = s1;   // Q6_K: the second 16 of a run of 32 have a scale of their own
+    };
+    auto scales_b = [&](uint32_t t, int pos) {
+        il_scales(wb, tile_at(t), whf, s0b, s1b, nbb, pos);
+        if (Q6 && wq) s0b = s1b;
+    };
+    auto read_ops = [&](uint32_t buf, int s, bf16x8 (&af)[TM], bf16x8 (&bfr)[TN]) {
+        const uint8_t* a = As + buf * A_BYTES + a_src + s * 32;
+        const uint8_t* b = Bs + buf * B_BYTES + b_src + s * 32;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[i] = *(const bf16x8*)(a + i * 32 * GEMM_LD);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bfr[j] = *(const bf16x8*)(b + j * 32 * GEMM_LD);
+    };
+    auto mfma_ops = [&](const bf16x8 (&af)[TM], const bf16x8 (&bfr)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    };
+    // piece v of tile t: the X copy and eight weights (v < 2 of item A, else of item B) into LDS buffer t&1; an
+    // item's registers are refilled from tile t+1 behind its second piece
+    auto convert_piece = [&](uint32_t t, int v, bool refill = true, bool extra = true) {
+        const uint32_t buf = t & 1u;
+        *(u32x4*)(As + buf * A_BYTES + x_dst + v * XROWS * GEMM_LD) = xr[v];
+        if (v < 2) *(u32x4*)(Bs + buf * B_BYTES + w_dst + v * 16) = il_expand(w, tile_at(t), whf, v, s0, s1, nb);
+        else *(u32x4*)(Bs + buf * B_BYTES + w_dst_b + (v - 2) * 16) = il_expand(wb, tile_at(t), whf, v - 2, s0b, s1b, nbb);
+        load_x(t + 1u, v);
+        if (v == 1 && refill) il1_load_q(wsrc, tile_at(t + 1u), whf, wq, w, extra);
+        if (v == 3 && refill) il1_load_q(wsrc_b, tile_at(t + 1u), whf, wq, wb, extra);
+    };
+    auto slice_schedule = [&]() {
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+#pragma unroll
+        for (int g = 0; g < TM * TN; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, KQ_N192_VALU, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_x(0, i);
+    il_load_head(wsrc, tile_at(0), whf, w);
+    il_load_head(wsrc_b, tile_at(0), whf, wb);
+    il1_load_q(wsrc, tile_at(0), whf, wq, w);
+    il1_load_q(wsrc_b, tile_at(0), whf, wq, wb);
+    scales_a(0, 0);
+    scales_b(0, 0);
+    il_load_head(wsrc, tile_at(1), whf, w);
+    il_load_head(wsrc_b, tile_at(1), whf, wb);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) convert_piece(0, v);
+    scales_a(1, 1);
+    il_load_head(wsrc, tile_at(2), whf, w);
+    convert_piece(1, 0);
+    __syncthreads();
+
+    bf16x8 af[2][TM], bfr[2][TN];
+    read_ops(0, 0, af[0], bfr[0]);
+    auto k_step = [&](uint32_t kt, bool refill, bool new_block, bool opens, int pos2) {
+        const uint32_t buf = kt & 1u;
+#pragma unroll
+        for (int s = 0; s < 3; ++s) {
+            read_ops(buf, s + 1, af[(s + 1) & 1], bfr[(s + 1) & 1]);
+            mfma_ops(af[s & 1], bfr[s & 1]);
+            if (s == 0) {   // item B runs a slice behind item A: its scales of tile kt+1, then the header of kt+2
+                scales_b(kt + 1u, (pos2 + 3) & 3);
+                il_load_head(wsrc_b, tile_at(kt + 2u), whf, wb, opens);
+            }
+            convert_piece(kt + 1u, s + 1, refill, opens);
+            slice_schedule();
+        }
+        __syncthreads();
+        read_ops(buf ^ 1u, 0, af[0], bfr[0]);
+        mfma_ops(af[1], bfr[1]);
+        scales_a(kt + 2u, pos2);
+        il_load_head(wsrc, tile_at(kt + 3u), whf, w, new_block);
+        convert_piece(kt + 2u, 0);
+        slice_schedule();
+    };
+    for (uint32_t kt = 0; kt < nk; kt += 4u) {
+        k_step(kt, true, false, false, 2);
+        k_step(kt + 1u, !Q6, true, false, 3);
+        k_step(kt + 2u, true, false, true, 0);
+        k_step(kt + 3u, !Q6, false, false, 1);
+    }
+    store_acc<TM, TN>(p, acc, m0 + wm * WM, n0 + wn * WN, lane);
+}
+
 // Sums the runs of the tiles that the persistent kernel's cut points split, adds the bias and stores Y.
 // blockIdx.x = cut point (between workgroups b and b+1 of the walk), blockIdx.y = which of the 8
 // accumulator blocks of every wave's 128 x 64 share; thread = (wave, lane) of the persistent kernel.  The
@@ -956,6 +1107,23 @@ static hipError_t launch_gemm_n128(GemmParams p, hipStream_t s)
     return hipGetLastError();
 }
 
+template <int TYPE>
+static hipError_t launch_gemm_n192(GemmParams p, hipStream_t s)
+{
+    constexpr size_t shmem = 2 * (size_t)(256 + 192) * GEMM_LD;
+    auto kern = gemm_bf16_n192_kernel<TYPE>;
+    static bool raised = false;   // per instantiation
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    p.tiles_n = (p.N + 191u) / 192u;
+    const uint32_t tiles = ((p.M + 255u) / 256u) * p.tiles_n;
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(512), shmem, s, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const SplitScratch& sc, hipStream_t s)
 {
     GemmParams p{};
@@ -972,6 +1140,8 @@ hipError_t launch_gemm_bf16(const MatmulArgs& a, int tile, int split, const Spli
     switch (plan.form) {
     case GEMM_FORM_HALF:
         return q4 ? launch_gemm_n128<KQ_TYPE_Q4_K>(p, s) : q5 ? launch_gemm_n128<KQ_TYPE_Q5_K>(p, s) : launch_gemm_n128<KQ_TYPE_Q6_K>(p, s);
+    case GEMM_FORM_192:
+        return q4 ? launch_gemm_n192<KQ_TYPE_Q4_K>(p, s) : q5 ? launch_gemm_n192<KQ_TYPE_Q5_K>(p, s) : launch_gemm_n192<KQ_TYPE_Q6_K>(p, s);
     case GEMM_FORM_ROUNDS_THEN_HALF: {
         GemmParams p1 = p, p2 = p;
         p1.N = plan.rows_first;

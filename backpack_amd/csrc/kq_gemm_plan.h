@@ -13,6 +13,7 @@ enum GemmForm : int {
     GEMM_FORM_SHARES = 2,            // the walk over the (256-tile, k step) units cut into equal shares, one per CU
     GEMM_FORM_HALF = 3,              // 256 tokens x 128 weight rows per workgroup, whole tiles
     GEMM_FORM_ROUNDS_THEN_HALF = 4,  // the full rounds of 256-tiles, then the last round's weight rows as 256 x 128 tiles
+    GEMM_FORM_192 = 5,               // 256 tokens x 192 weight rows per workgroup, whole tiles
 };
 
 struct GemmPlan {
@@ -26,7 +27,7 @@ struct GemmPlan {
 // equal shares, one per CU, where every run over part of a tile costs a workspace slot (256 KB written, read back
 // by the sum kernel); (c) 128-tiles, two workgroups per CU; (d) 256 x 128 tiles, whole, in rounds over the CUs.  A k
 // step of a 256-tile takes tk, of a 128-tile tk128, of a 256 x 128 tile tk_h; a 256-tile's epilogue te.
-// tile: 0 automatic, 128 / 256 force (c) / (a or b), 129 forces (d); split: 0 automatic, 1 whole tiles, 2 equal shares.
+// tile: 0 automatic, 128 / 256 force (c) / (a or b), 129 forces (d), 192 the 256 x 192 tile; split: 0 automatic, 1 whole tiles, 2 equal shares.
 inline GemmPlan plan_gemm_bf16(int type, uint32_t M, uint32_t N, uint32_t K, uint32_t cus, int tile, int split)
 {
     const bool q4 = type == KQ_TYPE_Q4_K, q5 = type == KQ_TYPE_Q5_K;
@@ -53,10 +54,19 @@ inline GemmPlan plan_gemm_bf16(int type, uint32_t M, uint32_t N, uint32_t K, uin
     const float t_ab = t_whole < t_shares ? t_whole : t_shares;
     const float t_best = t_small < t_ab ? t_small : t_ab;
     bool use_half = t_half < t_best;
+    if (tile == 192) return GemmPlan{GEMM_FORM_192, 0u, 0u};
     if (tile == 256) { use_big = true; use_half = false; }
     if (tile == 128) { use_big = false; use_half = false; }
     if (tile == 129) use_half = true;
     if (split != 0) use_half = use_half && tile == 129;   // a forced split means the 256-tile walk
+    // (e) 256 x 192 tiles where they fill one round over the CUs better than anything above: a k step 1.45 us
+    // (Q4_K) / 1.6 us (Q6_K).  Measured at M = 2048: 6144 x 4096 Q4_K 105 against 108-119 us for 192 whole 256-tiles,
+    // Q5_K 110 against 121-127, Q6_K 113 against 115-118; over several rounds it loses (128256 x 4096 Q6_K 2605
+    // against 2461 us, 28672 x 4096 Q4_K 480 against 445), so it is only priced for a single round.
+    const uint64_t n192 = (uint64_t)((M + 255u) / 256u) * ((N + 191u) / 192u);
+    const float t_192 = (float)nk * (q4 ? 1.45f : q5 ? 1.55f : 1.6f) + te;
+    if (tile == 0 && split == 0 && n192 <= cus && 4u * n192 > 3u * cus && t_192 < (use_half ? t_half : t_best))
+        return GemmPlan{GEMM_FORM_192, 0u, 0u};
     if (use_half) return GemmPlan{GEMM_FORM_HALF, 0u, 0u};
     if (split == 1) share = nk;
     if (split == 2) share = one_per_cu;              // forced: any number of runs per tile

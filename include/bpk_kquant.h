@@ -510,7 +510,8 @@ BPK_API int bpk_force_kernel(int family);
  * lanes-along-K GEMV; "gemv_waves": waves per workgroup of the row-per-lane
  * kernels (2, 4 or 8); "gemv_depth": rows a wave of the lanes-along-K GEMV
  * keeps in flight (1, 2 or 4); "gemm_tile": workgroup tile of the bf16
- * GEMM (128 or 256: square; 129: 256 tokens x 128 weight rows); "gemm_split": how the 256-tile GEMM hands out work
+ * GEMM (128 or 256: square; 129: 256 tokens x 128 weight rows; 192: 256 tokens
+ * x 192 weight rows); "gemm_split": how the 256-tile GEMM hands out work
  * (1 = one tile per workgroup, 2 = the walk over tiles and k steps cut into
  * equal shares per compute unit; the runs of a tile cut between workgroups go
  * through a per-device workspace and are added in the order of the walk, so
@@ -538,7 +539,8 @@ BPK_API int bpk_set_option(const char *name, int value);
  * *form: 0 = 128 x 128 tiles; 1 = 256 x 256 tiles, one workgroup each; 2 = the
  * walk over the 256-tiles' k steps cut into equal shares (*share k steps each);
  * 3 = tiles of 256 tokens x 128 weight rows; 4 = the full rounds of 256-tiles
- * over the first *rows_first weight rows, then the rest as in 3. */
+ * over the first *rows_first weight rows, then the rest as in 3; 5 = tiles of
+ * 256 tokens x 192 weight rows. */
 BPK_API int bpk_gemm_plan(int type, uint32_t M, uint32_t N, uint32_t K, uint32_t compute_units,
                           int *form, uint32_t *share, uint32_t *rows_first);
 

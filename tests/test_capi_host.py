@@ -68,13 +68,14 @@ def test_matmul_argument_validation_needs_no_gpu():
 
 
 # ---- which form of the bf16 dequant-GEMM serves a shape: host arithmetic, pinned on the shapes it was priced on ----
-SMALL, WHOLE, SHARES, HALF, ROUNDS_THEN_HALF = range(5)
+SMALL, WHOLE, SHARES, HALF, ROUNDS_THEN_HALF, N192 = range(6)
 
 
 @pytest.mark.parametrize("name,type_,N,K,M,want", [
     # the Llama-3-8B matrices at 2048 tokens on 256 CUs
     ("gate_up", Q4_K, 28672, 4096, 2048, ROUNDS_THEN_HALF),   # 896 tiles = 3.5 rounds: 3 rounds, then 4096 rows as 256 x 128 tiles
-    ("qkv", Q4_K, 6144, 4096, 2048, WHOLE),                    # 192 tiles, under one round
+    ("qkv", Q4_K, 6144, 4096, 2048, N192),                     # 256 tiles of 256 x 192: one per CU
+    ("qkv", Q4_K, 6144, 4096, 1024, HALF),                     # 128 such tiles would leave half the CUs idle
     ("o", Q4_K, 4096, 4096, 2048, HALF),                       # 256 tiles of 256 x 128: one per CU
     ("down", Q6_K, 4096, 14336, 2048, SHARES),                 # 128 tiles of long K: every tile cut in two
     ("lm_head", Q6_K, 128256, 4096, 2048, WHOLE),              # 4008 tiles; the last round is more than half full
@@ -107,6 +108,8 @@ def test_gemm_plan_follows_the_options_and_refuses_bad_arguments():
         assert capi.gemm_plan(Q4_K, 2048, 28672, 4096)[0] == SMALL
         capi.set_option("gemm_tile", 129)
         assert capi.gemm_plan(Q4_K, 2048, 28672, 4096)[0] == HALF
+        capi.set_option("gemm_tile", 192)
+        assert capi.gemm_plan(Q6_K, 2048, 4096, 14336)[0] == N192
         capi.set_option("gemm_tile", 256)
         capi.set_option("gemm_split", 1)
         assert capi.gemm_plan(Q6_K, 2048, 4096, 14336)[:2] == (WHOLE, 14336 // 64)

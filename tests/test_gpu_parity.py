@@ -534,6 +534,14 @@ GEMM_SHAPES = [
     (Q6_K, 190, 260, 1024, 129),
     (Q6_K, 256, 256, 768, 129),      # odd block count
     (Q6_K, 512, 512, 4096, 129),
+    # 256 tokens x 192 rows per workgroup (option value 192)
+    (Q4_K, 300, 520, 768, 192),
+    (Q4_K, 768, 512, 4096, 192),
+    (Q4_K, 33, 70, 2048, 192),
+    (Q5_K, 300, 580, 1024, 192),
+    (Q6_K, 190, 260, 1024, 192),
+    (Q6_K, 384, 256, 768, 192),      # odd block count
+    (Q6_K, 576, 512, 4096, 192),
 ]
 
 
