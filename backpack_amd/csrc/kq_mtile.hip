@@ -256,6 +256,17 @@ struct MtileStager {
             dst[0] = h;
             dst[HL8 ? 64 : 512] = l;   // the lo operand: 1024 bytes on, or (HL8) slot token + 8
         };
+        // Q6_K: the sum over the 16 elements of group g (its scale's reach) goes out as an A operand too, hi and lo
+        // in one: element g % 8 of lane (token, g / 8) and of lane (token, 2 + g / 8), scaled like the Q4_K sums.
+        // The product with the 16 scales of a weight row is then one matrix instruction per superblock.
+        auto put_half = [&](uint32_t g, float sum) {
+            const float a = sum * (s * 0.03125f);
+            const _Float16 h = (_Float16)a;
+            const _Float16 l = (_Float16)(a - (float)h);
+            _Float16* dst = (_Float16*)(xv + (size_t)bb * 2048u + (token + 16u * (g >> 3)) * 16u) + (g & 7u);
+            dst[0] = h;
+            dst[256] = l;   // 32 lanes on
+        };
         // groups of 8 consecutive k -> one operand slot: halves in the order k+0, k+2, k+1, k+3, k+4, k+6, k+5, k+7
 #pragma unroll
         for (int g8 = 0; g8 < EPT / 8; ++g8) {
@@ -289,8 +300,7 @@ struct MtileStager {
                     h1 += (v[8 * q + 4 + i].x + v[8 * q + 4 + i].y) + (v[8 * q + 4 + i].z + v[8 * q + 4 + i].w);
                 }
                 float* dst = xs + (bb * 8u + (sub * EPT) / 32u + q) * XSR + token;
-                if (SPLIT16) { dst[0] = h0; dst[8] = h1; }
-                else if (HALF) { dst[0] = h0; dst[16] = h1; }
+                if (SPLIT16 || HALF) { put_half(2u * ((sub * EPT) / 32u + q), h0); put_half(2u * ((sub * EPT) / 32u + q) + 1u, h1); }
                 else { if (!HL8) dst[0] = h0 + h1; put_sum((sub * EPT) / 32u + q, h0 + h1); }   // (HL8 reads xv only)
             }
         } else {
@@ -302,10 +312,8 @@ struct MtileStager {
             if (PER16 == 2) h += group_partner<1>(h);
             const uint32_t half = (sub / PER16) & 1u, run = sub / (2u * PER16);
             float* dst = xs + (bb * 8u + run) * XSR + token;
-            if (SPLIT16) {
-                if (sub % PER16 == 0u) dst[8u * half] = h;
-            } else if (HALF) {
-                if (sub % PER16 == 0u) dst[16u * half] = h;
+            if (SPLIT16 || HALF) {
+                if (sub % PER16 == 0u) put_half(2u * run + half, h);
             } else {
                 h += group_partner<PER16>(h);
                 if (sub % (2u * PER16) == 0u) { if (!HL8) dst[0] = h; put_sum(run, h); }
@@ -484,13 +492,35 @@ __device__ __forceinline__ void q6k_mtile_load(const uint8_t* blk, uint32_t kq, 
     w.d = d16;
 }
 
+// The B operand of the product of a superblock's 16 scales with the staged sums of x per group of 16: lane
+// (row, kq) holds the scales of groups 8 * (kq & 1) .. +7 (hi part of the sums for kq < 2, lo part above).  scu:
+// the scale bytes with the sign bit flipped (s + 128); 0x6400 | (s + 128) is the fp16 1024 + 128 + s.
+__device__ __forceinline__ t_half8 q6k_scale_operand(const t_u32x4 scu, uint32_t kq)
+{
+    const uint32_t a = (kq & 1u) ? scu.z : scu.x, b = (kq & 1u) ? scu.w : scu.y;
+    const t_half2 off = {(_Float16)1152.0f, (_Float16)1152.0f};
+    const t_half2 p0 = __builtin_bit_cast(t_half2, __builtin_amdgcn_perm(0x64646464u, a, 0x04010400u)) - off;
+    const t_half2 p1 = __builtin_bit_cast(t_half2, __builtin_amdgcn_perm(0x64646464u, a, 0x04030402u)) - off;
+    const t_half2 p2 = __builtin_bit_cast(t_half2, __builtin_amdgcn_perm(0x64646464u, b, 0x04010400u)) - off;
+    const t_half2 p3 = __builtin_bit_cast(t_half2, __builtin_amdgcn_perm(0x64646464u, b, 0x04030402u)) - off;
+    return t_half8{p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+}
+
 // One superblock of one 16-row tile, Q6_K.  Lanes 0..31 (tq < 2) hold the sums over the first
-// 16 elements of each run of 32 for tokens 4*tq .. +3, lanes 32..63 those over the second 16.
-__device__ __forceinline__ void q6k_mtile_block(const Q6TileW& w, const uint8_t* xa_b, const float* xs_b,
+// 16 elements of each run of 32 for tokens 4*tq .. +3, lanes 32..63 those over the second 16.  The -32 of the
+// 6-bit values: 32 * d * sum over groups of scale * (sum of x over the group), one more matrix instruction
+// (xv_b: those sums as an operand, in the slots of tq < 2 only).
+__device__ __forceinline__ void q6k_mtile_block(const Q6TileW& w, const uint8_t* xa_b, const uint8_t* xv_b,
                                                 const float* xinv_b, uint32_t lane, t_f32x4& tot)
 {
     const uint32_t tq = lane >> 4, u = tq >> 1;
-    t_f32x4 U = {0, 0, 0, 0}, V = {0, 0, 0, 0};
+    const t_u32x4 scu = {w.sc.x ^ 0x80808080u, w.sc.y ^ 0x80808080u, w.sc.z ^ 0x80808080u, w.sc.w ^ 0x80808080u};
+    // this lane's scales are the bytes 2t + u: moved down to the even bytes once
+    const t_u32x4 scl = {scu.x >> (8u * u), scu.y >> (8u * u), scu.z >> (8u * u), scu.w >> (8u * u)};
+    const t_half8 vx = *(const t_half8*)(xv_b + (size_t)lane * 16u);
+    t_f32x4 V = {0, 0, 0, 0};
+    V = __builtin_amdgcn_mfma_f32_16x16x32_f16(vx, q6k_scale_operand(scu, tq), V, 0, 0, 0);
+    t_f32x4 U = {0, 0, 0, 0}, U16 = {0, 0, 0, 0};   // U16: the runs whose fields sit four bits up
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         t_u32x4 bq[4];   // B operands of runs t = 0..3 of this half
@@ -519,35 +549,37 @@ __device__ __forceinline__ void q6k_mtile_block(const Q6TileW& w, const uint8_t*
             t_f32x4 D = {0, 0, 0, 0};
             D = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, b8, D, 0, 0, 0);
             D = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, b8, D, 0, 0, 0);
-            // scale of (half h, t, 16-element half u): byte 8h + 2t + u of the 16
-            const uint32_t word = w.sc[(8 * h + 2 * t) >> 2];
-            const uint32_t sh = 8u * ((2u * t) & 3u) + 8u * u;
-            const float scv = (float)(int)(int8_t)((word >> sh) & 255u);
-            const float sc = scv * (t >= 2 ? 0.0625f : 1.0f);   // t >= 2: the field sits four bits up
-            const float4 xsum = *(const float4*)(xs_b + run * 16 + 4u * tq);
-            U.x = fmaf(sc, D.x, U.x); U.y = fmaf(sc, D.y, U.y); U.z = fmaf(sc, D.z, U.z); U.w = fmaf(sc, D.w, U.w);
-            V.x = fmaf(scv, xsum.x, V.x); V.y = fmaf(scv, xsum.y, V.y); V.z = fmaf(scv, xsum.z, V.z); V.w = fmaf(scv, xsum.w, V.w);
+            // scale of (half h, t, 16-element half u): byte 8h + 2t + u of the 16, now byte 2t of its word
+            const uint32_t word = scl[(8 * h + 2 * t) >> 2];
+            const float sc = (float)((word >> (8 * ((2 * t) & 3))) & 255u) - 128.0f;
+            if (t >= 2) { U16.x = fmaf(sc, D.x, U16.x); U16.y = fmaf(sc, D.y, U16.y); U16.z = fmaf(sc, D.z, U16.z); U16.w = fmaf(sc, D.w, U16.w); }
+            else { U.x = fmaf(sc, D.x, U.x); U.y = fmaf(sc, D.y, U.y); U.z = fmaf(sc, D.z, U.z); U.w = fmaf(sc, D.w, U.w); }
         }
     }
+    // U carries 2^-24 from the subnormal fields and the token's scale s; V carries s / 32
     const float4 inv = *(const float4*)(xinv_b + 4u * tq);
     const float d = half_bits_to_float(w.d);
-    const float d24 = d * 16777216.0f, d32 = d * 32.0f;
-    tot.x += fmaf(d24 * inv.x, U.x, -(d32 * V.x));
-    tot.y += fmaf(d24 * inv.y, U.y, -(d32 * V.y));
-    tot.z += fmaf(d24 * inv.z, U.z, -(d32 * V.z));
-    tot.w += fmaf(d24 * inv.w, U.w, -(d32 * V.w));
+    const float d24 = d * 16777216.0f, d1k = d * 1024.0f;
+    tot.x += inv.x * fmaf(d24, fmaf(0.0625f, U16.x, U.x), -(d1k * V.x));
+    tot.y += inv.y * fmaf(d24, fmaf(0.0625f, U16.y, U.y), -(d1k * V.y));
+    tot.z += inv.z * fmaf(d24, fmaf(0.0625f, U16.z, U.z), -(d1k * V.z));
+    tot.w += inv.w * fmaf(d24, fmaf(0.0625f, U16.w, U.w), -(d1k * V.w));
 }
 
 // Q6_K with 16 tokens: lane l holds tokens 4*(l/16) .. +3 of weight row l%16 as in the Q4_K kernel.  Every run of
 // 32 elements is multiplied whole and with the second half of the weight operand zeroed (the lanes of k >= 16):
 // D1 = sum over the first 16 elements, Dw - D1 = sum over the second, each with its own scale:
-// sc1 * D1 + sc2 * (Dw - D1) = (sc1 - sc2) * D1 + sc2 * Dw.  xs_b holds the sums of x per half run.
-__device__ __forceinline__ void q6k_mtile_block_wide(const Q6TileW& w, const uint8_t* xa_b, const float* xs_b,
+// sc1 * D1 + sc2 * (Dw - D1) = (sc1 - sc2) * D1 + sc2 * Dw.  xv_b: the sums of x per group of 16 as an operand.
+__device__ __forceinline__ void q6k_mtile_block_wide(const Q6TileW& w, const uint8_t* xa_b, const uint8_t* xv_b,
                                                      const float* xinv_b, uint32_t lane, t_f32x4& tot)
 {
     const uint32_t tq = lane >> 4;
     const uint32_t first = tq < 2u ? 0xFFFFFFFFu : 0u;   // this lane's k belong to the first half of a run
-    t_f32x4 U = {0, 0, 0, 0}, V = {0, 0, 0, 0};
+    const t_u32x4 scu = {w.sc.x ^ 0x80808080u, w.sc.y ^ 0x80808080u, w.sc.z ^ 0x80808080u, w.sc.w ^ 0x80808080u};
+    const t_half8 vx = *(const t_half8*)(xv_b + (size_t)lane * 16u);
+    t_f32x4 V = {0, 0, 0, 0};
+    V = __builtin_amdgcn_mfma_f32_16x16x32_f16(vx, q6k_scale_operand(scu, tq), V, 0, 0, 0);
+    t_f32x4 U = {0, 0, 0, 0}, U16 = {0, 0, 0, 0};   // U16: the runs whose fields sit four bits up
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         t_u32x4 bq[4];   // B operands of runs t = 0..3 of this half
@@ -579,28 +611,28 @@ __device__ __forceinline__ void q6k_mtile_block_wide(const Q6TileW& w, const uin
             D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, b18, D1, 0, 0, 0);
             Dw = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bw8, Dw, 0, 0, 0);
             D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, b18, D1, 0, 0, 0);
-            // scales of (half h, t): bytes 8h + 2t (first 16 elements) and 8h + 2t + 1 of the 16
-            const uint32_t word = w.sc[(8 * h + 2 * t) >> 2];
-            const uint32_t sh = 8u * ((2u * t) & 3u);
-            const float sv1 = (float)(int)(int8_t)((word >> sh) & 255u);
-            const float sv2 = (float)(int)(int8_t)((word >> (sh + 8u)) & 255u);
-            const float f = t >= 2 ? 0.0625f : 1.0f;   // t >= 2: the field sits four bits up
-            const float s2 = sv2 * f, s12 = (sv1 - sv2) * f;
-            const float4 x1 = *(const float4*)(xs_b + run * 32 + 4u * tq);
-            const float4 x2 = *(const float4*)(xs_b + run * 32 + 16 + 4u * tq);
-            U.x = fmaf(s12, D1.x, fmaf(s2, Dw.x, U.x)); U.y = fmaf(s12, D1.y, fmaf(s2, Dw.y, U.y));
-            U.z = fmaf(s12, D1.z, fmaf(s2, Dw.z, U.z)); U.w = fmaf(s12, D1.w, fmaf(s2, Dw.w, U.w));
-            V.x = fmaf(sv1, x1.x, fmaf(sv2, x2.x, V.x)); V.y = fmaf(sv1, x1.y, fmaf(sv2, x2.y, V.y));
-            V.z = fmaf(sv1, x1.z, fmaf(sv2, x2.z, V.z)); V.w = fmaf(sv1, x1.w, fmaf(sv2, x2.w, V.w));
+            // scales of (half h, t): bytes 8h + 2t (first 16 elements) and 8h + 2t + 1 of the 16; the 128 added to
+            // both leaves their difference
+            const uint32_t word = scu[(8 * h + 2 * t) >> 2];
+            const int sh = 8 * ((2 * t) & 3);
+            const float u1 = (float)((word >> sh) & 255u), u2 = (float)((word >> (sh + 8)) & 255u);
+            const float s2 = u2 - 128.0f, s12 = u1 - u2;
+            if (t >= 2) {
+                U16.x = fmaf(s12, D1.x, fmaf(s2, Dw.x, U16.x)); U16.y = fmaf(s12, D1.y, fmaf(s2, Dw.y, U16.y));
+                U16.z = fmaf(s12, D1.z, fmaf(s2, Dw.z, U16.z)); U16.w = fmaf(s12, D1.w, fmaf(s2, Dw.w, U16.w));
+            } else {
+                U.x = fmaf(s12, D1.x, fmaf(s2, Dw.x, U.x)); U.y = fmaf(s12, D1.y, fmaf(s2, Dw.y, U.y));
+                U.z = fmaf(s12, D1.z, fmaf(s2, Dw.z, U.z)); U.w = fmaf(s12, D1.w, fmaf(s2, Dw.w, U.w));
+            }
         }
     }
     const float4 inv = *(const float4*)(xinv_b + 4u * tq);
     const float d = half_bits_to_float(w.d);
-    const float d24 = d * 16777216.0f, d32 = d * 32.0f;
-    tot.x += fmaf(d24 * inv.x, U.x, -(d32 * V.x));
-    tot.y += fmaf(d24 * inv.y, U.y, -(d32 * V.y));
-    tot.z += fmaf(d24 * inv.z, U.z, -(d32 * V.z));
-    tot.w += fmaf(d24 * inv.w, U.w, -(d32 * V.w));
+    const float d24 = d * 16777216.0f, d1k = d * 1024.0f;
+    tot.x += inv.x * fmaf(d24, fmaf(0.0625f, U16.x, U.x), -(d1k * V.x));
+    tot.y += inv.y * fmaf(d24, fmaf(0.0625f, U16.y, U.y), -(d1k * V.y));
+    tot.z += inv.z * fmaf(d24, fmaf(0.0625f, U16.z, U.z), -(d1k * V.z));
+    tot.w += inv.w * fmaf(d24, fmaf(0.0625f, U16.w, U.w), -(d1k * V.w));
 }
 
 // Weights travel HBM -> registers -> LDS in 16-byte units that are consecutive along a row, so every cache
@@ -702,7 +734,6 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
     // lanes l and l + 32 hold two addends of the same outputs (Q6_K's 16-element halves, or hi and lo parts)
     constexpr bool HALVES = Q6S || HL8;
     constexpr uint32_t BB = Q6 ? KQ_Q6K_BYTES : Q5 ? KQ_Q5K_BYTES : KQ_Q4K_BYTES;
-    constexpr uint32_t XSB = Q6W ? 256u : 128u;   // floats of xs per superblock
     constexpr uint32_t QOFF = Q5 ? 48u : 16u;   // where the quants start inside a block
     // A wave with a tile of its own stages two superblocks of its 16 rows at a time (two passes per chunk);
     // waves that share a tile stage the one superblock of the chunk that is theirs.
@@ -824,9 +855,9 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
                         Q6TileW w6;
                         q6k_mtile_load(blk, kq, w6);
                         if constexpr (Q6W)
-                            q6k_mtile_block_wide(w6, xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                            q6k_mtile_block_wide(w6, xa + (size_t)bb * (8 * MT_XA_PITCH), xv + (size_t)bb * 2048, xinv + bb * 16, lane, tot);
                         else
-                            q6k_mtile_block(w6, xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                            q6k_mtile_block(w6, xa + (size_t)bb * (8 * MT_XA_PITCH), xv + (size_t)bb * 2048, xinv + bb * 16, lane, tot);
                     } else {
                         const t_u32x4 hdr = *(const t_u32x4*)blk;
                         t_u32x2 w[4], qhw = {0, 0};
@@ -891,9 +922,9 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
                     for (int i = 0; i < BPC; ++i) {
                         if ((uint32_t)i < MT_KC && c_begin + i < c_end) {
                             if constexpr (Q6W)
-                                q6k_mtile_block_wide(cur.w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xs + i * XSB, xinv + i * 16, lane, tt);
+                                q6k_mtile_block_wide(cur.w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xv + (size_t)i * 2048, xinv + i * 16, lane, tt);
                             else if constexpr (Q6)
-                                q6k_mtile_block(cur.w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xs + i * XSB, xinv + i * 16, lane, tt);
+                                q6k_mtile_block(cur.w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xv + (size_t)i * 2048, xinv + i * 16, lane, tt);
                             else
                                 q4k_mtile_block_compact<Q5>(cur.hdr[i], cur.w[i], cur.qhw[i], xa + (size_t)i * (8 * MT_XA_PITCH), xs + i * 128, xinv + i * 16, lane, tt);
                         }
@@ -948,9 +979,9 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
                 const uint32_t bb = R == 1 ? wave + i * NW : i;
                 if (bb < MT_KC && c0 + bb < c_end) {
                     if constexpr (Q6W)
-                        q6k_mtile_block_wide(w6[i], xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                        q6k_mtile_block_wide(w6[i], xa + (size_t)bb * (8 * MT_XA_PITCH), xv + (size_t)bb * 2048, xinv + bb * 16, lane, tot);
                     else if constexpr (Q6)
-                        q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * XSB, xinv + bb * 16, lane, tot);
+                        q6k_mtile_block(w6[i], xa + (size_t)bb * (8 * MT_XA_PITCH), xv + (size_t)bb * 2048, xinv + bb * 16, lane, tot);
                     else
                         q4k_mtile_block_compact<Q5>(hdr[i], w[i], qhw[i], xa + (size_t)bb * (8 * MT_XA_PITCH), xs + bb * 128, xinv + bb * 16, lane, tot);
                 }
