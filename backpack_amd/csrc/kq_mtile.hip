@@ -884,61 +884,43 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
     // with it (no barrier after the first): such workgroups are otherwise mostly set-up.
     const uint32_t iters = (R == NW && p.tiles) ? p.tile_iters : 1u;
     constexpr int BPC = R == 1 ? (MT_KC + NW - 1) / NW : MT_KC;   // superblocks of a chunk this wave takes
-    if constexpr (R == NW && Q6) {   // (the grouped Q4_K kernel is held to 128 registers: no room for a second set)
+    if constexpr (R == NW && Q6) {   // (the grouped Q4_K kernel is held to 128 registers: no room for this)
         if (iters > 1u) {
-            // (iters is 2, 4 or 8.)  The weights of tile it + 1 are requested before tile it is multiplied: two
-            // register sets take turns, no register with a load in flight is copied, and every wait the
-            // compiler places leaves the younger set's loads outstanding.
-            struct TileRegs {
-                t_u32x4 hdr[BPC];
-                t_u32x2 w[BPC][4], qhw[BPC];
-                Q6TileW w6[BPC];
-            };
+            // (iters is 2, 4 or 8.)  One set of weight registers, refilled block by block: as soon as a superblock
+            // of tile it has been multiplied its registers are requested again for tile it + 1, so the loads of a
+            // tile travel under the products of the blocks after them and of the next tile's blocks before them.
+            // A second whole set (the next tile requested at once) took the kernel past 256 registers, to one
+            // wave per SIMD; with this it keeps two workgroups on a CU.
             auto tile_row = [&](uint32_t it) {
                 const uint32_t tile_i = (blockIdx.x * iters + it) * p.tiles_per_wg + wave;
                 return has_tile ? tile_i * 16u + (lane & 15u) : p.N;
             };
-            auto load_tile = [&](uint32_t it, TileRegs& r) {
+            auto block_at = [&](uint32_t it, int i) {   // (past the last tile: that tile again, cache hits, never multiplied)
                 const uint8_t* wrow = wmat + (size_t)min(tile_row(min(it, iters - 1u)), p.N - 1u) * p.row_stride_bytes;
+                return wrow + (size_t)min(c_begin + (uint32_t)i, p.n_blocks - 1u) * BB;
+            };
+            const uint32_t nb = min(c_end - c_begin, (uint32_t)BPC);
+            Q6TileW w6[BPC];
+#pragma unroll
+            for (int i = 0; i < BPC; ++i)
+                if ((uint32_t)i < nb) q6k_mtile_load(block_at(0u, i), kq, w6[i]);
+            stager.park(xa, xs, xinv, xv);
+            __syncthreads();
+            for (uint32_t it = 0; it < iters; ++it) {
+                t_f32x4 tt = {0, 0, 0, 0};
 #pragma unroll
                 for (int i = 0; i < BPC; ++i) {
-                    const uint8_t* blk = wrow + (size_t)min(c_begin + (uint32_t)i, p.n_blocks - 1u) * BB;
-                    if constexpr (Q6) {
-                        q6k_mtile_load(blk, kq, r.w6[i]);
-                    } else {
-                        r.hdr[i] = *(const t_u32x4*)blk;
-#pragma unroll
-                        for (int g = 0; g < 4; ++g) r.w[i][g] = *(const t_u32x2*)(blk + QOFF + 32u * g + 8u * kq);
-                        r.qhw[i] = t_u32x2{0, 0};
-                        if constexpr (Q5) r.qhw[i] = *(const t_u32x2*)(blk + 16u + 8u * kq);
-                    }
-                }
-            };
-            auto run_tile = [&](uint32_t it, TileRegs& cur, TileRegs& nxt) {
-                load_tile(it + 1u, nxt);   // (past the last tile: that tile again, cache hits, never multiplied)
-                t_f32x4 tt = {0, 0, 0, 0};
-                if (has_tile) {
-#pragma unroll
-                    for (int i = 0; i < BPC; ++i) {
-                        if ((uint32_t)i < MT_KC && c_begin + i < c_end) {
+                    if ((uint32_t)i < nb) {
+                        if (has_tile) {
                             if constexpr (Q6W)
-                                q6k_mtile_block_wide(cur.w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xv + (size_t)i * 2048, xinv + i * 16, lane, tt);
-                            else if constexpr (Q6)
-                                q6k_mtile_block(cur.w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xv + (size_t)i * 2048, xinv + i * 16, lane, tt);
+                                q6k_mtile_block_wide(w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xv + (size_t)i * 2048, xinv + i * 16, lane, tt);
                             else
-                                q4k_mtile_block_compact<Q5>(cur.hdr[i], cur.w[i], cur.qhw[i], xa + (size_t)i * (8 * MT_XA_PITCH), xs + i * 128, xinv + i * 16, lane, tt);
+                                q6k_mtile_block(w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xv + (size_t)i * 2048, xinv + i * 16, lane, tt);
                         }
+                        q6k_mtile_load(block_at(it + 1u, i), kq, w6[i]);
                     }
                 }
                 store_tile(tile_row(it), tt);
-            };
-            TileRegs ra, rb;
-            load_tile(0u, ra);
-            stager.park(xa, xs, xinv, xv);
-            __syncthreads();
-            for (uint32_t it = 0; it < iters; it += 2u) {
-                run_tile(it, ra, rb);
-                run_tile(it + 1u, rb, ra);
             }
             return;
         }
@@ -1141,7 +1123,7 @@ struct MtileRest {
 };
 
 template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0, bool HL8 = false>
-__global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : 1) void mtile_kernel(
+__global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : (!STAGED && NW == 4) ? 2 : 1) void mtile_kernel(
     const uint8_t* W, const float* X, const uint32_t* tiles, uint32_t M, uint32_t N, uint32_t K, uint32_t n_blocks,
     uint32_t row_stride_bytes, uint32_t tiles_per_wg, uint32_t chunks_per_split, uint32_t n_splits, uint32_t x_stride,
     MtileRest r)
