@@ -1130,10 +1130,17 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
         const int rsets = wide ? 8 : 4;
         const uint32_t rbound = kq::moe_tiles_bound(P, n_experts, rsets), rcap = 2u * (uint32_t)rsets;
         e = kq::launch_moe_group(expert_idx, P, n_experts, rsets, tiles, n_tiles, s);
-        if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, rbound, rcap, s);
-        a.W = (const uint8_t*)up; a.Y = U;
-        if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, rbound, rcap, s);
-        if (e == hipSuccess) e = kq::launch_moe_silu_mul(G, U, G, (size_t)P * inter, s);
+        a.W2 = (const uint8_t*)up;
+        if (t_moe_fold && kq::mtile_grouped_dual_supported(a)) {
+            // gate and up in one launch that converts the records' X once and stores silu(gate x) * (up x)
+            if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, rbound, rcap, s);
+        } else {
+            a.W2 = nullptr;
+            if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, rbound, rcap, s);
+            a.W = (const uint8_t*)up; a.Y = U;
+            if (e == hipSuccess) e = kq::launch_mtile_grouped(a, tiles, n_tiles, rbound, rcap, s);
+            if (e == hipSuccess) e = kq::launch_moe_silu_mul(G, U, G, (size_t)P * inter, s);
+        }
         if (e == hipSuccess) e = kq::launch_mtile_grouped(d, tiles, n_tiles, rbound, rcap, s);
     } else if (fast) {
         t_kernel = "moe_ffn_mrow";

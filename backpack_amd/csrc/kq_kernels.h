@@ -21,7 +21,8 @@ struct MatmulArgs {
     const uint32_t* expert_idx;
     uint32_t k_slots;
     int x_per_slot;
-    // fusions of the MoE FFN, honoured by the grouped lanes-along-K launch only: a twin matrix W2 of the
+    // fusions of the MoE FFN, honoured by the grouped lanes-along-K launch (and W2 by the grouped tile launch,
+    // which then stores silu(W x) * (W2 x) to Y): a twin matrix W2 of the
     // same shape whose products go to Y2 (gate and up in one launch), and X2: x = silu(X) * X2
     const uint8_t* W2;
     float* Y2;
@@ -133,6 +134,7 @@ uint32_t mtile_group_cap(int type);
 // the fused forms (MatmulArgs pro / residual / epi) on the tile kernel, up to 16 tokens, one launch
 bool mtile_fused_supported(const MatmulArgs& a);
 hipError_t launch_mtile_fused(const MatmulArgs& a, const SplitScratch& sc, hipStream_t s);
+bool mtile_grouped_dual_supported(const MatmulArgs& a);   // a.W2 honoured: Y = silu(W x) * (W2 x)
 hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, const uint32_t* n_tiles,
                                 uint32_t tiles_bound, uint32_t cap, hipStream_t s);
 

@@ -107,6 +107,7 @@ struct MtileParams {
     uint32_t pair_tile0;    // tiles of gate rows (= outputs / 16)
     const uint32_t* tiles;
     const uint32_t* n_tiles;
+    const uint8_t* W2;      // DUAL kernels (grouped calls): a twin matrix (up beside gate); Y = silu(W x) * (W2 x)
     uint32_t tile_iters;    // grouped calls whose K is a single chunk: tiles a wave walks with X staged once
     uint32_t tile_stride;   // words per record
     uint32_t k_slots;
@@ -683,7 +684,7 @@ struct MtileWStage {
 // of two) costs more than the line re-fetches, so they load each lane's pieces straight from global memory.
 // (the grouped Q4_K kernel is held to 128 registers so that two of its workgroups share a CU)
 // FUSED: residual and pair epilogue; PRO: the prologue (1 RMSNorm, 2 act(gate) * up)
-template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0, bool HL8 = false>
+template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0, bool HL8 = false, bool DUAL = false>
 __device__ __forceinline__ void mtile_body(const MtileParams& p)
 // (Q5_K: the Q4_K code with blocks of 176 bytes — header, 32 bytes of fifth bits, quants — and one more
 // 8-byte piece per lane and superblock)
@@ -880,6 +881,77 @@ __device__ __forceinline__ void mtile_body(const MtileParams& p)
     for (uint32_t i = threadIdx.x; i < MT_STAGE_BYTES / 16; i += 64 * NW)
         ((t_u32x4*)smem)[i] = t_u32x4{0, 0, 0, 0};
     __syncthreads();
+    if constexpr (DUAL) {
+        // Gate and up of a routed expert in one walk: a chunk of the record's X is converted once and multiplied
+        // with the wave's tile of W, then with the same tile of W2; one set of weight registers, refilled block by
+        // block with what is multiplied next (W2's blocks of this chunk, then W's of the next), and
+        // silu(W x) * (W2 x) is what gets stored.
+        static_assert(R == NW && !STAGED && !FUSED, "a grouped kernel, a wave per tile");
+        constexpr int NBLK = MT_KC;
+        const uint8_t* wrow_g = wmat + (size_t)min(row, p.N - 1u) * p.row_stride_bytes;
+        const uint8_t* wrow_u = p.W2 + (wrow_g - p.W);
+        t_u32x4 hdr[NBLK];
+        t_u32x2 w[NBLK][4], qhw[NBLK];
+        Q6TileW w6[NBLK];
+        auto load_block = [&](const uint8_t* wrow, uint32_t c0, int i) {
+            const uint8_t* blk = wrow + (size_t)min(c0 + (uint32_t)i, p.n_blocks - 1u) * BB;
+            if constexpr (Q6) {
+                q6k_mtile_load(blk, kq, w6[i]);
+            } else {
+                hdr[i] = *(const t_u32x4*)blk;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) w[i][g] = *(const t_u32x2*)(blk + QOFF + 32u * g + 8u * kq);
+                qhw[i] = t_u32x2{0, 0};
+                if constexpr (Q5) qhw[i] = *(const t_u32x2*)(blk + 16u + 8u * kq);
+            }
+        };
+        auto mul_block = [&](int i, t_f32x4& t) {
+            if constexpr (Q6W)
+                q6k_mtile_block_wide(w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xv + (size_t)i * 2048, xinv + i * 16, lane, t);
+            else if constexpr (Q6)
+                q6k_mtile_block(w6[i], xa + (size_t)i * (8 * MT_XA_PITCH), xv + (size_t)i * 2048, xinv + i * 16, lane, t);
+            else
+                q4k_mtile_block_compact<Q5>(hdr[i], w[i], qhw[i], xa + (size_t)i * (8 * MT_XA_PITCH), xs + i * 128, xinv + i * 16, lane, t);
+        };
+#pragma unroll
+        for (int i = 0; i < NBLK; ++i) load_block(wrow_g, c_begin, i);
+        t_f32x4 tot2 = {0, 0, 0, 0};
+        for (uint32_t c0 = c_begin; c0 < c_end; c0 += MT_KC) {
+            stager.park(xa, xs, xinv, xv);
+            __syncthreads();
+            if (c0 + MT_KC < c_end) stager.fetch(p, c0 + MT_KC);   // the next chunk of X travels while this one is multiplied
+#pragma unroll
+            for (int i = 0; i < NBLK; ++i) {
+                if (has_tile && c0 + i < c_end) mul_block(i, tot);
+                load_block(wrow_u, c0, i);
+            }
+#pragma unroll
+            for (int i = 0; i < NBLK; ++i) {
+                if (has_tile && c0 + i < c_end) mul_block(i, tot2);
+                load_block(wrow_g, c0 + MT_KC, i);   // (past the end: the last block again, never multiplied)
+            }
+            __syncthreads();
+        }
+        if constexpr (HALVES) {   // lanes l and l + 32 hold two addends of the same tokens
+            tot.x += __shfl_xor(tot.x, 32, 64); tot.y += __shfl_xor(tot.y, 32, 64);
+            tot.z += __shfl_xor(tot.z, 32, 64); tot.w += __shfl_xor(tot.w, 32, 64);
+            tot2.x += __shfl_xor(tot2.x, 32, 64); tot2.y += __shfl_xor(tot2.y, 32, 64);
+            tot2.z += __shfl_xor(tot2.z, 32, 64); tot2.w += __shfl_xor(tot2.w, 32, 64);
+        }
+        if (row < p.N && (!HALVES || kq < 2u)) {
+            const float g4[4] = {tot.x, tot.y, tot.z, tot.w}, u4[4] = {tot2.x, tot2.y, tot2.z, tot2.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t token = 4u * kq + r;
+                if (token < count) {
+                    const uint32_t yrow = rec ? rec[2u + token] : token;
+                    // the formula of the separate activation kernel, so that the two ways agree to the bit
+                    p.Y[(size_t)yrow * p.ldy + p.y_offset + row] = g4[r] / (expf(-g4[r]) + 1.0f) * u4[r];
+                }
+            }
+        }
+        return;
+    }
     // A grouped call whose K fits one chunk stages the record's X once and lets every wave walk `iters` tiles
     // with it (no barrier after the first): such workgroups are otherwise mostly set-up.
     const uint32_t iters = (R == NW && p.tiles) ? p.tile_iters : 1u;
@@ -1120,15 +1192,17 @@ struct MtileRest {
     const uint32_t* n_tiles;
     uint32_t tile_iters, tile_stride, k_slots;
     int x_per_slot;
+    const uint8_t* W2;
 };
 
-template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0, bool HL8 = false>
+template <int TYPE, int NW, int R, bool STAGED, int TOK, bool FUSED = false, int PRO = 0, bool HL8 = false, bool DUAL = false>
 __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : (!STAGED && NW == 4) ? 2 : 1) void mtile_kernel(
     const uint8_t* W, const float* X, const uint32_t* tiles, uint32_t M, uint32_t N, uint32_t K, uint32_t n_blocks,
     uint32_t row_stride_bytes, uint32_t tiles_per_wg, uint32_t chunks_per_split, uint32_t n_splits, uint32_t x_stride,
     MtileRest r)
 {
     MtileParams p;
+    p.W2 = nullptr;
     p.X = X; p.W = W; p.bias = r.bias; p.Y = r.Y;
     p.M = M; p.N = N; p.K = K; p.n_blocks = n_blocks; p.row_stride_bytes = row_stride_bytes;
     p.y_offset = r.y_offset; p.ldy = r.ldy;
@@ -1137,8 +1211,8 @@ __global__ __launch_bounds__(64 * NW, (!STAGED && TYPE == KQ_TYPE_Q4_K) ? 4 : (!
     p.pro = r.pro; p.epi = r.epi; p.eps = r.eps; p.norm_w = r.norm_w; p.residual = r.residual;
     p.x_stride = x_stride; p.pair_tile0 = r.pair_tile0;
     p.tiles = tiles; p.n_tiles = r.n_tiles; p.tile_iters = r.tile_iters; p.tile_stride = r.tile_stride;
-    p.k_slots = r.k_slots; p.x_per_slot = r.x_per_slot;
-    mtile_body<TYPE, NW, R, STAGED, TOK, FUSED, PRO, HL8>(p);
+    p.k_slots = r.k_slots; p.x_per_slot = r.x_per_slot; p.W2 = r.W2;
+    mtile_body<TYPE, NW, R, STAGED, TOK, FUSED, PRO, HL8, DUAL>(p);
 }
 
 bool mtile_supported(const MatmulArgs& a)
@@ -1153,7 +1227,7 @@ bool mtile_supported(const MatmulArgs& a)
     return false;
 }
 
-template <int TYPE, int NW, int R, bool STAGED = true, int TOK = 16, bool FUSED = false, int PRO = 0, bool HL8 = false>
+template <int TYPE, int NW, int R, bool STAGED = true, int TOK = 16, bool FUSED = false, int PRO = 0, bool HL8 = false, bool DUAL = false>
 static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t wgs_y, hipStream_t s, uint32_t wgs_z = 1)
 {
     constexpr bool Q6 = TYPE == KQ_TYPE_Q6_K || TYPE == MT_TYPE_Q6K_WIDE, Q5 = TYPE == KQ_TYPE_Q5_K;
@@ -1161,7 +1235,7 @@ static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t 
     // + the sums of squares per token and two chunks of norm weights
     constexpr size_t shmem = MT_STAGE_BYTES + (STAGED ? (size_t)NW * 16 * PITCH : 0) + (FUSED ? 64 : 0) +
                              (PRO == 1 ? 2 * MT_KC * KQ_QK * 4 : 0);
-    auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK, FUSED, PRO, HL8>;
+    auto kern = mtile_kernel<TYPE, NW, R, STAGED, TOK, FUSED, PRO, HL8, DUAL>;
     static bool raised = false;   // per instantiation
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -1169,13 +1243,20 @@ static hipError_t launch_mtile_one(const MtileParams& p, uint32_t wgs, uint32_t 
         raised = true;
     }
     const MtileRest r{p.bias, p.Y, p.y_offset, p.ldy, p.partial, p.counters, p.pro, p.epi, p.eps, p.norm_w, p.residual,
-                      p.pair_tile0, p.n_tiles, p.tile_iters, p.tile_stride, p.k_slots, p.x_per_slot};
+                      p.pair_tile0, p.n_tiles, p.tile_iters, p.tile_stride, p.k_slots, p.x_per_slot, p.W2};
     hipLaunchKernelGGL(kern, dim3(wgs, wgs_y, wgs_z), dim3(64 * NW), shmem, s, p.W, p.X, p.tiles, p.M, p.N, p.K, p.n_blocks,
                        p.row_stride_bytes, p.tiles_per_wg, p.chunks_per_split, p.n_splits, p.x_stride, r);
     return hipGetLastError();
 }
 
 uint32_t mtile_group_cap(int) { return 16u; }
+
+// The grouped call can take a twin matrix W2 (a.W2) and store silu(W x) * (W2 x): where K spans more than one chunk
+// of four superblocks (a single chunk runs the form that walks several tiles per wave with X staged once).
+bool mtile_grouped_dual_supported(const MatmulArgs& a)
+{
+    return mtile_supported(a) && a.n_blocks > (uint32_t)MT_KC && !(((uintptr_t)a.W2) & (a.type == KQ_TYPE_Q6_K ? 1u : 15u));
+}
 
 hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, const uint32_t* n_tiles,
                                 uint32_t tiles_bound, uint32_t cap, hipStream_t s)
@@ -1185,6 +1266,7 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
     const uint32_t slices = 1;
     if (cap == 0 || cap > 16u || tiles_bound == 0 || tiles_bound > 65535u) return hipErrorInvalidValue;
     MtileParams p;
+    p.W2 = nullptr;
     p.X = (const float*)a.X;
     p.W = a.W;
     p.bias = nullptr;
@@ -1196,6 +1278,7 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
     p.ldy = a.ldy;
     p.tiles = tiles;
     p.n_tiles = n_tiles;
+    p.W2 = nullptr;
     p.tile_stride = 2u + cap;
     p.n_splits = 1; p.chunks_per_split = (a.n_blocks + MT_KC - 1) / MT_KC; p.partial = nullptr; p.counters = nullptr;
     p.k_slots = a.k_slots;
@@ -1215,6 +1298,15 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
         p.tile_iters = groups >= 32u ? 8u : groups >= 16u ? 4u : groups >= 8u ? 2u : 1u;
     }
     const uint32_t wgs = (row_tiles + tpw * p.tile_iters - 1u) / (tpw * p.tile_iters);
+    if (a.W2) {
+        // gate and up in one walk, the activation in its store (several chunks of K: see mtile_grouped_dual_supported)
+        if (!mtile_grouped_dual_supported(a)) return hipErrorInvalidValue;
+        p.W2 = a.W2;
+        if (q6_wide) return launch_mtile_one<MT_TYPE_Q6K_WIDE, 4, 4, false, 16, false, 0, false, true>(p, wgs, tiles_bound, s, slices);
+        if (a.type == KQ_TYPE_Q6_K) return launch_mtile_one<KQ_TYPE_Q6_K, 4, 4, false, 16, false, 0, false, true>(p, wgs, tiles_bound, s, slices);
+        if (a.type == KQ_TYPE_Q5_K) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, false, 16, false, 0, false, true>(p, wgs, tiles_bound, s, slices);
+        return launch_mtile_one<KQ_TYPE_Q4_K, 8, 8, false, 16, false, 0, false, true>(p, wgs, tiles_bound, s, slices);
+    }
     if (q6_wide) return launch_mtile_one<MT_TYPE_Q6K_WIDE, 4, 4, false>(p, wgs, tiles_bound, s, slices);
     if (a.type == KQ_TYPE_Q6_K) return launch_mtile_one<KQ_TYPE_Q6_K, 4, 4, false>(p, wgs, tiles_bound, s, slices);
     if (a.type == KQ_TYPE_Q5_K) return launch_mtile_one<KQ_TYPE_Q5_K, 8, 8, false>(p, wgs, tiles_bound, s, slices);
@@ -1256,6 +1348,7 @@ hipError_t launch_mtile(const MatmulArgs& a, const SplitScratch& sc, hipStream_t
 
     for (uint32_t m0 = 0; m0 < a.M; m0 += group) {
         MtileParams p;
+        p.W2 = nullptr;
         p.X = (const float*)a.X + (size_t)m0 * a.K;
         p.W = a.W;
         p.bias = a.bias;
@@ -1337,6 +1430,7 @@ hipError_t launch_mtile_fused(const MatmulArgs& a, const SplitScratch& sc, hipSt
         }
     }
     MtileParams p;
+    p.W2 = nullptr;
     p.X = (const float*)a.X;
     p.W = a.W;
     p.bias = a.bias;

@@ -522,7 +522,10 @@ BPK_API int bpk_force_kernel(int family);
  * 2 from 16384 rows on (gate|up: level on most parts, ahead where the clock runs low);
  * "moe_fold": 0 keeps the weighted sum over a token's slots behind the expert FFN
  * a launch of its own (default 1: inside the last matvec's launch where its
- * kernel can: a few pairs, Q6_K down projection, at most 8 slots per token);
+ * kernel can: a few pairs, Q6_K down projection, at most 8 slots per token),
+ * and the batched tile path's gate and up two launches and an activation
+ * kernel (default: one launch that stores silu(gate x) * (up x), where hidden
+ * spans more than four superblocks);
  * "chain_spin_us": bound of a wait between the ops of a chain in microseconds
  * (at most ten seconds);
  * "chain_hold" (test hook, refused unless chain_spin_us is 1..100000): 1 keeps

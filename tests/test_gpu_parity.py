@@ -751,6 +751,34 @@ def test_moe_ffn_slot_sum_inside_the_last_matvec(gpu, kqo, T, E, k, H, I):
     assert np.abs(got[1] - got[0]).max() <= 1e-5 * rms
 
 
+@pytest.mark.parametrize("tgu,T,E,k,H,I", [(Q4_K, 40, 8, 2, 2048, 512), (Q4_K, 33, 4, 3, 1280, 512), (Q5_K, 24, 4, 2, 1536, 256),
+                                           (Q6_K, 40, 8, 2, 2048, 256), (Q6_K, 10, 8, 2, 1280, 256)])
+def test_moe_ffn_gate_and_up_in_one_tile_launch(gpu, kqo, tgu, T, E, k, H, I):
+    """Batches of pairs on the tile kernel, hidden of more than one chunk of four superblocks: gate and up are
+    walked in one launch that stores silu(gate x) * (up x) (option moe_fold 0: two launches and the activation
+    kernel).  The same products in the same order and the same activation formula: equal bits; and the oracle."""
+    from backpack_amd import capi, kquant
+    _say("moe dual", tgu, T, E, k, H, I)
+    _, gp, gw = gpu.make_weight(tgu, E * I, H, seed=71)
+    _, up, uw = gpu.make_weight(tgu, E * I, H, seed=72)
+    _, dp, dw = gpu.make_weight(Q6_K, E * H, I, seed=73)
+    rng = np.random.default_rng(T * 5 + k)
+    eidx, ew = _routing(rng, T, E, k)
+    X = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
+    got = {}
+    try:
+        for fold in (1, 0):
+            capi.set_option("moe_fold", fold)
+            got[fold] = kquant.moe_ffn(gpu.dev(X), gw, uw, dw, gpu.dev(eidx.view(np.int32)), gpu.dev(ew), E).cpu().numpy()
+            assert capi.last_kernel() == "moe_ffn_mtile"
+    finally:
+        capi.set_option("moe_fold", 1)
+    want = kqo.moe_ffn(tgu, Q6_K, X, gp, up, dp, eidx, ew, H, I)
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    assert np.all(np.abs(got[1] - want) <= 1e-3 * rms + 1e-3 * np.abs(want))
+    assert np.array_equal(got[1], got[0])
+
+
 @pytest.mark.parametrize("family,kernel", [(0, "mtile_grouped"), (3, "mrow_grouped")])
 @pytest.mark.parametrize("type_,N,K,per_slot", [(Q4_K, 768, 2048, False), (Q6_K, 2048, 768, True),
                                                  # K of one chunk: waves walk several tiles per staged X; ragged last tile
