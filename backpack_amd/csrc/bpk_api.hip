@@ -1102,10 +1102,13 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
                       kq::mrow_supported(d);
     hipError_t e = hipSuccess;
     const uint32_t bound8 = kq::moe_tiles_bound(P, n_experts, 4);
-    const bool dense = (uint64_t)P >= 2ull * n_experts;
+    // Pairs per expert from which the tile kernel's records (every touched expert's matrices read once per record
+    // of pairs) beat one lanes-along-K matvec per pair.  Measured on 128 experts x 8 slots, 2048 / 768: 128 pairs 119
+    // against 104 us, 160 pairs 142 against 150-159, 192 pairs 145 against 179.
+    const bool dense = 4ull * P >= 5ull * n_experts;
     const bool tile_ok = (t_family == 0 || t_family == 6) && n_experts <= 8192u && bound8 <= 65535u && inter >= 128u &&
                          hidden >= 128u && kq::mtile_supported(a) && kq::mtile_supported(d);
-    const bool stream_path = (t_family == 0 || t_family == 5) && !(tile_ok && dense) && P <= 64u &&
+    const bool stream_path = (t_family == 0 || t_family == 5) && !(tile_ok && dense) && P <= 256u &&
                              kq::gemv_stream_supported(a) && kq::gemv_stream_supported(d);
     // (Q5_K has no matrix-core row kernel: its thinly spread pairs take the tile kernel too)
     const bool tile_path = tile_ok && !stream_path && (dense || !fast);

@@ -529,10 +529,14 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
 
 // Workgroup = KW waves, one K slice of 8*P superblocks each; the workgroup walks
 // rows blockIdx.x, + gridDim.x, ...; D rows in flight per wave.
-template <int P, int KW, int D, int MT, typename PT>
+// RW = 2 (combining launches, rows of at most four superblocks): the two halves of a wave take two rows at a
+// time, four superblocks of eight lanes each, so that a row of three superblocks keeps 48 of the 64 lanes busy
+// instead of 24; a step's two sums are those of the halves.
+template <int P, int KW, int D, int MT, typename PT, int RW = 1>
 __device__ __forceinline__ void q6k_stream_body(PT p)
 {
     constexpr bool COMBINE = PT::kCombine;   // the waves are a token's slots, not K slices
+    static_assert(RW == 1 || (RW == 2 && COMBINE && P == 1 && MT == 1), "two rows per step: the combining launch");
     __shared__ float part[KW > 1 ? KW : 1][MT][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -543,8 +547,14 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
     const uint32_t kslice = COMBINE ? 0u : wave;
     const uint32_t g = blockIdx.x, stride = stream_grid_x(p);
     const uint32_t n_rows = g < p.N ? (p.N - g + stride - 1u) / stride : 0u;
-    const uint32_t bl = lane >> 3, t = lane & 7u, n = t >> 2, lg = t & 3u;
+    const uint32_t bl = RW == 2 ? (lane >> 3) & 3u : lane >> 3, t = lane & 7u, n = t >> 2, lg = t & 3u;
+    const uint32_t rsel = RW == 2 ? lane >> 5 : 0u;   // which of a step's rows this half of the wave takes
     const uint32_t sc_shift = 8u * (lg >> 1);
+    // row of this workgroup's walk that the lane takes in step j (clamped to the last: fetched, never stored)
+    auto row_ptr = [&](uint32_t j) {
+        const uint32_t ri = min(RW == 2 ? 2u * j + rsel : j, n_rows - 1u);
+        return p.W + (size_t)(g + ri * stride) * p.row_stride_bytes;
+    };
 
     float x[P][MT][4][8], m32xs[P][MT][4];
     uint32_t boff[P];
@@ -627,8 +637,7 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
         for (int tk = 0; tk < MT; ++tk)
             asm volatile("" : "+v"(m32xs[pass][tk][0]), "+v"(m32xs[pass][tk][1]), "+v"(m32xs[pass][tk][2]), "+v"(m32xs[pass][tk][3]));
 #pragma unroll
-    for (int d = 0; d < D; ++d)
-        ring[d].fill(p.W + (size_t)(g + min((uint32_t)d, n_rows - 1u) * stride) * p.row_stride_bytes, boff, n, lg);
+    for (int d = 0; d < D; ++d) ring[d].fill(row_ptr((uint32_t)d), boff, n, lg);
     stream_touch_late_args(p);
     // Rows are taken 64 at a time: lane i keeps the sums of the chunk's row i; the K
     // slices are folded and the chunk stored after its last row.  The row loop is
@@ -638,10 +647,10 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
         float res[MT];
 #pragma unroll
         for (int tk = 0; tk < MT; ++tk) res[tk] = 0.0f;
-        for (uint32_t i0 = 0; i0 < cnt; i0 += D) {
+        for (uint32_t i0 = 0; RW * i0 < cnt; i0 += D) {
 #pragma unroll
             for (int d = 0; d < D; ++d) {
-                const uint32_t i = i0 + d;
+                const uint32_t i = i0 + d;   // step of the chunk: row i, or (RW = 2) rows 2i and 2i + 1
                 ring[d].template wait<(D - 1) * SLOT_LOADS>();
                 float acc[MT];
 #pragma unroll
@@ -649,11 +658,21 @@ __device__ __forceinline__ void q6k_stream_body(PT p)
 #pragma unroll
                 for (int pass = 0; pass < P; ++pass)
                     q6k_piece_dot<MT>(ring[d].v[pass], x[pass], m32xs[pass], sc_shift, acc);
-                ring[d].fill(p.W + (size_t)(g + min(c0 + i + D, n_rows - 1u) * stride) * p.row_stride_bytes, boff, n, lg);
+                ring[d].fill(row_ptr(c0 / RW + i + D), boff, n, lg);
+                if constexpr (RW == 2) {
+                    float v = acc[0];
+                    v += group_partner<1>(v); v += group_partner<2>(v); v += group_partner<4>(v); v += group_partner<8>(v);
+                    const float q0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+                    const float q1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+                    const float q2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+                    const float q3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+                    res[0] = lane == 2u * i ? q0 + q1 : lane == 2u * i + 1u ? q2 + q3 : res[0];   // (rows past cnt are not stored)
+                } else {
 #pragma unroll
-                for (int tk = 0; tk < MT; ++tk) {
-                    const float tot = wave_sum(acc[tk]);
-                    res[tk] = (lane == i && i < cnt) ? tot : res[tk];
+                    for (int tk = 0; tk < MT; ++tk) {
+                        const float tot = wave_sum(acc[tk]);
+                        res[tk] = (lane == i && i < cnt) ? tot : res[tk];
+                    }
                 }
             }
         }
@@ -730,10 +749,10 @@ __global__ __launch_bounds__(64 * NW * KW) void q4k_stream_dense_kernel(KQ_DENSE
 {
     q4k_stream_body<P, NW, D, MT, StreamDense, Q5, KW>(KQ_DENSE_STRUCT);
 }
-template <int P, int KW, int D, int MT, typename PT>
+template <int P, int KW, int D, int MT, typename PT, int RW = 1>
 __global__ __launch_bounds__(64 * KW) void q6k_stream_kernel(PT p)
 {
-    q6k_stream_body<P, KW, D, MT, PT>(p);
+    q6k_stream_body<P, KW, D, MT, PT, RW>(p);
 }
 template <int P, int KW, int D, int MT>
 __global__ __launch_bounds__(64 * KW) void q6k_stream_dense_kernel(KQ_DENSE_PARAMS)
@@ -762,10 +781,12 @@ static void launch_q4k_entry(dim3 grid, dim3 block, hipStream_t s, const PT& p)
         hipLaunchKernelGGL((q4k_stream_kernel<P, NW, D, MT, PT, Q5, KW>), grid, block, shmem, s, p);
     }
 }
-template <int P, int KW, int D, int MT, typename PT>
+template <int P, int KW, int D, int MT, typename PT, int RW = 1>
 static void launch_q6k_entry(dim3 grid, dim3 block, hipStream_t s, const PT& p)
 {
-    if constexpr (std::is_same<PT, StreamDense>::value)
+    if constexpr (RW != 1)
+        hipLaunchKernelGGL((q6k_stream_kernel<P, KW, D, MT, PT, RW>), grid, block, 0, s, p);
+    else if constexpr (std::is_same<PT, StreamDense>::value)
         hipLaunchKernelGGL((q6k_stream_dense_kernel<P, KW, D, MT>), grid, block, 0, s, KQ_DENSE_ARGS(p, grid.x));
     else if constexpr (std::is_same<PT, StreamFused>::value)
         hipLaunchKernelGGL((q6k_stream_fused_kernel<P, KW, D, MT>), grid, block, 0, s, KQ_FUSED_ARGS(p, grid.x));
@@ -949,6 +970,9 @@ static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, h
                                 : stream_workgroups((a.N + NW - 1u) / NW, 1u, 0);
     wgs = (wgs + pairs * twins - 1u) / (pairs * twins);
     if (PT::kGrouped) wgs *= 2u;   // (as for Q6_K above)
+    // ... and at least 512 workgroups in the launch, while a wave keeps four rows (a 128-expert layer of 768 x 2048
+    // matrices: 2 tokens x 8 slots 27.7 -> 25.0 us for the layer, 8 tokens 63.6 -> 59.1, 10 tokens 97 -> 88)
+    if (PT::kGrouped) wgs = max(wgs, min((512u + pairs * twins - 1u) / (pairs * twins), (a.N + 4u * NW - 1u) / (4u * NW)));
     int depth = t.depth > 0 ? t.depth : (a.N + wgs * NW - 1u) / (wgs * NW) <= 8u ? 2 : 4;
     if (q5 && depth > 2) depth = 2;
     if (PT::kFused) depth = depth >= 4 && !two ? 4 : 2;   // the fused forms come with two or four rows in flight
@@ -1025,11 +1049,14 @@ hipError_t launch_stream_combine(const MatmulArgs& a, const float* wt, float* ou
     // other tokens', twice over.  (Measured on a 128-expert layer, 8 slots, 2048 x 768, one token: 18.5-19.0 us for
     // the layer against 18.9-19.5 with the sum as a launch of its own; four rows in flight, or fewer rows per
     // workgroup, are slower.)
+    // (Rounded down: two workgroups of eight waves fill a CU, and a launch of a few more than twice the CU count —
+    // 3 tokens x 172 — ran its last four alone: 27.3 us against 24.6 for 4 tokens x 128.)
     uint32_t wgs = stream_workgroups(a.N, 1u, t.splits);
-    wgs = (wgs + tokens - 1u) / tokens;
-    if (t.splits == 0) wgs *= 2u;
+    if (t.splits == 0) wgs = max(1u, 2u * wgs / tokens);
+    else wgs = (wgs + tokens - 1u) / tokens;
     const dim3 grid(wgs, tokens, 1);
-    if (a.n_blocks <= 8u) launch_q6k_entry<1, 8, 2, 1>(grid, dim3(512), s, p);
+    if (a.n_blocks <= 4u) launch_q6k_entry<1, 8, 2, 1, StreamCombine, 2>(grid, dim3(512), s, p);   // two rows per step
+    else if (a.n_blocks <= 8u) launch_q6k_entry<1, 8, 2, 1>(grid, dim3(512), s, p);
     else launch_q6k_entry<2, 8, 2, 1>(grid, dim3(512), s, p);
     return hipGetLastError();
 }
