@@ -1045,14 +1045,13 @@ hipError_t launch_stream_combine(const MatmulArgs& a, const float* wt, float* ou
     p.wt = wt;
     p.Y = out;
     p.M = a.k_slots;
-    // as many waves as the grouped launch would start: the workgroups of one token share the machine with the
-    // other tokens', twice over.  (Measured on a 128-expert layer, 8 slots, 2048 x 768, one token: 18.5-19.0 us for
-    // the layer against 18.9-19.5 with the sum as a launch of its own; four rows in flight, or fewer rows per
-    // workgroup, are slower.)
-    // (Rounded down: two workgroups of eight waves fill a CU, and a launch of a few more than twice the CU count —
-    // 3 tokens x 172 — ran its last four alone: 27.3 us against 24.6 for 4 tokens x 128.)
+    // One workgroup per CU over all tokens (rounded down: a few workgroups more than fit at once run alone at the
+    // end).  Measured on a 128-expert layer, 8 slots, 2048 x 768, with the two-rows form: one token 15.9-16.5 us
+    // for the layer against 18.2 with twice and 26.8 with four times the workgroups (every workgroup loads its
+    // slots' activations again: at four rows per wave they outweigh the weights), 17.1 with half; two tokens 19.2
+    // against 22.2; 16 tokens 83-85 against 86, 93 at three quarters.
     uint32_t wgs = stream_workgroups(a.N, 1u, t.splits);
-    if (t.splits == 0) wgs = max(1u, 2u * wgs / tokens);
+    if (t.splits == 0) wgs = max(1u, wgs / tokens);
     else wgs = (wgs + tokens - 1u) / tokens;
     const dim3 grid(wgs, tokens, 1);
     if (a.n_blocks <= 4u) launch_q6k_entry<1, 8, 2, 1, StreamCombine, 2>(grid, dim3(512), s, p);   // two rows per step

@@ -576,7 +576,7 @@ def verify_leg(mats, wb, use_graph):
         sec, _ = run_region(ms, 10, 2, use_graph)
         act = sum((w.K + w.N) * 4 * M for _, w, _, _ in ms)
         res[f"M{M}"] = {"ms_per_step": round(sec / 10 * 1e3, 4), "GBps": round((wb + act) / (sec / 10) / 1e9, 1),
-                        "kernel": capi.last_kernel()}
+                        "kernel": ffn_kernel}
     return res
 
 
@@ -615,6 +615,7 @@ def moe_leg():
         e1.record()
         torch.cuda.synchronize()
         sec = e0.elapsed_time(e1) * 1e-3 / (reps * len(layers))
+        ffn_kernel = capi.last_kernel()
         nbytes = touched * per_expert
         flops = 2.0 * T * k * 3 * H * I
         # the router stage in front of it: fp32 router matvec + top-k softmax, timed in a replayed graph
