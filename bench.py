@@ -576,7 +576,7 @@ def verify_leg(mats, wb, use_graph):
         sec, _ = run_region(ms, 10, 2, use_graph)
         act = sum((w.K + w.N) * 4 * M for _, w, _, _ in ms)
         res[f"M{M}"] = {"ms_per_step": round(sec / 10 * 1e3, 4), "GBps": round((wb + act) / (sec / 10) / 1e9, 1),
-                        "kernel": ffn_kernel}
+                        "kernel": capi.last_kernel()}
     return res
 
 
@@ -645,7 +645,7 @@ def moe_leg():
         res[f"T{T}"] = {"us_per_layer": round(sec * 1e6, 2), "route_us": round(route_us, 2),
                         "experts_touched": touched, "weight_bytes": nbytes,
                         "GBps": round(nbytes / sec / 1e9, 1), "TFLOPs": round(flops / sec / 1e12, 2),
-                        "kernel": capi.last_kernel()}
+                        "kernel": ffn_kernel}
     return res
 
 
