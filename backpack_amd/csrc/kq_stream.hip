@@ -529,14 +529,15 @@ __device__ __forceinline__ void q4k_stream_body(PT p)
 
 // Workgroup = KW waves, one K slice of 8*P superblocks each; the workgroup walks
 // rows blockIdx.x, + gridDim.x, ...; D rows in flight per wave.
-// RW = 2 (combining launches, rows of at most four superblocks): the two halves of a wave take two rows at a
+// RW = 2 (combining and grouped launches, rows of at most four superblocks): the two halves of a wave take two rows at a
 // time, four superblocks of eight lanes each, so that a row of three superblocks keeps 48 of the 64 lanes busy
 // instead of 24; a step's two sums are those of the halves.
 template <int P, int KW, int D, int MT, typename PT, int RW = 1>
 __device__ __forceinline__ void q6k_stream_body(PT p)
 {
     constexpr bool COMBINE = PT::kCombine;   // the waves are a token's slots, not K slices
-    static_assert(RW == 1 || (RW == 2 && COMBINE && P == 1 && MT == 1), "two rows per step: the combining launch");
+    static_assert(RW == 1 || (RW == 2 && (COMBINE || (PT::kGrouped && KW == 1)) && P == 1 && MT == 1),
+                  "two rows per step: the combining launch, or a grouped one whose rows one wave walks");
     __shared__ float part[KW > 1 ? KW : 1][MT][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -934,6 +935,12 @@ static hipError_t launch_stream_with(const MatmulArgs& a, const GemvTuning& t, h
         if (two) KQ_STREAM6_MT(P, KW, 2); \
         else KQ_STREAM6_MT(P, KW, 1); \
     } while (0)
+        if constexpr (PT::kGrouped) {
+            if (nb <= 4u) {   // short rows (an expert's down projection): two rows per step, see q6k_stream_body
+                launch_q6k_entry<1, 1, 2, 1, PT, 2>(grid, dim3(64), s, p);
+                return hipGetLastError();
+            }
+        }
         if (kw == 1 && pp == 1) KQ_STREAM6(1, 1);
         else if (kw == 1) KQ_STREAM6(2, 1);
         else if (kw == 4) KQ_STREAM6(1, 4);
