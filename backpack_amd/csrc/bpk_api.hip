@@ -32,6 +32,7 @@ thread_local int t_family = 0;
 thread_local kq::GemvTuning t_gemv;
 thread_local int t_gemm_tile = 0;
 thread_local int t_gemm_split = 0;
+thread_local int t_moe_tile_iters = 0; // option "moe_tile_iters": tiles a wave of the grouped tile kernel walks per staged X (0: chosen per call)
 thread_local bool t_moe_fold = true;    // option "moe_fold": the slots' weighted sum inside the last matvec where its kernel can
 thread_local int t_fused_separate = 0;
 thread_local int t_chain_spin_us = 0;    // 0 = default
@@ -231,6 +232,11 @@ int bpk_set_option(const char* name, int value)
     }
     if (!strcmp(name, "chain_hold")) {
         t_chain_hold = value != 0;
+        return BPK_OK;
+    }
+    if (!strcmp(name, "moe_tile_iters")) {
+        if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8) return fail(BPK_ERR_SHAPE, "moe_tile_iters must be 0, 1, 2, 4 or 8");
+        t_moe_tile_iters = value;
         return BPK_OK;
     }
     if (!strcmp(name, "moe_fold")) {
@@ -1098,6 +1104,7 @@ int bpk_kq_moe_ffn(int type_gu, int type_dn, const float* X, const void* gate, c
     d.type = type_dn; d.X = G; d.W = (const uint8_t*)down; d.Y = D;
     d.M = P; d.N = hidden; d.K = inter; d.n_blocks = nb_dn; d.row_stride_bytes = rs_dn * 4u; d.ldy = hidden;
     d.expert_idx = expert_idx; d.k_slots = k; d.x_per_slot = 1;
+    a.tile_iters = d.tile_iters = (uint32_t)t_moe_tile_iters;
     const bool fast = t_family != 1 && n_experts <= 8192u && bound <= 65535u && kq::mrow_supported(a) &&
                       kq::mrow_supported(d);
     hipError_t e = hipSuccess;

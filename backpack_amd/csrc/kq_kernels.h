@@ -27,6 +27,7 @@ struct MatmulArgs {
     const uint8_t* W2;
     float* Y2;
     const float* X2;
+    uint32_t tile_iters;   // grouped tile launch of one chunk of K: tiles a wave walks with X staged once (0: chosen by the launcher)
     // fused forms of the dense decode matvec, honoured by the lanes-along-K launch only (other launches
     // must be given pro == 0 and residual == nullptr): pro 1 = RMSNorm of the X row with weight norm_w,
     // 2 / 3 = X rows are gate | up (2K floats) and x = silu / gelu_tanh (gate) * up; residual is added to
@@ -151,6 +152,7 @@ uint32_t moe_tiles_bound(uint32_t n_pairs, uint32_t n_experts, int sets);
 size_t moe_tiles_words(uint32_t n_pairs, uint32_t n_experts, int sets);
 hipError_t launch_moe_group(const uint32_t* expert_idx, uint32_t n_pairs, uint32_t n_experts, int sets, uint32_t* tiles,
                             uint32_t* n_tiles, hipStream_t s);
+double moe_expected_records(uint32_t n_pairs, uint32_t n_experts, uint32_t cap);
 hipError_t launch_moe_silu_mul(const float* gate, const float* up, float* act, size_t n, hipStream_t s);
 hipError_t launch_moe_combine(const float* down, const float* wt, float* out, uint32_t T, uint32_t k, uint32_t hidden,
                               hipStream_t s);

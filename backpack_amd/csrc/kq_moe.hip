@@ -8,6 +8,7 @@
 // grid.z slice of the row kernel, so an expert's rows are streamed once per
 // tile and shared by its pairs.  Nothing returns to the host: tile count and
 // contents stay in device memory and surplus grid slices exit at once.
+#include <cmath>
 #include "kq_format.h"
 #include "kq_kernels.h"
 
@@ -147,6 +148,23 @@ uint32_t moe_tiles_bound(uint32_t n_pairs, uint32_t n_experts, int sets)
     const uint32_t cap = 2u * (uint32_t)sets;
     const uint32_t a = n_pairs / cap + n_experts;   // every expert can add one partial tile
     return a < n_pairs ? a : n_pairs;
+}
+
+// Records that n_pairs pairs spread evenly (independently) over n_experts experts are expected to make at cap
+// pairs per record: n_experts * E[ceil(n / cap)] for n ~ Poisson(n_pairs / n_experts).  Host arithmetic for launch
+// shapes only; the device counts the real ones.
+double moe_expected_records(uint32_t n_pairs, uint32_t n_experts, uint32_t cap)
+{
+    if (n_experts == 0u || cap == 0u) return 0.0;
+    const double lambda = (double)n_pairs / (double)n_experts;
+    if (lambda > 500.0) return (double)n_experts * (lambda / (double)cap + 0.5);
+    double pmf = std::exp(-lambda), sum = 0.0;
+    const uint32_t top = (uint32_t)(lambda + 12.0 * std::sqrt(lambda) + 24.0);
+    for (uint32_t n = 1; n <= top; ++n) {
+        pmf *= lambda / (double)n;
+        sum += pmf * (double)((n + cap - 1u) / cap);
+    }
+    return (double)n_experts * sum;
 }
 
 size_t moe_tiles_words(uint32_t n_pairs, uint32_t n_experts, int sets)

@@ -41,6 +41,8 @@
 // owns a tile and walks all of K; with R = 1 (matrices of few rows) the waves of
 // the workgroup take different superblocks of the chunk and fold their partial
 // tiles through LDS at the end.  There is no fold across workgroups.
+#include <cmath>
+
 #include "kq_format.h"
 #include "kq_kernels.h"
 #include "kq_wave.h"
@@ -1296,6 +1298,25 @@ hipError_t launch_mtile_grouped(const MatmulArgs& a, const uint32_t* tiles, cons
     if (p.chunks_per_split == 1u) {
         const uint32_t groups = (row_tiles + tpw - 1u) / tpw;
         p.tile_iters = groups >= 32u ? 8u : groups >= 16u ? 4u : groups >= 8u ? 2u : 1u;
+        // ... and as long as the launch's workgroups fill whole rounds over the two a CU holds at once: the record
+        // count is only known on the device, so it is estimated for pairs spread evenly over the experts, and a
+        // workgroup is priced at 1.2 tiles for its conversion of X plus the tiles a wave walks.  (128 experts,
+        // 2048 x 768: 2048 pairs are about 186 records; walking 8 tiles these are 744 workgroups on 512 places,
+        // 115 us, walking 4 they are 1488, 103 us; 1024 pairs, 128 records, 512 workgroups: 8 tiles lead by 7 us.)
+        if (a.tile_iters) p.tile_iters = min(p.tile_iters, a.tile_iters);
+        else if (tiles_bound < a.M) {   // (the bound is pairs / cap + experts)
+            const double records = moe_expected_records(a.M, tiles_bound - a.M / cap, cap);
+            const double places = 2.0 * (double)device_cu_count();
+            double best = 0.0;
+            uint32_t best_iters = p.tile_iters;
+            for (uint32_t it = p.tile_iters; it >= 1u; it >>= 1) {
+                const double wg_per_record = (double)((groups + it - 1u) / it);
+                // (a few workgroups more than a whole number of rounds do not make a round)
+                const double cost = std::ceil(records * wg_per_record / places - 0.05) * (1.2 + (double)it);
+                if (best == 0.0 || cost < best) { best = cost; best_iters = it; }
+            }
+            p.tile_iters = best_iters;
+        }
     }
     const uint32_t wgs = (row_tiles + tpw * p.tile_iters - 1u) / (tpw * p.tile_iters);
     if (a.W2) {

@@ -525,7 +525,10 @@ BPK_API int bpk_force_kernel(int family);
  * kernel can: a few pairs, Q6_K down projection, at most 8 slots per token),
  * and the batched tile path's gate and up two launches and an activation
  * kernel (default: one launch that stores silu(gate x) * (up x), where hidden
- * spans more than four superblocks);
+ * spans more than four superblocks); "moe_tile_iters": tiles of 16 rows a wave
+ * of the batched tile path walks with a record's activations staged once, where
+ * K is at most four superblocks (1, 2, 4 or 8; 0 = chosen per call from the
+ * expected number of records, so that the workgroups fill whole rounds);
  * "chain_spin_us": bound of a wait between the ops of a chain in microseconds
  * (at most ten seconds);
  * "chain_hold" (test hook, refused unless chain_spin_us is 1..100000): 1 keeps

@@ -125,3 +125,19 @@ def test_gemm_plan_follows_the_options_and_refuses_bad_arguments():
         capi.gemm_plan(11, 2048, 4096, 4096)      # unknown type
     # a part with fewer CUs: o no longer fits one round of half tiles and the answer changes with the count
     assert capi.gemm_plan(Q4_K, 2048, 4096, 4096, 128)[0] in (WHOLE, SHARES, HALF, SMALL)
+
+
+def test_options_take_their_values_and_refuse_others():
+    """bpk_set_option is host state: it can be checked without a device."""
+    for name, good, bad in [("moe_tile_iters", (0, 1, 2, 4, 8), (3, 16, -1)), ("gemm_tile", (0, 128, 129, 192, 256), (64, 130)),
+                            ("gemm_split", (0, 1, 2), (3,))]:
+        try:
+            for v in good:
+                capi.set_option(name, v)
+            for v in bad:
+                with pytest.raises(capi.BpkError):
+                    capi.set_option(name, v)
+        finally:
+            capi.set_option(name, 0)
+    with pytest.raises(capi.BpkError):
+        capi.set_option("no_such_option", 1)
