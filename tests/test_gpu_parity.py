@@ -723,7 +723,9 @@ def test_moe_ffn_qwen3_shapes_decode_and_prefill(gpu, kqo, tgu, tdn):
             assert np.all(np.abs(rowk - ref) <= 1e-3 * rms + 1e-3 * np.abs(ref))
 
 
-@pytest.mark.parametrize("T,E,k,H,I", [(1, 16, 8, 512, 768), (3, 8, 2, 512, 256), (5, 64, 7, 768, 2304), (2, 16, 9, 512, 512)])
+@pytest.mark.parametrize("T,E,k,H,I", [(1, 16, 8, 512, 768), (3, 8, 2, 512, 256), (5, 64, 7, 768, 2304), (2, 16, 9, 512, 512),
+                                       # rows of exactly four superblocks (two rows per step, every lane busy); odd rows per workgroup
+                                       (4, 32, 4, 768, 1024), (7, 64, 8, 1280, 768)])
 def test_moe_ffn_slot_sum_inside_the_last_matvec(gpu, kqo, T, E, k, H, I):
     """A few pairs with a Q6_K down projection: the weighted sum over a token's slots rides in down's launch
     (up to 8 slots; option moe_fold 0 keeps it a launch of its own).  Both against the oracle and each other."""
