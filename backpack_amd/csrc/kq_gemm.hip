@@ -846,9 +846,6 @@ __global__ __launch_bounds__(512) void gemm_bf16_n128_kernel(GemmParams p)
     store_acc<TM, TN>(p, acc, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
-#ifndef KQ_N192_VALU
-#define KQ_N192_VALU 5
-#endif
 // 256 tokens x 192 weight rows per workgroup, whole tiles: N = 6144 at M = 2048 is 256 such tiles, one per CU, where
 // 256 x 256 tiles leave a quarter of the CUs without one.  The kernel above with waves of 64 x 96 and two items
 // per thread: a quarter row of rows 0..127 (as above) and one of rows 128..191 — those 64 rows are taken twice,
@@ -943,7 +940,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_n192_kernel(GemmParams p)
 #pragma unroll
         for (int g = 0; g < TM * TN; ++g) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, KQ_N192_VALU, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);   // (4 .. 8 per group measured level)
         }
         __builtin_amdgcn_sched_barrier(0);
     };
